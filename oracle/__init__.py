@@ -1,0 +1,239 @@
+"""CPU oracle for the quantize / FP4-matmul path -- TEST INFRASTRUCTURE ONLY.
+
+Thin ctypes/numpy wrapper around ``fos_oracle.c`` (a scalar C restatement of the
+reference's PyTorch path; its header lists the reference file:line of every function).
+Only tests, the smoke check and the CPU-baseline leg of the benchmark may import this
+package; the product package never does.
+
+The host-side glue here restates ``PyTorchQuantizeBackend.quantize``
+(reference ``src/fouroversix/quantize/pytorch/backend.py:39-121``): zero-pad to a
+multiple of (128, 64), quantize, put NVFP4 scales into the 128x4-tile layout and leave
+IF4 scales row-major.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SRC = os.path.join(_HERE, "fos_oracle.c")
+_LIB = os.path.join(_HERE, "libfos_oracle.so")
+
+DTYPE_IDS = {"nvfp4": 0, "if4": 1}
+RULE_IDS = {"static_6": 0, "static_4": 1, "mae": 2, "mse": 3, "abs_max": 4}
+ROUND_IDS = {"nearest": 0, "stochastic": 1, "stochastic_unbiased": 2}
+
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle with gcc (strict IEEE: no contraction, no fast-math)."""
+    if force or not os.path.exists(_LIB) or os.path.getmtime(_LIB) < os.path.getmtime(_SRC):
+        cmd = [
+            "gcc", "-O2", "-std=c11", "-fPIC", "-shared", "-fopenmp",
+            "-ffp-contract=off", "-fno-fast-math", "-o", _LIB, _SRC, "-lm",
+        ]
+        subprocess.run(cmd, check=True)
+    return _LIB
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            build()
+        L = ctypes.CDLL(_LIB)
+        c = ctypes
+        vp, i64, u64, f32, i32 = c.c_void_p, c.c_int64, c.c_uint64, c.c_float, c.c_int
+        L.fos_oracle_e4m3_from_f32.argtypes = [f32]
+        L.fos_oracle_e4m3_from_f32.restype = c.c_uint8
+        L.fos_oracle_e4m3_to_f32.argtypes = [c.c_uint8]
+        L.fos_oracle_e4m3_to_f32.restype = f32
+        L.fos_oracle_e2m1_rtn.argtypes = [f32]
+        L.fos_oracle_e2m1_rtn.restype = f32
+        L.fos_oracle_e2m1_decode.argtypes = [c.c_uint8]
+        L.fos_oracle_e2m1_decode.restype = f32
+        L.fos_oracle_sum16.argtypes = [vp]
+        L.fos_oracle_sum16.restype = f32
+        L.fos_oracle_sum256.argtypes = [vp]
+        L.fos_oracle_sum256.restype = f32
+        L.fos_oracle_philox4x32_10.argtypes = [vp, vp, vp]
+        L.fos_oracle_philox4x32_10.restype = None
+        L.fos_oracle_quantize.argtypes = [vp, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, i32]
+        L.fos_oracle_quantize.restype = i32
+        L.fos_oracle_blocked_offset.argtypes = [i64, i64, i64]
+        L.fos_oracle_blocked_offset.restype = i64
+        L.fos_oracle_to_blocked.argtypes = [vp, i64, i64, vp]
+        L.fos_oracle_to_blocked.restype = None
+        L.fos_oracle_from_blocked.argtypes = [vp, i64, i64, vp]
+        L.fos_oracle_from_blocked.restype = None
+        L.fos_oracle_dequantize.argtypes = [vp, vp, f32, i32, c.c_double, i64, i64, vp, i32]
+        L.fos_oracle_dequantize.restype = i32
+        L.fos_oracle_matmul_nt.argtypes = [vp, vp, i64, i64, i64, vp, vp, i32]
+        L.fos_oracle_matmul_nt.restype = None
+        L.fos_oracle_gemm_nvfp4.argtypes = [vp, vp, vp, vp, f32, i64, i64, i64, vp, vp, i32]
+        L.fos_oracle_gemm_nvfp4.restype = None
+        _lib = L
+    return _lib
+
+
+def _ptr(a: np.ndarray) -> int:
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data
+
+
+def default_threads() -> int:
+    return max(1, len(os.sched_getaffinity(0)))
+
+
+def bf16_bits(x) -> np.ndarray:
+    """torch bf16 tensor (CPU) or uint16 ndarray -> contiguous uint16 ndarray."""
+    if isinstance(x, np.ndarray):
+        assert x.dtype == np.uint16
+        return np.ascontiguousarray(x)
+    import torch
+
+    assert x.dtype == torch.bfloat16
+    return x.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def qmax_smax(dtype: str, rule: str) -> tuple[float, float]:
+    """(largest element magnitude, largest block scale) used by the format + rule."""
+    qmax = 4.0 if rule == "static_4" else 6.0
+    smax = 448.0 if (dtype == "if4" or rule in ("static_6", "static_4")) else 256.0
+    return qmax, smax
+
+
+def adjustment(round_style: str) -> float:
+    return 16 / 17 if round_style == "stochastic_unbiased" else 1.0
+
+
+@dataclass
+class OracleQuantized:
+    values: np.ndarray          # u8 [Mp, Np/2]
+    scale_factors: np.ndarray   # u8 flat: 128x4 tiles (nvfp4) or row-major (if4)
+    scale_rows: np.ndarray      # u8 [Mp, Np/16] row-major, always
+    amax: np.float32
+    dtype: str
+    scale_rule: str
+    round_style: str
+    original_shape: tuple[int, int]
+    padded_shape: tuple[int, int]
+    blocked: bool
+
+
+def pad_bits(xb: np.ndarray) -> np.ndarray:
+    m, n = xb.shape
+    mp, np_ = -(-m // 128) * 128, -(-n // 64) * 64
+    if (mp, np_) == (m, n):
+        return xb
+    out = np.zeros((mp, np_), dtype=np.uint16)
+    out[:m, :n] = xb
+    return out
+
+
+def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
+             block_scale_2d=False, seed=0, offset=0, threads=None) -> OracleQuantized:
+    xb = bf16_bits(x)
+    assert xb.ndim == 2
+    orig = tuple(int(v) for v in xb.shape)
+    xp = np.ascontiguousarray(pad_bits(xb))
+    mp, np_ = xp.shape
+    codes = np.zeros((mp, np_ // 2), dtype=np.uint8)
+    sf = np.zeros((mp, np_ // 16), dtype=np.uint8)
+    amax = np.zeros(1, dtype=np.float32)
+    rc = lib().fos_oracle_quantize(
+        _ptr(xp), mp, np_, DTYPE_IDS[dtype], RULE_IDS[scale_rule], ROUND_IDS[round_style],
+        int(block_scale_2d), seed, offset, _ptr(codes), _ptr(sf), _ptr(amax),
+        threads or default_threads(),
+    )
+    if rc != 0:
+        raise ValueError(f"oracle: unsupported combination {dtype}/{scale_rule}")
+    blocked = dtype == "nvfp4"
+    flat = to_blocked(sf) if blocked else sf.reshape(-1).copy()
+    return OracleQuantized(codes, flat, sf, amax[0], dtype, scale_rule, round_style,
+                           orig, (mp, np_), blocked)
+
+
+def to_blocked(sf_rows: np.ndarray) -> np.ndarray:
+    sf_rows = np.ascontiguousarray(sf_rows)
+    out = np.zeros(sf_rows.size, dtype=np.uint8)
+    lib().fos_oracle_to_blocked(_ptr(sf_rows), sf_rows.shape[0], sf_rows.shape[1], _ptr(out))
+    return out
+
+
+def from_blocked(flat: np.ndarray, rows: int, cols: int) -> np.ndarray:
+    flat = np.ascontiguousarray(flat)
+    out = np.zeros((rows, cols), dtype=np.uint8)
+    lib().fos_oracle_from_blocked(_ptr(flat), rows, cols, _ptr(out))
+    return out
+
+
+def dequantize(values: np.ndarray, scale_rows: np.ndarray, amax, *, dtype="nvfp4",
+               scale_rule="mse", round_style="nearest", original_shape=None,
+               threads=None) -> np.ndarray:
+    """f32 [M, N] = the reference's ``dequantize(..., dtype=float32)`` (fp16 intermediate)."""
+    values = np.ascontiguousarray(values)
+    scale_rows = np.ascontiguousarray(scale_rows)
+    mp, half = values.shape
+    qmax, smax = qmax_smax(dtype, scale_rule)
+    div = qmax * smax * adjustment(round_style)
+    out = np.zeros((mp, half * 2), dtype=np.float32)
+    rc = lib().fos_oracle_dequantize(_ptr(values), _ptr(scale_rows), float(amax), DTYPE_IDS[dtype],
+                                     div, mp, half * 2, _ptr(out), threads or default_threads())
+    assert rc == 0
+    if original_shape is not None:
+        out = out[: original_shape[0], : original_shape[1]]
+    return out
+
+
+def matmul_nt(a: np.ndarray, b: np.ndarray, threads=None) -> tuple[np.ndarray, np.ndarray]:
+    """(bf16 bits, f32) of a @ b.T accumulated in double."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    m, k = a.shape
+    n = b.shape[0]
+    o16 = np.zeros((m, n), dtype=np.uint16)
+    o32 = np.zeros((m, n), dtype=np.float32)
+    lib().fos_oracle_matmul_nt(_ptr(a), _ptr(b), m, n, k, _ptr(o16), _ptr(o32), threads or default_threads())
+    return o16, o32
+
+
+def quantized_matmul(qa: OracleQuantized, qb: OracleQuantized, threads=None):
+    """PyTorch-backend form: dequantize both to f32, multiply, round to bf16, crop."""
+    a = dequantize(qa.values, qa.scale_rows, qa.amax, dtype=qa.dtype, scale_rule=qa.scale_rule,
+                   round_style=qa.round_style, threads=threads)
+    b = dequantize(qb.values, qb.scale_rows, qb.amax, dtype=qb.dtype, scale_rule=qb.scale_rule,
+                   round_style=qb.round_style, threads=threads)
+    o16, o32 = matmul_nt(a, b, threads)
+    m, n = qa.original_shape[0], qb.original_shape[0]
+    return o16[:m, :n], o32[:m, :n]
+
+
+def gemm_alpha(qa: OracleQuantized, qb: OracleQuantized) -> np.float32:
+    """alpha of the native GEMM form (reference matmul/cutlass/backend.py:86-98)."""
+    qa_max, sa_max = qmax_smax(qa.dtype, qa.scale_rule)
+    qb_max, sb_max = qmax_smax(qb.dtype, qb.scale_rule)
+    den = qa_max * sa_max * qb_max * sb_max * adjustment(qa.round_style) * adjustment(qb.round_style)
+    return np.float32(np.float32(qa.amax * qb.amax) / np.float32(den))
+
+
+def gemm_nvfp4(values_a, sf_rows_a, values_b, sf_rows_b, alpha, threads=None):
+    """Native-GEMM form: bf16(alpha * sum_k (vA sA)(vB sB)) on padded operands."""
+    m, n, k = values_a.shape[0], values_b.shape[0], values_a.shape[1] * 2
+    o16 = np.zeros((m, n), dtype=np.uint16)
+    o32 = np.zeros((m, n), dtype=np.float32)
+    lib().fos_oracle_gemm_nvfp4(
+        _ptr(np.ascontiguousarray(values_a)), _ptr(np.ascontiguousarray(values_b)),
+        _ptr(np.ascontiguousarray(sf_rows_a)), _ptr(np.ascontiguousarray(sf_rows_b)),
+        float(alpha), m, n, k, _ptr(o16), _ptr(o32), threads or default_threads())
+    return o16, o32
+
+
+def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)

@@ -1,0 +1,184 @@
+"""Write golden vectors for the quantize / dequantize / matmul path by running the
+REFERENCE implementation (its PyTorch CPU backend) on seeded inputs.
+
+Run in the build container only (the reference tree is not available anywhere else):
+
+    python tests/golden/make_golden.py [--time]
+
+The reference package is not pip-installed, so the script puts its ``src`` directory on
+``sys.path`` and answers the one ``importlib.metadata.version("fouroversix")`` lookup it
+makes at import time.  Outputs are data only (inputs + expected bytes) in
+``tests/golden/*.npz``; large cases store SHA-256 digests instead of arrays.
+
+What these vectors pin that nothing else can: the mse/mae block decisions on real data
+(they depend on torch.sum's fp32 summation order), the zero-padding of shapes that are
+not multiples of (128, 64), and the PyTorch matmul backend's bf16 outputs.
+"""
+
+from __future__ import annotations
+
+import argparse
+import hashlib
+import importlib.metadata as md
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+REFERENCE_SRC = "/root/reference/src"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def import_reference():
+    real_version = md.version
+    md.version = lambda name: "1.1.0" if name == "fouroversix" else real_version(name)
+    sys.path.insert(0, REFERENCE_SRC)
+    import fouroversix  # noqa: PLC0415
+
+    md.version = real_version
+    return fouroversix
+
+
+def bits(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.int16).numpy().view(np.uint16).copy()
+
+
+def u8(t: torch.Tensor) -> np.ndarray:
+    return t.contiguous().view(torch.uint8).numpy().copy()
+
+
+def sha(a: np.ndarray) -> str:
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def make_input(kind: str, shape: tuple[int, int], seed: int) -> torch.Tensor:
+    g = torch.Generator("cpu").manual_seed(seed)
+    if kind == "randn":
+        x = torch.randn(*shape, generator=g)
+    elif kind == "weight":
+        x = 0.02 * torch.randn(*shape, generator=g)
+    elif kind == "rand01":
+        x = torch.randint(0, 2, shape, generator=g).float()
+    elif kind == "outlier":
+        # rows N(0,1); 1 % of the channels replaced by 50 * Student-t(nu=3)
+        x = torch.randn(*shape, generator=g)
+        n_out = max(1, shape[1] // 100)
+        idx = torch.randperm(shape[1], generator=g)[:n_out]
+        z = torch.randn(4, shape[0], n_out, generator=g)
+        t3 = z[0] / torch.sqrt((z[1] ** 2 + z[2] ** 2 + z[3] ** 2) / 3)
+        x[:, idx] = 50 * t3
+    elif kind == "tiny_blocks":
+        # blocks whose maximum is far below the tensor maximum: sub-normal E4M3 scales
+        x = torch.randn(*shape, generator=g)
+        per_block = 10.0 ** (-torch.rand(shape[1] // 16, generator=g) * 6)
+        per_block[0] = 1.0
+        x = x * per_block.repeat_interleave(16)
+    else:
+        raise ValueError(kind)
+    return x.bfloat16()
+
+
+QUANT_INPUTS = [
+    ("randn_256x128", "randn", (256, 128), 11),
+    ("outlier_128x256", "outlier", (128, 256), 12),
+    ("weight_128x128", "weight", (128, 128), 13),
+    ("rand01_128x64", "rand01", (128, 64), 14),
+    ("ragged_100x80", "randn", (100, 80), 15),
+    ("ragged_16x64", "randn", (16, 64), 16),
+    ("tiny_blocks_128x128", "tiny_blocks", (128, 128), 17),
+]
+
+QUANT_CONFIGS = [
+    ("nvfp4", rule, two_d)
+    for rule in ("mse", "mae", "abs_max", "static_6", "static_4")
+    for two_d in (False, True)
+] + [("if4", rule, two_d) for rule in ("mse", "mae", "abs_max") for two_d in (False, True)]
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
+    args = ap.parse_args()
+
+    fos = import_reference()
+    from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
+
+    torch.set_num_threads(os.cpu_count() or 1)
+
+    # ---- quantize + dequantize ------------------------------------------------------
+    for name, kind, shape, seed in QUANT_INPUTS:
+        x = make_input(kind, shape, seed)
+        out: dict[str, np.ndarray] = {"x": bits(x), "shape": np.array(shape)}
+        for dtype, rule, two_d in QUANT_CONFIGS:
+            cfg = QuantizationConfig(backend="pytorch", dtype=dtype, scale_rule=rule, block_scale_2d=two_d)
+            q = quantize(x.clone(), cfg)
+            key = f"{dtype}.{rule}.{'2d' if two_d else '1d'}"
+            out[key + ".values"] = u8(q.values)
+            out[key + ".sf"] = u8(q.scale_factors)
+            out[key + ".amax"] = np.array([float(q.amax)], dtype=np.float32)
+            out[key + ".padded"] = np.array(q.padded_shape)
+            out[key + ".blocked"] = np.array([int(q.scale_factors_are_in_blackwell_layout)])
+            if name in ("randn_256x128", "ragged_100x80", "tiny_blocks_128x128") and not two_d:
+                out[key + ".deq_bf16"] = bits(dequantize(q))
+                out[key + ".deq_f32_sha"] = np.array(sha(dequantize(q, torch.float32).numpy()))
+        np.savez_compressed(os.path.join(HERE, f"quantize_{name}.npz"), **out)
+        print("wrote", name, len(out))
+
+    # ---- the CPU-runnable headline case: 1024x1024 randn seed 0, static_6 ------------
+    g = torch.Generator("cpu").manual_seed(0)
+    x = torch.randn(1024, 1024, generator=g).bfloat16()
+    big = {"x_sha": np.array(sha(bits(x)))}
+    for rule in ("static_6", "mse"):
+        q = quantize(x, QuantizationConfig(backend="pytorch", scale_rule=rule))
+        big[f"{rule}.values_sha"] = np.array(sha(u8(q.values)))
+        big[f"{rule}.sf_sha"] = np.array(sha(u8(q.scale_factors)))
+        big[f"{rule}.amax"] = np.array([float(q.amax)], dtype=np.float32)
+        big[f"{rule}.values_head"] = u8(q.values)[:4].copy()
+        big[f"{rule}.sf_head"] = u8(q.scale_factors)[:512].copy()
+    np.savez_compressed(os.path.join(HERE, "quantize_config1_1024x1024.npz"), **big)
+    print("wrote config1")
+
+    # ---- matmul (PyTorch backend: dequantize -> fp32 matmul -> bf16) -----------------
+    mm: dict[str, np.ndarray] = {}
+    for tag, (m, n, k), rule, seed in [
+        ("mse_256x256x256", (256, 256, 256), "mse", 21),
+        ("static6_128x256x512", (128, 256, 512), "static_6", 22),
+        ("static4_128x128x128", (128, 128, 128), "static_4", 23),
+        ("ragged_100x72x80", (100, 72, 80), "mse", 24),
+    ]:
+        g = torch.Generator("cpu").manual_seed(seed)
+        a = torch.randn(m, k, generator=g).bfloat16()
+        b = torch.randn(n, k, generator=g).bfloat16()
+        cfg = QuantizationConfig(backend="pytorch", scale_rule=rule)
+        qa, qb = quantize(a, cfg), quantize(b, cfg)
+        o = quantized_matmul(qa, qb, backend="pytorch")
+        mm[tag + ".a"] = bits(a)
+        mm[tag + ".b"] = bits(b)
+        mm[tag + ".out"] = bits(o)
+        mm[tag + ".rule"] = np.array(rule)
+    np.savez_compressed(os.path.join(HERE, "matmul.npz"), **mm)
+    print("wrote matmul")
+
+    if args.time:
+        from torch.utils.benchmark import Timer  # noqa: PLC0415
+
+        g = torch.Generator("cpu").manual_seed(0)
+        x1 = torch.randn(1024, 1024, generator=g).bfloat16()
+        cfg1 = QuantizationConfig(backend="pytorch", scale_rule="static_6")
+        t1 = Timer("quantize(x, cfg)", globals={"quantize": quantize, "x": x1, "cfg": cfg1}).timeit(5).mean
+        g = torch.Generator("cpu").manual_seed(1)
+        x2 = torch.randn(8192, 4096, generator=g).bfloat16()
+        cfg2 = QuantizationConfig(backend="pytorch", scale_rule="mse")
+        t0 = time.time()
+        quantize(x2, cfg2)
+        t2 = time.time() - t0
+        print(f"reference CPU path, {torch.get_num_threads()} threads: "
+              f"1024x1024 static_6 {t1 * 1e3:.1f} ms ({1024 * 1024 * 2.5625 / t1 / 1e9:.3f} GB/s); "
+              f"8192x4096 mse {t2:.2f} s ({8192 * 4096 * 2.5625 / t2 / 1e9:.3f} GB/s)")
+    del fos
+
+
+if __name__ == "__main__":
+    main()
