@@ -1,0 +1,242 @@
+"""Benchmark of the quantize + FP4-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one pass of the hot path over one synthetic batch already resident in HBM:
+``quantize`` of an 8192 x 8192 bf16 tensor to NVFP4 with 4/6-MSE selection, round to
+nearest, 1x16 blocks (tensor-max pass + quantize pass).  Inputs rotate over four buffers
+(512 MiB) so that a step never finds its input in the 256 MB Infinity Cache left over from
+the previous step.  ``value`` is algorithmic GB/s (2.5625 B per element: bf16 in, packed
+nibbles + E4M3 scales out) of the whole step.  The same line carries the FP4 GEMM at
+8192^3 (TFLOP/s, ``gemm``), the roofline of the dominant kernel of each, and the CPU
+oracle timed on the host cores on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+BYTES_PER_ELEM = 2.0 + 0.5 + 1.0 / 16.0
+
+
+def make_activation(rows, cols, seed, outliers=False):
+    import torch
+
+    g = torch.Generator("cpu").manual_seed(seed)
+    x = torch.randn(rows, cols, generator=g)
+    if outliers:
+        n_out = max(1, cols // 100)
+        idx = torch.randperm(cols, generator=g)[:n_out]
+        z = torch.randn(4, rows, n_out, generator=g)
+        x[:, idx] = 50 * z[0] / torch.sqrt((z[1] ** 2 + z[2] ** 2 + z[3] ** 2) / 3)
+    return x.bfloat16()
+
+
+def event_ms(fn, steps):
+    """Average milliseconds of ``fn`` per call, from HIP events on the current stream."""
+    import torch
+
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--rows", type=int, default=8192)
+    ap.add_argument("--cols", type=int, default=8192)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
+    ap.add_argument("--no-gemm", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import fouroversix_amd as fos
+    from fouroversix_amd import _native as nat
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    L = nat.lib()
+    rows, cols, K, W = args.rows, args.cols, args.steps, args.warmup
+    elems = rows * cols
+    algo_bytes = elems * BYTES_PER_ELEM
+
+    # ---- quantize: whole step through the public API -------------------------------
+    n_buf = 4
+    xs = [make_activation(rows, cols, 100 + i).to(dev) for i in range(n_buf)]
+    cfg = fos.QuantizationConfig(scale_rule="mse")
+    for i in range(W):
+        fos.quantize(xs[i % n_buf], cfg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        q = fos.quantize(xs[i % n_buf], cfg)
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) * 1e3 / K
+    value = algo_bytes / (step_ms * 1e-3) / 1e9
+
+    # ---- quantize: per-kernel durations from HIP events, straight through the C ABI --
+    rows_p, cols_p = L.fos_padded_rows(rows), L.fos_padded_cols(cols)
+    codes = torch.empty(rows_p, cols_p // 2, dtype=torch.uint8, device=dev)
+    sf = torch.empty(rows_p * cols_p // 16, dtype=torch.uint8, device=dev)
+    amax = torch.zeros(1, dtype=torch.float32, device=dev)
+    ws_bytes = L.fos_quantize_workspace_bytes(rows, cols)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = nat.current_stream(dev)
+    counter = [0]
+
+    def run_amax():
+        x = xs[counter[0] % n_buf]
+        nat.check(L.fos_amax(x.data_ptr(), 0, rows, cols, cols, amax.data_ptr(), ws.data_ptr(), ws_bytes, stream), "amax")
+
+    def run_quant_only():
+        x = xs[counter[0] % n_buf]
+        counter[0] += 1
+        nat.check(L.fos_quantize(x.data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(),
+                                 sf.data_ptr(), amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")
+
+    def run_both():
+        run_amax()
+        run_quant_only()
+
+    for _ in range(W):
+        run_both()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3 * K)]
+    for i in range(K):
+        ev[3 * i].record()
+        run_amax()
+        ev[3 * i + 1].record()
+        run_quant_only()
+        ev[3 * i + 2].record()
+    torch.cuda.synchronize()
+    amax_ms = sum(ev[3 * i].elapsed_time(ev[3 * i + 1]) for i in range(K)) / K
+    quant_ms = sum(ev[3 * i + 1].elapsed_time(ev[3 * i + 2]) for i in range(K)) / K
+    counter[0] = 0
+    same_buffer_ms = event_ms(lambda: (run_amax(), nat.check(L.fos_quantize(
+        xs[0].data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(), sf.data_ptr(),
+        amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")), K)
+    q_achieved = algo_bytes / (quant_ms * 1e-3) / 1e9
+    roofline = {
+        "kernel": "quantize_kernel (pass 2: scale, 4/6 select, pack)",
+        "bound": "hbm",
+        "achieved": round(q_achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(q_achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "kernel_ms": round(quant_ms, 5),
+        "amax_pass_ms": round(amax_ms, 5),
+        "amax_pass_GBs": round(elems * 2 / (amax_ms * 1e-3) / 1e9, 1),
+        "whole_step_frac": round(value / HBM_PEAK_GBS, 4),
+        "same_buffer_step_ms": round(same_buffer_ms, 5),
+    }
+
+    # ---- activation-style input with outlier channels (8192 x 4096) -----------------
+    xo = [make_activation(8192, 4096, 1 + i, outliers=True).to(dev) for i in range(6)]
+    for i in range(W):
+        fos.quantize(xo[i % 6], cfg)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        fos.quantize(xo[i % 6], cfg)
+    torch.cuda.synchronize()
+    act_ms = (time.perf_counter() - t0) * 1e3 / K
+    del xo
+
+    # ---- FP4 GEMM 8192^3 on pre-quantized operands ------------------------------------
+    gemm = None
+    if not args.no_gemm:
+        m = n = k = 8192
+        qa = fos.quantize(make_activation(m, k, 5).to(dev), cfg)
+        qb = fos.quantize(make_activation(n, k, 6).to(dev), cfg)
+        for _ in range(max(2, W // 2)):
+            fos.quantized_matmul(qa, qb)
+        gk = max(5, K // 2)
+        gemm_ms = event_ms(lambda: fos.quantized_matmul(qa, qb), gk)
+        tflops = 2.0 * m * n * k / (gemm_ms * 1e-3) / 1e12
+        gemm = {
+            "workload": "NVFP4 x NVFP4 -> bf16, M=N=K=8192, FP32 accumulate, alpha on device",
+            "ms": round(gemm_ms, 4),
+            "value": round(tflops, 1),
+            "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
+        }
+
+    # ---- CPU baseline: the C oracle on the host cores, bounded sample -----------------
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+
+        oracle.build()
+        threads = min(oracle.default_threads(), 16)
+        sample_rows = 1024
+        sample = xs[0][:sample_rows].cpu()
+        oracle.quantize(sample[:128], scale_rule="mse", threads=threads)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 3 or (time.perf_counter() - t0 < 10 and reps < 50):
+            oracle.quantize(sample, scale_rule="mse", threads=threads)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
+        cpu = {
+            "value": round(sample_rows * cols * BYTES_PER_ELEM / cpu_s / 1e9, 4),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{sample_rows} x {cols} rows of the same tensor, {reps} repetitions, C oracle with OpenMP",
+        }
+
+    line = {
+        "metric": "quantize GB/s (% HBM peak) + FP4 GEMM TFLOP/s (% roofline), 1 MI355X",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(step_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"quantize {rows}x{cols} bf16 N(0,1) -> NVFP4, 4/6-MSE, round-to-nearest, 1x16 blocks, "
+                        "E4M3 scales in the 128x4-tile layout (tensor-max pass + quantize pass), "
+                        "4 rotating input buffers",
+            "algorithmic_bytes_per_element": BYTES_PER_ELEM,
+            "activation_8192x4096_outliers_ms": round(act_ms, 5),
+            "activation_8192x4096_outliers_GBs": round(8192 * 4096 * BYTES_PER_ELEM / (act_ms * 1e-3) / 1e9, 1),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "gemm": gemm,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

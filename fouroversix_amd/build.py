@@ -1,0 +1,75 @@
+"""Build the gfx950 shared library (``libfouroversix_hip.so``) with hipcc.
+
+    python -m fouroversix_amd.build [--force]
+
+hipcc cross-compiles for gfx950 without a GPU.  The flags matter for bit-exactness:
+no fp contraction (fused multiply-adds only where the source spells them), correctly
+rounded fp32 division, fp32 denormals kept, and no packed-fp32 instructions.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+LIB_PATH = os.path.join(HERE, "libfouroversix_hip.so")
+OBJ_DIR = os.path.join(CSRC, "build")
+
+SOURCES = ["fos_common.hip", "fos_quantize.hip", "fos_gemm.hip", "fos_dequantize.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-fno-gpu-flush-denormals-to-zero",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{INCLUDE}",
+    f"-I{CSRC}",
+]
+
+
+def _deps(src: str) -> list[str]:
+    return [src] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")] + [
+        os.path.join(INCLUDE, f) for f in os.listdir(INCLUDE)
+    ]
+
+
+def _compile(name: str, force: bool) -> str:
+    src = os.path.join(CSRC, name)
+    obj = os.path.join(OBJ_DIR, name.replace(".hip", ".o"))
+    if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in _deps(src)):
+        return obj
+    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "packed-fp32-ops"
+    err = "\n".join(line for line in res.stderr.splitlines() if noise not in line)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {name}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(force: bool = False) -> str:
+    """Compile every HIP source and link the shared library; returns its path."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(lambda n: _compile(n, force), SOURCES))
+    if force or not os.path.exists(LIB_PATH) or any(os.path.getmtime(o) > os.path.getmtime(LIB_PATH) for o in objs):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+        subprocess.run(cmd, check=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

@@ -1,0 +1,87 @@
+"""``quantized_matmul``: the reference's frontend
+(``src/fouroversix/matmul/frontend.py:18-132``) over the gfx950 FP4 GEMM.
+
+``input @ other.T`` with both operands block-scaled 4-bit.  Operands given in high
+precision are quantized first with ``input_config`` / ``other_config``.  The GEMM is the
+native-op form of the reference (``src/fouroversix/matmul/cutlass/backend.py:56-155``):
+``alpha = amaxA * amaxB / (qA * sA * qB * sB * adjA * adjB)`` stays on the device and the
+padded result is cropped to ``(M, N)``.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from fouroversix_amd.quantize import QuantizationConfig, QuantizedTensor, quantize
+from fouroversix_amd.quantize import ops
+from fouroversix_amd.quantize.frontend import dequantize_divisor
+from fouroversix_amd.utils import DataType, MatmulBackend
+
+
+def is_supported(input: QuantizedTensor, other: QuantizedTensor, *, out_dtype: DataType) -> bool:
+    """Mirror of ``MatmulBackendBase.is_supported`` + the native backend's conditions."""
+    if input.original_shape[1] != other.original_shape[1]:
+        msg = (
+            "The first input must be in row-major layout, the second input must be"
+            "in column-major layout, and both inputs must have the same inner "
+            "dimension"
+        )
+        raise ValueError(msg)
+    return (
+        input.dtype == other.dtype
+        and input.dtype == DataType.nvfp4
+        and input.device.type == "cuda"
+        and out_dtype in (DataType.bfloat16, DataType.float16)
+        and input.scale_factors_are_in_blackwell_layout
+        and other.scale_factors_are_in_blackwell_layout
+    )
+
+
+def gemm_alpha(input: QuantizedTensor, other: QuantizedTensor) -> torch.Tensor:
+    den = dequantize_divisor(input) * dequantize_divisor(other)
+    return ((input.amax * other.amax) / den).to(torch.float32).reshape(1)
+
+
+def quantized_matmul(
+    input: torch.Tensor | QuantizedTensor,
+    other: torch.Tensor | QuantizedTensor,
+    *,
+    backend: MatmulBackend | None = None,
+    input_config: QuantizationConfig | None = None,
+    other_config: QuantizationConfig | None = None,
+    out_dtype: DataType = DataType.bfloat16,
+    **kwargs: dict[str, Any],
+) -> torch.Tensor:
+    """FP4 matrix product ``input @ other.T`` -> ``[M, N]`` tensor of ``out_dtype``."""
+    del kwargs
+    if input_config is None:
+        input_config = QuantizationConfig()
+    if isinstance(input, torch.Tensor):
+        input = quantize(input, input_config)
+    if other_config is None:
+        other_config = QuantizationConfig()
+    if isinstance(other, torch.Tensor):
+        other = quantize(other, other_config)
+    if isinstance(out_dtype, str):
+        out_dtype = DataType(out_dtype)
+
+    if not is_supported(input, other, out_dtype=out_dtype):
+        if backend is None:
+            msg = "No backend found that supports the given parameters"
+        else:
+            msg = f"Backend {backend} does not support the given parameters"
+        raise ValueError(msg)
+
+    alpha = gemm_alpha(input, other)
+    gemm = (
+        ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
+        if out_dtype == DataType.bfloat16
+        else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
+    )
+    out = gemm(input.values, other.values, input.scale_factors, other.scale_factors, alpha)
+    out_shape = (input.original_shape[0], other.original_shape[0])
+    if tuple(out.shape) != out_shape:
+        out = out[: out_shape[0], : out_shape[1]]
+    return out

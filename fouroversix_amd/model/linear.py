@@ -1,0 +1,145 @@
+"""``FourOverSixLinear``: ``nn.Linear`` whose forward quantizes the activations on the fly
+and multiplies them with a (pre-)quantized weight on the FP4 GEMM
+(reference ``src/fouroversix/model/modules/linear.py:43-94, 291-453``; forward pass only,
+the reference's quantized backward is training machinery outside this library).
+
+The quantized weight lives in four buffers with the reference's names and shapes --
+``quantized_weight_values`` u8 [out, in/2], ``quantized_weight_scale_factors`` E4M3 flat,
+``quantized_weight_amax`` f32[1], ``quantized_weight_metadata`` int32[6] = (rows, cols,
+padded rows, padded cols, 1, tiled-layout flag) -- so checkpoints interchange.
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+from fouroversix_amd.matmul import quantized_matmul
+from fouroversix_amd.quantize import QuantizedTensor, quantize
+
+from .config import ModuleQuantizationConfig
+from .quantize import QuantizedModule
+
+
+def fp4_linear(
+    config: ModuleQuantizationConfig,
+    input: torch.Tensor,
+    weight: QuantizedTensor | torch.Tensor,
+    bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``input @ weight.T + bias`` with both operands in the configured 4-bit formats."""
+    if config.disable_fprop_quantization:
+        out = torch.matmul(input, weight.T)
+    else:
+        if isinstance(weight, torch.Tensor):
+            weight = quantize(weight.data if isinstance(weight, nn.Parameter) else weight, config.get_weight_config())
+        flat = input.reshape(-1, input.shape[-1])
+        if config.pseudo_quantize:
+            out = torch.matmul(quantize(flat, config.get_activation_config()), weight.T)
+            out = out.reshape(*input.shape[:-1], weight.shape[0])
+        else:
+            out = quantized_matmul(
+                flat,
+                weight,
+                backend=config.matmul_backend,
+                input_config=config.get_activation_config(),
+                out_dtype=config.output_dtype,
+            ).reshape(*input.shape[:-1], weight.original_shape[0])
+    if bias is not None:
+        out = out + bias
+    return out
+
+
+@QuantizedModule.register(nn.Linear)
+class FourOverSixLinear(nn.Linear):
+    """Drop-in ``nn.Linear`` replacement with 4-bit weights and activations."""
+
+    def __init__(self, module: nn.Linear, config: ModuleQuantizationConfig) -> None:
+        super().__init__(
+            module.in_features,
+            module.out_features,
+            module.bias is not None,
+            module.weight.device,
+            module.weight.dtype,
+        )
+        self.weight = module.weight
+        self.bias = module.bias
+        self.config = config
+
+        if not config.keep_master_weights:
+            wdt = config.weight_dtype
+            pack = wdt.quantized_value_type.packing_factor
+            self.register_buffer(
+                "quantized_weight_values",
+                torch.zeros(self.out_features, self.in_features // pack, dtype=torch.uint8),
+            )
+            self.register_buffer(
+                "quantized_weight_scale_factors",
+                torch.zeros(self.out_features * self.in_features // wdt.block_size, dtype=wdt.scale_type.torch_dtype),
+            )
+            self.register_buffer("quantized_weight_amax", torch.zeros(1, dtype=torch.float32))
+            self.register_buffer("quantized_weight_metadata", torch.zeros(6, dtype=torch.int32))
+
+    @property
+    def parameters_to_quantize(self) -> tuple[str, ...]:
+        return ("weight",)
+
+    def get_element_size(self, parameter_name: str) -> float:
+        """Bytes per element: 0.5 for the packed values, (8 + 1) / 16 for a quantized weight."""
+        sizes = {"quantized_weight_values": 0.5, "weight": 9 / 16}
+        if parameter_name in sizes:
+            return sizes[parameter_name]
+        return getattr(self, parameter_name).element_size()
+
+    def get_quantized_parameters(self, parameter_name: str, parameter: torch.Tensor) -> dict[str, Any]:
+        """Quantize ``parameter`` (the weight) and return the four buffers as a dict."""
+        if parameter_name != "weight":
+            msg = f"Unsupported high-precision parameter: {parameter_name}"
+            raise ValueError(msg)
+        q = quantize(parameter, self.config.get_weight_config())
+        return {
+            "quantized_weight_values": q.values,
+            "quantized_weight_scale_factors": q.scale_factors,
+            "quantized_weight_amax": q.amax,
+            "quantized_weight_metadata": torch.tensor(
+                [*q.original_shape, *q.padded_shape, 1, int(q.scale_factors_are_in_blackwell_layout)],
+            ),
+        }
+
+    def quantize_weight_(self) -> "FourOverSixLinear":
+        """Fill the quantized buffers from ``self.weight`` and drop the high-precision
+        weight (what the reference leaves to its checkpoint-loading integrations)."""
+        if self.config.keep_master_weights:
+            return self
+        params = self.get_quantized_parameters("weight", self.weight.data)
+        dev = self.weight.device
+        for name, value in params.items():
+            setattr(self, name, value.reshape(getattr(self, name).shape if name == "quantized_weight_amax" else value.shape).to(dev))
+        self.quantized_weight_metadata = self.quantized_weight_metadata.to(torch.int32)
+        self.weight = None
+        if hasattr(self, "_quantized_weight"):
+            del self._quantized_weight
+        return self
+
+    def quantized_weight(self) -> QuantizedTensor | nn.Parameter:
+        if self.config.keep_master_weights:
+            return self.weight
+        if not hasattr(self, "_quantized_weight"):
+            meta = self.quantized_weight_metadata.tolist()
+            self._quantized_weight = QuantizedTensor(
+                self.quantized_weight_values,
+                self.quantized_weight_scale_factors,
+                self.quantized_weight_amax,
+                self.config.weight_dtype,
+                tuple(meta[:2]),
+                self.config.weight_scale_rule,
+                self.config.weight_round_style,
+                tuple(meta[2:4]),
+                scale_factors_are_in_blackwell_layout=meta[5] == 1,
+            )
+        return self._quantized_weight
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        return fp4_linear(self.config, input, self.quantized_weight(), self.bias)

@@ -1,0 +1,14 @@
+from .config import QuantizationConfig
+from .frontend import can_quantize, dequantize, quantize
+from .layout import from_blocked, to_blocked
+from .quantized_tensor import QuantizedTensor
+
+__all__ = [
+    "QuantizationConfig",
+    "QuantizedTensor",
+    "can_quantize",
+    "dequantize",
+    "from_blocked",
+    "quantize",
+    "to_blocked",
+]

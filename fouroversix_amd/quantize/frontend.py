@@ -1,0 +1,152 @@
+"""``quantize`` / ``dequantize``: the reference's frontends
+(``src/fouroversix/quantize/frontend.py:19-157``) over the gfx950 kernels.
+
+There is one implementation, so the reference's backend auto-selection collapses to a
+support check with the same outcome for the caller: a ``ValueError`` when nothing can
+quantize the given tensor/config.  The result follows the reference's PyTorch backend
+(``src/fouroversix/quantize/pytorch/backend.py:39-121``): values padded to (128, 64)
+multiples, NVFP4 scales in the 128x4-tile layout, IF4 scales row-major, 0-dim fp32 amax.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from fouroversix_amd import _native as nat
+from fouroversix_amd.utils import NATIVE_FORMAT_IDS, DataType, QuantizeBackend, ScaleType
+
+from . import ops
+from .config import QuantizationConfig
+from .quantized_tensor import QuantizedTensor
+
+_LINEAR_SCALE_FORMATS = {DataType.if4, DataType.nvint4}
+
+
+def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | None:
+    """Why this (tensor, config) cannot be quantized, or None if it can."""
+    if x.ndim != 2:
+        return "input must be 2-D"
+    if config.scale_rule not in config.dtype.supported_scale_rules:
+        return f"scale rule {config.scale_rule.value} is not defined for {config.dtype.value}"
+    if config.dtype.value not in NATIVE_FORMAT_IDS:
+        return f"format {config.dtype.value} has no gfx950 kernel"
+    if config.rht:
+        return "the random Hadamard transform is not implemented"
+    if config.transpose:
+        return "transposed quantization is not implemented"
+    if x.device.type != "cuda":
+        return f"input must live on the GPU, got {x.device}"
+    if x.dtype != torch.bfloat16:
+        return f"input must be bfloat16, got {x.dtype}"
+    return None
+
+
+def can_quantize(x: torch.Tensor, config: QuantizationConfig) -> bool:
+    return unsupported_reason(x, config) is None
+
+
+def quantize(
+    x: torch.Tensor,
+    config: QuantizationConfig | None = None,
+) -> QuantizedTensor | torch.Tensor:
+    """Quantize a 2-D bf16 GPU tensor to a block-scaled 4-bit format.
+
+    With no config: NVFP4, 1x16 blocks, round-to-nearest, 4/6 selection by block MSE.
+    ``config.kwargs`` may carry ``seed`` / ``offset`` (ints) keying the dither of the
+    stochastic rounding styles (default: drawn from torch's global generator) and
+    ``amax`` (a tensor) to skip the tensor-wide maximum pass.
+    """
+    if config is None:
+        config = QuantizationConfig()
+
+    reason = unsupported_reason(x, config)
+    if reason is not None:
+        if config.backend is None:
+            msg = f"No backend found that supports the given parameters ({reason})"
+        else:
+            msg = f"Backend {config.backend} does not support the given parameters ({reason})"
+        raise ValueError(msg)
+
+    if config.pseudo_quantize:
+        plain = QuantizationConfig(**{**config.__dict__, "pseudo_quantize": False})
+        return dequantize(quantize(x, plain), dtype=x.dtype)
+
+    if config.round_style.is_stochastic and "seed" not in config.kwargs:
+        seed = int(torch.randint(0, 2**62, (1,)).item())
+    else:
+        seed = int(config.kwargs.get("seed", config.kwargs.get("rbits", 0)))
+        seed = max(seed, 0)
+    offset = int(config.kwargs.get("offset", 0))
+    linear = config.dtype in _LINEAR_SCALE_FORMATS
+
+    x_rows = x if x.stride(-1) == 1 else x.contiguous()
+    values, scale_factors, amax = ops.quantize_ex(
+        x_rows,
+        NATIVE_FORMAT_IDS[config.dtype.value],
+        config.scale_rule.cuda_id,
+        config.round_style.native_id,
+        config.block_scale_2d,
+        seed,
+        offset,
+        nat.SF_LINEAR if linear else nat.SF_TILED,
+        config.kwargs.get("amax"),
+    )
+    return QuantizedTensor(
+        values,
+        scale_factors,
+        amax.reshape(()),
+        config.dtype,
+        tuple(x.shape),
+        config.scale_rule,
+        config.round_style,
+        scale_factors_are_in_blackwell_layout=not linear,
+    )
+
+
+def dequantize_divisor(tensor: QuantizedTensor) -> float:
+    """qmax * smax * adjustment of the tensor's scale rule and rounding style."""
+    return (
+        tensor.dtype.quantized_value_type.get_maximum_value(tensor.scale_rule)
+        * tensor.dtype.scale_type.get_maximum_value(tensor.scale_rule)
+        * tensor.round_style.adjustment_factor
+    )
+
+
+def dequantize(
+    tensor: QuantizedTensor,
+    dtype: torch.dtype = torch.bfloat16,
+    *,
+    backend: QuantizeBackend | None = None,
+    intermediate_dtype: torch.dtype = torch.float16,
+) -> torch.Tensor:
+    """High-precision tensor of ``tensor.original_shape`` from a quantized tensor.
+
+    Value and block scale are multiplied in fp16 (exact for NVFP4, so
+    ``intermediate_dtype=float32`` gives the same result there), widened to fp32,
+    scaled by ``amax / (qmax * smax * adjustment)`` and cast to ``dtype``.
+    """
+    del backend
+    if tensor.dtype.value not in NATIVE_FORMAT_IDS or tensor.dtype.scale_type == ScaleType.mx:
+        msg = f"No backend can dequantize {tensor.dtype.value}"
+        raise ValueError(msg)
+    if tensor.amax is None:
+        msg = "dequantize needs the tensor-wide amax"
+        raise ValueError(msg)
+    if intermediate_dtype != torch.float16 and tensor.dtype != DataType.nvfp4:
+        msg = "only intermediate_dtype=float16 is implemented for this format"
+        raise ValueError(msg)
+    if dtype not in nat.TORCH_TO_T:
+        msg = f"unsupported output dtype {dtype}"
+        raise ValueError(msg)
+    rows, cols = tensor.original_shape
+    return ops.dequantize(
+        tensor.values,
+        tensor.scale_factors,
+        tensor.amax,
+        NATIVE_FORMAT_IDS[tensor.dtype.value],
+        nat.SF_TILED if tensor.scale_factors_are_in_blackwell_layout else nat.SF_LINEAR,
+        float(dequantize_divisor(tensor)),
+        rows,
+        cols,
+        dtype,
+    )

@@ -1,0 +1,211 @@
+"""``torch.ops.fouroversix.*`` operators backed by the gfx950 library.
+
+The operator names and schemas are the reference's
+(``src/fouroversix/csrc/bindings.cpp:26-35``), with the fake (meta) shapes of
+``src/fouroversix/quantize/cuda/ops.py:28-47`` and
+``src/fouroversix/matmul/cutlass/ops.py:82-92``, so code that calls the ops directly, or
+traces them, keeps working.  ``quantize_ex`` / ``dequantize`` are additions carrying the
+options the reference's native op does not have (format, dither key, output layout).
+Each implementation allocates the outputs and makes one call through the C ABI on the
+current stream.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from fouroversix_amd import _native as nat
+
+_LIB = torch.library.Library("fouroversix", "DEF")
+_LIB.define(
+    "quantize(Tensor x, bool is_nvfp4, bool is_rtn, bool is_rht, bool is_2d, bool is_transpose, "
+    "int selection_rule, int rbits) -> (Tensor, Tensor, Tensor)"
+)
+_LIB.define(
+    "quantize_ex(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, int seed, int offset, "
+    "int sf_layout, Tensor? amax) -> (Tensor, Tensor, Tensor)"
+)
+_LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
+_LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
+_LIB.define(
+    "dequantize(Tensor values, Tensor scale_factors, Tensor amax, int dtype, int sf_layout, float divisor, "
+    "int rows, int cols, ScalarType out_dtype) -> Tensor"
+)
+
+
+def _padded(rows: int, cols: int) -> tuple[int, int]:
+    return -(-rows // 128) * 128, -(-cols // 64) * 64
+
+
+def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
+    if x.dim() != 2:
+        raise RuntimeError("quantize: x must be 2-D")
+    if x.dtype != torch.bfloat16:
+        raise RuntimeError("quantize: x must be bfloat16")
+    if x.stride(-1) != 1:
+        raise RuntimeError("quantize: x must be contiguous on the last dim")
+    nat.require_gpu_tensor(x, "x")
+    rows, cols = x.shape
+    rows_p, cols_p = _padded(rows, cols)
+    dev = x.device
+    values = torch.empty(rows_p, cols_p // 2, dtype=torch.uint8, device=dev)
+    sf = torch.empty(rows_p * cols_p // 16, dtype=torch.float8_e4m3fn, device=dev)
+    if rows == 0 or cols == 0:
+        values.zero_()
+        sf.view(torch.uint8).zero_()
+        return values, sf, torch.zeros(1, dtype=torch.float32, device=dev)
+    L = nat.lib()
+    ws_bytes = L.fos_quantize_workspace_bytes(rows, cols)
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    amax_is_input = amax is not None
+    amax_buf = (
+        amax.reshape(1).to(device=dev, dtype=torch.float32).contiguous()
+        if amax_is_input
+        else torch.empty(1, dtype=torch.float32, device=dev)
+    )
+    with torch.cuda.device(dev):
+        rc = L.fos_quantize(
+            x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), dtype, selection_rule, round_style, int(is_2d),
+            seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, sf_layout,
+            values.data_ptr(), sf.data_ptr(), amax_buf.data_ptr(), int(amax_is_input),
+            workspace.data_ptr(), ws_bytes, nat.current_stream(dev),
+        )
+    nat.check(rc, "fouroversix::quantize")
+    return values, sf, amax_buf
+
+
+def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
+    if not is_nvfp4:
+        raise RuntimeError("quantize: only the NVFP4 format is implemented by this op (use quantize_ex for IF4)")
+    if is_rht or is_transpose:
+        raise RuntimeError("quantize: rht / transpose are not implemented")
+    if not 0 <= selection_rule <= 4:
+        raise RuntimeError(f"Invalid selection_rule: {selection_rule}")
+    seed = 0 if rbits < 0 else rbits
+    return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, None)
+
+
+def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
+    for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), ("alpha", alpha)):
+        nat.require_gpu_tensor(t, name)
+        if not t.is_contiguous():
+            raise RuntimeError(f"gemm: {name} must be contiguous")
+        if t.device != a.device:
+            raise RuntimeError("gemm: all operands must be on the same GPU")
+    if a.dtype != torch.uint8 or b.dtype != torch.uint8:
+        raise RuntimeError("A and B must be uint8")
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("A and B must be 2D")
+    if a_sf.dtype != torch.float8_e4m3fn or b_sf.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("A_sf and B_sf must be Float8_e4m3fn")
+    m, ka = a.shape[0], a.shape[1] * 2
+    n, kb = b.shape[0], b.shape[1] * 2
+    if ka < 16 or kb < 16:
+        raise RuntimeError("K-dim must be >= 16")
+    if ka != kb:
+        raise RuntimeError(f"Inner dims mismatch: {ka} vs {kb}")
+    if a_sf.numel() * 16 != m * ka:
+        raise RuntimeError("A_sf size mismatch")
+    if b_sf.numel() * 16 != n * kb:
+        raise RuntimeError("B_sf size mismatch")
+    out = torch.empty(m, n, dtype=out_dtype, device=a.device)
+    with torch.cuda.device(a.device):
+        rc = nat.lib().fos_gemm_nvfp4(
+            a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(),
+            m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n, nat.current_stream(a.device),
+        )
+    nat.check(rc, "fouroversix::gemm_nvfp4nvfp4_accum_fp32")
+    return out
+
+
+def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+    nat.require_gpu_tensor(values, "values")
+    rows_p, cols_p = values.shape[0], values.shape[1] * 2
+    out = torch.empty(rows, cols, dtype=out_dtype, device=values.device)
+    if rows == 0 or cols == 0:
+        return out
+    amax32 = amax.reshape(1).to(device=values.device, dtype=torch.float32)
+    with torch.cuda.device(values.device):
+        rc = nat.lib().fos_dequantize(
+            values.contiguous().data_ptr(), scale_factors.contiguous().data_ptr(), amax32.data_ptr(),
+            dtype, sf_layout, divisor, rows, cols, rows_p, cols_p,
+            out.data_ptr(), nat.TORCH_TO_T[out_dtype], cols, nat.current_stream(values.device),
+        )
+    nat.check(rc, "fouroversix::dequantize")
+    return out
+
+
+_LIB.impl("quantize", _quantize_ref_schema, "CUDA")
+_LIB.impl("quantize_ex", _quantize_impl, "CUDA")
+_LIB.impl(
+    "gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt",
+    lambda a, b, a_sf, b_sf, alpha: _gemm_impl(a, b, a_sf, b_sf, alpha, torch.bfloat16),
+    "CUDA",
+)
+_LIB.impl(
+    "gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt",
+    lambda a, b, a_sf, b_sf, alpha: _gemm_impl(a, b, a_sf, b_sf, alpha, torch.float16),
+    "CUDA",
+)
+_LIB.impl("dequantize", _dequantize_impl, "CUDA")
+
+
+def _fake_quantize_shapes(x):
+    rows_p, cols_p = _padded(x.shape[0], x.shape[1])
+    return (
+        torch.empty(rows_p, cols_p // 2, dtype=torch.uint8, device=x.device),
+        torch.empty(rows_p * cols_p // 16, dtype=torch.float8_e4m3fn, device=x.device),
+        torch.empty(1, dtype=torch.float32, device=x.device),
+    )
+
+
+@torch.library.register_fake("fouroversix::quantize")
+def _(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
+    return _fake_quantize_shapes(x)
+
+
+@torch.library.register_fake("fouroversix::quantize_ex")
+def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
+    return _fake_quantize_shapes(x)
+
+
+@torch.library.register_fake("fouroversix::gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt")
+def _(a, b, a_sf, b_sf, alpha):
+    return torch.empty(a.shape[0], b.shape[0], dtype=torch.bfloat16, device=a.device)
+
+
+@torch.library.register_fake("fouroversix::gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt")
+def _(a, b, a_sf, b_sf, alpha):
+    return torch.empty(a.shape[0], b.shape[0], dtype=torch.float16, device=a.device)
+
+
+@torch.library.register_fake("fouroversix::dequantize")
+def _(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+    return torch.empty(rows, cols, dtype=out_dtype, device=values.device)
+
+
+def quantize(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
+    """Same call as the reference's ``fouroversix.quantize.cuda.ops.quantize``."""
+    return torch.ops.fouroversix.quantize.default(
+        x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits
+    )
+
+
+def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax=None):
+    return torch.ops.fouroversix.quantize_ex.default(
+        x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax
+    )
+
+
+def gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha):
+    return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt.default(a, b, a_sf, b_sf, alpha)
+
+
+def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
+    return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
+
+
+def dequantize(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+    return torch.ops.fouroversix.dequantize.default(
+        values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype
+    )

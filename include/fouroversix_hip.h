@@ -1,0 +1,127 @@
+/*
+ * fouroversix_hip.h -- C ABI of the gfx950 (MI355X) quantize / FP4-matmul library.
+ *
+ * Plain pointers and sizes only; every pointer except the error strings is DEVICE memory.
+ * All entry points are asynchronous on the given HIP stream, never synchronise, and keep
+ * no mutable global state, so they are safe to call from several host threads on
+ * different streams.  Return value: 0 on success, a negative FOS_E_* code otherwise
+ * (nothing is launched when an argument check fails).
+ *
+ * Each function names the interface of the reference (mit-han-lab/fouroversix, paths
+ * relative to its tree) that it stands in for.
+ */
+#ifndef FOUROVERSIX_HIP_H
+#define FOUROVERSIX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *fos_stream_t; /* a hipStream_t; NULL = the default stream */
+
+enum {
+    FOS_OK = 0,
+    FOS_E_BAD_SHAPE = -1,     /* negative / zero-size / unsupported dimension */
+    FOS_E_BAD_ALIGNMENT = -2, /* pointer or leading dimension not aligned as documented */
+    FOS_E_UNSUPPORTED = -3,   /* format / rule / rounding combination without a kernel */
+    FOS_E_NULL_POINTER = -4,
+    FOS_E_WORKSPACE = -5, /* workspace missing or too small */
+    FOS_E_LAUNCH = -6     /* hipGetLastError() reported a launch failure */
+};
+
+/* formats, mirroring DataType members of src/fouroversix/utils.py:13-41 */
+enum { FOS_DTYPE_NVFP4 = 0, FOS_DTYPE_IF4 = 1 };
+/* scale rules with the ids of ScaleRule.cuda_id, src/fouroversix/utils.py:271-280 and
+ * csrc/quantize/fp4_quant.cu:111-119 */
+enum { FOS_RULE_STATIC_6 = 0, FOS_RULE_STATIC_4 = 1, FOS_RULE_MAE = 2, FOS_RULE_MSE = 3, FOS_RULE_ABS_MAX = 4 };
+/* RoundStyle, src/fouroversix/utils.py:223-247 */
+enum { FOS_ROUND_NEAREST = 0, FOS_ROUND_STOCHASTIC = 1, FOS_ROUND_STOCHASTIC_UNBIASED = 2 };
+/* block-scale layout: row-major [rows, cols/16], or the 128x4-tile layout of
+ * to_blocked(), src/fouroversix/quantize/utils.py:88-96 */
+enum { FOS_SF_LINEAR = 0, FOS_SF_TILED_128X4 = 1 };
+/* input / output element types */
+enum { FOS_T_BF16 = 0, FOS_T_F16 = 1, FOS_T_F32 = 2 };
+
+/* Library version (major * 10000 + minor * 100 + patch). */
+int fos_version(void);
+
+/* Human-readable text for a return code (host pointer, static storage). */
+const char *fos_error_string(int code);
+
+/* Rows / columns of the padded outputs: rows up to a multiple of 128, columns up to a
+ * multiple of 64 (QuantizedTensor, src/fouroversix/quantize/quantized_tensor.py:65-78). */
+int64_t fos_padded_rows(int64_t rows);
+int64_t fos_padded_cols(int64_t cols);
+
+/* Bytes of device workspace fos_quantize needs for an [rows, cols] input (never 0). */
+size_t fos_quantize_workspace_bytes(int64_t rows, int64_t cols);
+
+/*
+ * amax[0] = max |x| over a row-major 16-bit float matrix (pass 1 of fos_quantize on its
+ * own).  Stands in for `x.abs().max().float()` of the reference quantizer
+ * (src/fouroversix/quantize/pytorch/reference.py:573-578; the prologue kernel of the
+ * native op, src/fouroversix/csrc/include/fp4_quant_kernel.h:195-215).  Same workspace
+ * as fos_quantize.
+ */
+int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, float *amax,
+             void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * Quantize a row-major 16-bit float matrix x[rows, cols] (leading dimension ld elements)
+ * to packed 4-bit codes with one E4M3 scale per 1x16 block and one FP32 tensor scale.
+ * Stands in for torch.ops.fouroversix.quantize (src/fouroversix/csrc/bindings.cpp:28,
+ * csrc/quantize/fp4_quant.cu:99-239) with the semantics of the reference's PyTorch
+ * backend (src/fouroversix/quantize/pytorch/backend.py:39-121,
+ * quantize/pytorch/reference.py:555-679): the input is zero-padded to
+ * (fos_padded_rows, fos_padded_cols) and every padded output element is written.
+ *
+ *   x_type      FOS_T_BF16 or FOS_T_F16
+ *   dtype       FOS_DTYPE_*; rule FOS_RULE_* (IF4 takes only the adaptive rules)
+ *   round_style FOS_ROUND_*; seed/offset key the Philox dither of the stochastic styles
+ *   block2d     non-zero: one scale and one decision per 16x16 tile
+ *   sf_layout   FOS_SF_* layout of `sf`
+ *   codes       u8 [rows_p, cols_p / 2], low nibble = even column
+ *   sf          u8 [rows_p * cols_p / 16] E4M3 bytes (IF4: bit 7 marks integer blocks)
+ *   amax        f32[1]; written with max|x| unless amax_is_input, in which case it is read
+ *   workspace   >= fos_quantize_workspace_bytes(rows, cols) bytes, 256-byte aligned
+ */
+int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                 int dtype, int rule, int round_style, int block2d,
+                 uint64_t seed, uint64_t offset, int sf_layout,
+                 uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                 void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * D[M, N] = alpha * sum_k (A[m,k] * sfA[m,k/16]) * (B[n,k] * sfB[n,k/16]), FP32
+ * accumulation, written as out_type (FOS_T_BF16 or FOS_T_F16) with leading dimension ldd.
+ * Stands in for torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_{bf16,fp16}_tnt
+ * (src/fouroversix/csrc/bindings.cpp:31-33, csrc/fp4_gemm.cu:40-154).
+ *   A  u8 [M, K/2], B u8 [N, K/2]: packed E2M1, low nibble = even k
+ *   sfA, sfB  E4M3 bytes in the FOS_SF_TILED_128X4 layout of [M, K/16] / [N, K/16]
+ *   alpha f32[1] on the device
+ * M and N must be multiples of 128 and K a multiple of 64 (the padded shapes that
+ * fos_quantize produces).
+ */
+int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                   const float *alpha, int64_t M, int64_t N, int64_t K,
+                   void *D, int out_type, int64_t ldd, fos_stream_t stream);
+
+/*
+ * out[rows, cols] = dequantized values of a quantized tensor, cropped to (rows, cols).
+ * Stands in for QuantizeBackendBase.dequantize (src/fouroversix/quantize/backend.py:89-160).
+ *   codes u8 [rows_p, cols_p/2], sf in sf_layout over [rows_p, cols_p/16], amax f32[1]
+ *   divisor = qmax * smax * adjustment of the tensor's scale rule and rounding style
+ *   out_type FOS_T_BF16 / FOS_T_F16 / FOS_T_F32, leading dimension ldo
+ */
+int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const float *amax,
+                   int dtype, int sf_layout, double divisor,
+                   int64_t rows, int64_t cols, int64_t rows_p, int64_t cols_p,
+                   void *out, int out_type, int64_t ldo, fos_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FOUROVERSIX_HIP_H */

@@ -1,0 +1,120 @@
+"""Parity of the gfx950 FP4 GEMM (and the linear layer on top of it) with the CPU oracle
+and the reference's matmul vectors.  Budget, as the reference holds its own backends to
+(tests/test_matmul.py:15,81-88): at most 1e-3 of the bf16 outputs differ at all; and
+max |diff| <= 1e-2 of the output range."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import fouroversix_amd as fos
+from gpu_utils import bits16, make_input, u8
+
+pytestmark = pytest.mark.gpu
+
+MISMATCH_BUDGET = 1e-3
+MAX_REL = 1e-2
+
+
+def check(out_bits, ref_bits, oracle, what):
+    frac = float((out_bits != ref_bits).mean())
+    a, b = oracle.bf16_bits_to_f32(out_bits), oracle.bf16_bits_to_f32(ref_bits)
+    rel = float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+    assert frac <= MISMATCH_BUDGET and rel <= MAX_REL, f"{what}: {frac:.2e} of outputs differ, max rel {rel:.2e}"
+
+
+@pytest.mark.parametrize("rule", ["static_6", "static_4", "mse"])
+@pytest.mark.parametrize(("m", "n", "k"), [(256, 256, 256), (256, 512, 1024), (1024, 256, 512), (512, 1024, 256),
+                                           (1024, 1024, 1024), (128, 128, 64)])
+def test_gemm_matches_oracle(oracle, m, n, k, rule):
+    a, b = make_input("randn", (m, k), 31), make_input("randn", (n, k), 32)
+    cfg = fos.QuantizationConfig(scale_rule=rule)
+    qa, qb = fos.quantize(a.cuda(), cfg), fos.quantize(b.cuda(), cfg)
+    out = fos.quantized_matmul(qa, qb)
+    assert out.shape == (m, n) and out.dtype == torch.bfloat16
+    ra, rb = oracle.quantize(a, scale_rule=rule), oracle.quantize(b, scale_rule=rule)
+    native, _ = oracle.gemm_nvfp4(ra.values, ra.scale_rows, rb.values, rb.scale_rows, oracle.gemm_alpha(ra, rb))
+    check(bits16(out), native[:m, :n], oracle, f"{m}x{n}x{k} {rule} (native form)")
+    pt, _ = oracle.quantized_matmul(ra, rb)
+    check(bits16(out), pt, oracle, f"{m}x{n}x{k} {rule} (dequantize-matmul form)")
+
+
+def test_gemm_matches_reference_vectors(oracle, golden_dir):
+    mm = np.load(os.path.join(golden_dir, "matmul.npz"))
+    for tag in sorted({k.rsplit(".", 1)[0] for k in mm.files}):
+        rule = str(mm[tag + ".rule"])
+        a = torch.from_numpy(mm[tag + ".a"].view(np.int16).copy()).view(torch.bfloat16).cuda()
+        b = torch.from_numpy(mm[tag + ".b"].view(np.int16).copy()).view(torch.bfloat16).cuda()
+        cfg = fos.QuantizationConfig(scale_rule=rule)
+        out = fos.quantized_matmul(a, b, input_config=cfg, other_config=cfg)
+        check(bits16(out), mm[tag + ".out"], oracle, tag)
+
+
+def test_gemm_fp16_output_and_mixed_rules(oracle):
+    a, b = make_input("randn", (256, 512), 33), make_input("weight", (384, 512), 34)
+    qa = fos.quantize(a.cuda(), fos.QuantizationConfig(scale_rule="mse"))
+    qb = fos.quantize(b.cuda(), fos.QuantizationConfig(scale_rule="static_6", block_scale_2d=True))
+    out = fos.quantized_matmul(qa, qb, out_dtype=fos.DataType.float16)
+    assert out.dtype == torch.float16 and out.shape == (256, 384)
+    ra = oracle.quantize(a, scale_rule="mse")
+    rb = oracle.quantize(b, scale_rule="static_6", block_scale_2d=True)
+    _, f32 = oracle.gemm_nvfp4(ra.values, ra.scale_rows, rb.values, rb.scale_rows, oracle.gemm_alpha(ra, rb))
+    expect = torch.from_numpy(f32[:256, :384].copy()).half()
+    got = out.cpu()
+    assert float((got != expect).float().mean()) <= MISMATCH_BUDGET
+    assert float((got.float() - expect.float()).abs().max() / expect.float().abs().max()) <= MAX_REL
+
+
+@pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), (16, 4096, 4096), (128, 14336, 4096), (2048, 4096, 14336)])
+def test_gemm_full_size_sampled(oracle, m, n, k):
+    """Headline and Llama-3-8B shapes: 192 sampled rows of each operand are multiplied by
+    the oracle (fp64 accumulation) and compared with the same entries of the GPU result."""
+    a, b = make_input("randn", (m, k), 5), make_input("randn", (n, k), 6)
+    cfg = fos.QuantizationConfig(scale_rule="mse")
+    qa, qb = fos.quantize(a.cuda(), cfg), fos.quantize(b.cuda(), cfg)
+    out = fos.quantized_matmul(qa, qb)
+    assert out.shape == (m, n)
+    g = torch.Generator("cpu").manual_seed(7)
+    rows = torch.randperm(m, generator=g)[: min(m, 192)].sort().values
+    cols = torch.randperm(n, generator=g)[:192].sort().values
+    va, vb = u8(qa.values), u8(qb.values)
+    mp, npad = va.shape[0], vb.shape[0]
+    sa = oracle.from_blocked(u8(qa.scale_factors).reshape(-1), mp, k // 16)
+    sb = oracle.from_blocked(u8(qb.scale_factors).reshape(-1), npad, k // 16)
+    alpha = float(fos.matmul.frontend.gemm_alpha(qa, qb))
+    ref, _ = oracle.gemm_nvfp4(va[rows.numpy()], sa[rows.numpy()], vb[cols.numpy()], sb[cols.numpy()], alpha)
+    got = bits16(out[rows.cuda()][:, cols.cuda()])
+    check(got, ref, oracle, f"{m}x{n}x{k}")
+
+
+def test_linear_layer_forward(oracle):
+    """quantize_model + FourOverSixLinear forward == oracle quantize (activations 1-D mse,
+    weights 2-D mse) + oracle matmul + bias."""
+    torch.manual_seed(0)
+    lin = nn.Linear(512, 384, bias=True, dtype=torch.bfloat16)
+    model = nn.Sequential(lin).cuda()
+    w, bias = lin.weight.detach().cpu().clone(), lin.bias.detach().cpu().clone()
+    fos.quantize_model(model, fos.ModelQuantizationConfig(weight_scale_2d=True))
+    layer = model[0]
+    assert isinstance(layer, fos.FourOverSixLinear)
+    layer.quantize_weight_()
+    assert layer.weight is None and int(layer.quantized_weight_metadata[0]) == 384
+    x = make_input("randn", (4, 50, 512), 35)
+    y = model(x.cuda())
+    assert y.shape == (4, 50, 384) and y.dtype == torch.bfloat16
+    rx = oracle.quantize(x.reshape(-1, 512), scale_rule="mse")
+    rw = oracle.quantize(w, scale_rule="mse", block_scale_2d=True)
+    assert np.array_equal(u8(layer.quantized_weight_values), rw.values)
+    assert np.array_equal(u8(layer.quantized_weight_scale_factors), rw.scale_factors)
+    o16, _ = oracle.gemm_nvfp4(rx.values, rx.scale_rows, rw.values, rw.scale_rows, oracle.gemm_alpha(rx, rw))
+    expect = torch.from_numpy(o16[:200, :384].view(np.int16).copy()).view(torch.bfloat16) + bias
+    got = y.reshape(200, 384).cpu()
+    assert float((got != expect).float().mean()) <= 2 * MISMATCH_BUDGET
+    # master-weight mode re-quantizes the weight on every call and must agree
+    lin2 = nn.Linear(512, 384, bias=True, dtype=torch.bfloat16)
+    lin2.load_state_dict({"weight": w, "bias": bias})
+    keep = fos.FourOverSixLinear(lin2.cuda(), fos.ModuleQuantizationConfig(weight_scale_2d=True, keep_master_weights=True))
+    assert torch.equal(keep(x.cuda()), y)

@@ -1,0 +1,207 @@
+"""Pins of the CPU oracle (oracle/fos_oracle.c) that do not need a GPU.
+
+Each test checks the oracle against something it was not derived from: vectors written by
+the reference itself, torch library routines, the reference's second statement of a
+rule, or a closed form.
+"""
+
+import glob
+import hashlib
+import os
+
+import numpy as np
+import pytest
+import torch
+
+QUANT_FILES = sorted(
+    f for f in glob.glob(os.path.join(os.path.dirname(__file__), "golden", "quantize_*.npz")) if "config1" not in f
+)
+
+
+def _keys(d):
+    return sorted({k.rsplit(".", 1)[0] for k in d.files if k.endswith(".values")})
+
+
+@pytest.mark.parametrize("path", QUANT_FILES, ids=[os.path.basename(p)[9:-4] for p in QUANT_FILES])
+def test_quantize_matches_reference_vectors(oracle, path):
+    """Bit-exact codes, scales (in the stored layout) and amax for every format / rule /
+    1-D / 2-D combination, incl. ragged shapes and sub-normal block scales."""
+    d = np.load(path)
+    for k in _keys(d):
+        dt, rule, dim = k.split(".")
+        q = oracle.quantize(d["x"], dtype=dt, scale_rule=rule, block_scale_2d=(dim == "2d"))
+        assert q.padded_shape == tuple(d[k + ".padded"]), k
+        assert q.blocked == bool(d[k + ".blocked"][0]), k
+        assert q.amax == d[k + ".amax"][0], k
+        assert np.array_equal(q.values, d[k + ".values"]), k
+        assert np.array_equal(q.scale_factors, d[k + ".sf"].reshape(-1)), k
+
+
+def test_quantize_config1_digest(oracle, golden_dir):
+    """1024x1024 randn seed 0, static_6 and mse: SHA-256 of codes and scales."""
+    d = np.load(os.path.join(golden_dir, "quantize_config1_1024x1024.npz"))
+    g = torch.Generator("cpu").manual_seed(0)
+    x = torch.randn(1024, 1024, generator=g).bfloat16()
+    xb = oracle.bf16_bits(x)
+    if hashlib.sha256(xb.tobytes()).hexdigest() != str(d["x_sha"]):
+        pytest.skip("torch.randn stream differs from the one the vectors were made with")
+    for rule in ("static_6", "mse"):
+        q = oracle.quantize(xb, scale_rule=rule)
+        assert q.amax == d[f"{rule}.amax"][0]
+        assert hashlib.sha256(q.values.tobytes()).hexdigest() == str(d[f"{rule}.values_sha"])
+        assert hashlib.sha256(q.scale_factors.tobytes()).hexdigest() == str(d[f"{rule}.sf_sha"])
+
+
+def test_dequantize_matches_reference_vectors(oracle, golden_dir):
+    for name in ("randn_256x128", "ragged_100x80", "tiny_blocks_128x128"):
+        d = np.load(os.path.join(golden_dir, f"quantize_{name}.npz"))
+        for k in sorted({k.rsplit(".", 1)[0] for k in d.files if k.endswith(".deq_bf16")}):
+            dt, rule, _ = k.split(".")
+            pad = tuple(d[k + ".padded"])
+            sf = d[k + ".sf"].reshape(-1)
+            rows = oracle.from_blocked(sf, pad[0], pad[1] // 16) if d[k + ".blocked"][0] else sf.reshape(pad[0], pad[1] // 16)
+            out = oracle.dequantize(d[k + ".values"], rows, d[k + ".amax"][0], dtype=dt, scale_rule=rule,
+                                    original_shape=tuple(d["shape"]))
+            assert hashlib.sha256(np.ascontiguousarray(out).tobytes()).hexdigest() == str(d[k + ".deq_f32_sha"]), k
+            bf = torch.from_numpy(out.copy()).bfloat16().view(torch.int16).numpy().view(np.uint16)
+            assert np.array_equal(bf, d[k + ".deq_bf16"]), k
+
+
+def test_matmul_within_reference_budget(oracle, golden_dir):
+    """The reference allows <= 1e-3 of the bf16 outputs to differ between its own matmul
+    backends (tests/test_matmul.py:15,81-88); the oracle is held to the same budget
+    against the PyTorch backend's outputs, in both the dequantize-matmul form and the
+    native alpha-in-epilogue form."""
+    mm = np.load(os.path.join(golden_dir, "matmul.npz"))
+    for tag in sorted({k.rsplit(".", 1)[0] for k in mm.files}):
+        rule = str(mm[tag + ".rule"])
+        qa = oracle.quantize(mm[tag + ".a"], scale_rule=rule)
+        qb = oracle.quantize(mm[tag + ".b"], scale_rule=rule)
+        ref = mm[tag + ".out"]
+        o16, _ = oracle.quantized_matmul(qa, qb)
+        assert (o16 != ref).mean() <= 1e-3, tag
+        g16, _ = oracle.gemm_nvfp4(qa.values, qa.scale_rows, qb.values, qb.scale_rows, oracle.gemm_alpha(qa, qb))
+        assert (g16[: ref.shape[0], : ref.shape[1]] != ref).mean() <= 1e-3, tag
+        rel = np.abs(oracle.bf16_bits_to_f32(o16) - oracle.bf16_bits_to_f32(ref)).max() / np.abs(
+            oracle.bf16_bits_to_f32(ref)).max()
+        assert rel <= 1e-2
+
+
+def test_e4m3_cast_equals_torch(oracle):
+    """torch's own float32 -> float8_e4m3fn cast is the reference semantics
+    (reference.py:225): every bf16-representable value plus dense samples around every
+    rounding boundary."""
+    L = oracle.lib()
+    vals = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    grid = torch.tensor([L.fos_oracle_e4m3_to_f32(b) for b in range(0x7F)], dtype=torch.float64)
+    mids = (grid[:-1] + grid[1:]) / 2
+    near = torch.cat([mids * (1 + e) for e in (-1e-6, -6e-8, 0.0, 6e-8, 1e-6)]).float()
+    extra = torch.tensor([0.0, 2.0**-10, 2.0**-10 * 1.0000001, 463.9, 464.0, 464.1, 479.9])
+    allv = torch.cat([vals, near, extra])
+    allv = allv[allv < 480]  # beyond that torch yields NaN patterns; the scale path cannot get there
+    expect = allv.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = np.array([L.fos_oracle_e4m3_from_f32(float(v)) for v in allv.tolist()], dtype=np.uint8)
+    assert np.array_equal(got, expect)
+    # decode against torch's widening cast
+    back = torch.arange(0, 0x7F, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(back, grid.float().numpy())
+
+
+def test_e2m1_rounding_equals_threshold_table(oracle):
+    """The reference states round-to-nearest a second time as thresholds
+    (kernels/triton/fp4.py:21-41): <=.25 0, <.75 .5, <=1.25 1, <1.75 1.5, <=2.5 2,
+    <3.5 3, <=5 4, else 6.  Brute force over every non-negative bf16 below 7."""
+    L = oracle.lib()
+    vals = torch.arange(0, 0x7F80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    vals = vals[vals < 7.0].tolist()
+
+    def table(a):
+        if a <= 0.25: return 0.0
+        if a < 0.75: return 0.5
+        if a <= 1.25: return 1.0
+        if a < 1.75: return 1.5
+        if a <= 2.5: return 2.0
+        if a < 3.5: return 3.0
+        if a <= 5.0: return 4.0
+        return 6.0
+
+    for a in vals:
+        assert L.fos_oracle_e2m1_rtn(a) == table(a), a
+        assert L.fos_oracle_e2m1_rtn(-a) == -table(a), a
+    # the unclamped top regime: [7, 9) -> 8 (reference.py:38)
+    assert L.fos_oracle_e2m1_rtn(7.0) == 8.0 and L.fos_oracle_e2m1_rtn(8.9) == 8.0
+    # codes <-> values (kernels/triton/fp4.py:78-102)
+    mags = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    for c in range(16):
+        assert L.fos_oracle_e2m1_decode(c) == (-1.0 if c & 8 else 1.0) * mags[c & 7]
+
+
+def test_sum_order_equals_torch_sum(oracle):
+    """The mse/mae decisions hinge on torch.sum(dim=-1)'s fp32 summation order over 16 and
+    256 elements; the oracle's order must reproduce torch.sum on this host bit for bit."""
+    L = oracle.lib()
+    g = torch.Generator("cpu").manual_seed(5)
+    for n, fn in ((16, L.fos_oracle_sum16), (256, L.fos_oracle_sum256)):
+        v = (torch.randn(20000, n, generator=g) ** 2) * torch.logspace(-3, 3, 20000).unsqueeze(1)
+        expect = v.sum(dim=-1).numpy()
+        arr = np.ascontiguousarray(v.numpy())
+        got = np.array([fn(arr[i].ctypes.data) for i in range(arr.shape[0])], dtype=np.float32)
+        assert np.array_equal(got, expect), f"sum over {n} differs from torch.sum on this host"
+
+
+def test_closed_forms(oracle):
+    """Inputs of the reference's own tests (tests/test_quantize.py:155-164) whose outputs
+    follow from the definition."""
+    z = np.zeros((128, 64), dtype=np.uint16)
+    for rule in ("static_6", "mse"):
+        q = oracle.quantize(z, scale_rule=rule)
+        assert q.amax == 0 and not q.values.any() and not q.scale_factors.any()
+    ones = np.full((128, 64), 0x3F80, dtype=np.uint16)
+    q = oracle.quantize(ones, scale_rule="static_6")
+    assert q.amax == 1 and (q.values == 0x77).all() and (q.scale_factors == 0x7E).all()
+    q = oracle.quantize(ones, scale_rule="static_4")
+    assert (q.values == 0x66).all() and (q.scale_factors == 0x7E).all()
+    q = oracle.quantize(ones, scale_rule="mse")  # both candidates exact, tie goes to "6"
+    assert (q.values == 0x77).all() and (q.scale_factors == 0x78).all()
+    # 2-D scaling: 16 equal scale bytes down every tile column, and W / W.T commute
+    g = torch.Generator("cpu").manual_seed(3)
+    w = (0.02 * torch.randn(128, 128, generator=g)).bfloat16()
+    q = oracle.quantize(w, scale_rule="static_6", block_scale_2d=True)
+    assert (q.scale_rows.reshape(8, 16, 8) == q.scale_rows.reshape(8, 16, 8)[:, :1]).all()
+    qt = oracle.quantize(w.T.contiguous(), scale_rule="static_6", block_scale_2d=True)
+    a = oracle.dequantize(q.values, q.scale_rows, q.amax, scale_rule="static_6")
+    b = oracle.dequantize(qt.values, qt.scale_rows, qt.amax, scale_rule="static_6")
+    assert np.array_equal(a, b.T)
+
+
+def test_tiled_layout_round_trip_and_formula(oracle):
+    """Offset formula (quantize/utils.py:88-96 restated in fp4_quant_kernel.h:447-454)
+    against the reshape/transpose statement, via torch on a ragged-tile shape."""
+    rows, cols = 256, 12
+    a = np.arange(rows * cols, dtype=np.uint32).astype(np.uint8).reshape(rows, cols)
+    t = torch.from_numpy(a)
+    expect = (
+        t.view(rows // 128, 128, cols // 4, 4).transpose(1, 2).reshape(-1, 4, 32, 4).transpose(1, 2).reshape(-1, 32, 16).flatten()
+    ).numpy()
+    got = oracle.to_blocked(a)
+    assert np.array_equal(got, expect)
+    assert np.array_equal(oracle.from_blocked(got, rows, cols), a)
+
+
+def test_stochastic_rounding_known_answers(oracle):
+    """The reference's SR known answers (tests/test_quantize.py:360-372): L2 distance of
+    dequantize(quantize(randn 1024^2)) to the input within 5 % of 137 (static_6) / 122
+    (mse), 158 / 139 for the unbiased variant; and the dither is unbiased in range."""
+    g = torch.Generator("cpu").manual_seed(0)
+    x = torch.randn(1024, 1024, generator=g).bfloat16()
+    xf = x.float().numpy()
+    for rule, style, expect in (("static_6", "stochastic", 137), ("mse", "stochastic", 122),
+                                ("static_6", "stochastic_unbiased", 158), ("mse", "stochastic_unbiased", 139)):
+        q = oracle.quantize(x, scale_rule=rule, round_style=style, seed=1234)
+        deq = oracle.dequantize(q.values, q.scale_rows, q.amax, scale_rule=rule, round_style=style)
+        deq = torch.from_numpy(deq).bfloat16().float().numpy()
+        dist = float(np.sqrt(((deq - xf) ** 2).sum()))
+        assert abs(dist - expect) / expect < 0.05, (rule, style, dist)
+    q = oracle.quantize(x, scale_rule="static_6", round_style="stochastic", seed=7)
+    deq = oracle.dequantize(q.values, q.scale_rows, q.amax, scale_rule="static_6", round_style="stochastic")
+    assert abs(float((deq - xf).mean())) < 2e-3
