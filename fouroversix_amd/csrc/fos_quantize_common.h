@@ -1,0 +1,315 @@
+// Shared pieces of the gfx950 quantize kernels: launch parameters, workgroup reductions and
+// the operation-by-operation ("generic") quantisation of one 1x16 block, which restates
+// the reference's PyTorch backend one IEEE fp32 rounding per reference operation
+// (src/fouroversix/quantize/pytorch/reference.py:30-63, 184-552).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fos_device.h"
+#include "fouroversix_hip.h"
+
+namespace fos {
+
+
+constexpr int kThreads = 256;
+constexpr int kMaxPartials = 1024;  // pairs of 32-bit words in the workspace
+
+struct QuantParams {
+    const uint16_t *x;
+    int64_t rows, cols, ld;      // logical input
+    int64_t rows_p, cols_p;      // padded output extents
+    uint8_t *codes;              // [rows_p, cols_p / 2]
+    uint8_t *sf;                 // rows_p * cols_p / 16 bytes
+    const uint32_t *partials;    // pass-1 results, pairs {max|x| as f32 bits, 1 if a -0.0 was seen}
+    int n_partials;              // number of pairs; 0 = `partials` points at a caller-supplied f32 amax
+    float *amax_out;             // written by workgroup 0 when not null
+    uint64_t seed, offset;
+    int sf_layout;
+    int tiles_x;                 // workgroup tiles along the columns
+    float c, qdiv, errdiv;       // f32(qmax*smax*adj), f32(qmax*adj), selection divisor
+};
+
+// ---- workgroup reductions ------------------------------------------------------------
+
+FOS_DEVICE uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+    typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+    u16x2 va = __builtin_bit_cast(u16x2, a), vb = __builtin_bit_cast(u16x2, b);
+    u16x2 r = __builtin_elementwise_max(va, vb);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+FOS_DEVICE uint32_t pk_min_i16(uint32_t a, uint32_t b) {
+    typedef int16_t i16x2 __attribute__((ext_vector_type(2)));
+    i16x2 va = __builtin_bit_cast(i16x2, a), vb = __builtin_bit_cast(i16x2, b);
+    i16x2 r = __builtin_elementwise_min(va, vb);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+FOS_DEVICE uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        uint32_t o = (uint32_t)__shfl_xor((int)v, off);
+        v = v > o ? v : o;
+    }
+    return v;
+}
+
+// Max over the workgroup; valid in every thread.
+FOS_DEVICE uint32_t block_max_u32(uint32_t v, uint32_t *smem /* >= 4 words */) {
+    v = wave_max_u32(v);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) smem[wave] = v;
+    __syncthreads();
+    uint32_t r = smem[0];
+#pragma unroll
+    for (int i = 1; i < kThreads / 64; ++i) r = r > smem[i] ? r : smem[i];
+    __syncthreads();
+    return r;
+}
+
+// Tensor-wide results of pass 1, valid in every thread: bits of max|x| and whether the
+// input may contain a negative zero (unknown, hence assumed, for a caller-supplied amax).
+FOS_DEVICE void reduce_partials(const QuantParams &p, uint32_t *smem, uint32_t &amax_bits, bool &maybe_negzero) {
+    if (p.n_partials == 0) {
+        amax_bits = p.partials[0];
+        maybe_negzero = true;
+        return;
+    }
+    uint32_t m = 0, z = 0;
+    for (int i = threadIdx.x; i < p.n_partials; i += kThreads) {
+        const uint2 v = reinterpret_cast<const uint2 *>(p.partials)[i];
+        m = m > v.x ? m : v.x;
+        z |= v.y;
+    }
+    amax_bits = block_max_u32(m, smem);
+    maybe_negzero = block_max_u32(z, smem) != 0;
+}
+
+// ---------------------------------------------------------------------------------------
+// building blocks of one 1x16 block
+// ---------------------------------------------------------------------------------------
+
+struct QuantConsts {
+    float amax, enc, dec, qdiv, errdiv;
+};
+
+// compute_nv_scale_factors (reference.py:184-241) for one block maximum.
+FOS_DEVICE void block_scale(const QuantConsts &k, float bmax, bool expand, uint32_t &s, float &sf, float &inv) {
+    float s_hp = (k.amax == 0.0f) ? 0.0f : (bmax / k.qdiv) * k.enc;
+    if (expand) s_hp = s_hp * 1.5f;
+    s = e4m3_encode(s_hp);
+    sf = e4m3_decode(s);
+    inv = 1.0f / (k.dec * sf);
+}
+
+// E2M1 grid rounding of a magnitude (reference.py:30-51).  Round-to-nearest has no clamp
+// (a magnitude in [7, 9) gives 8, which the nibble encoding below spills into bit 3
+// exactly as the reference's bit extraction does); the dithered variant clamps to 6.
+template <bool SR>
+FOS_DEVICE float e2m1_round(float a, float u) {
+    float r;
+    if (SR) {
+        float r1 = __builtin_rintf((a + a) + u) * 0.5f;
+        float r2 = __builtin_rintf(a + u);
+        float r3 = fminf(2.0f * __builtin_rintf(a * 0.5f + u), 6.0f);
+        r = a < 2.0f ? r1 : (a < 4.0f ? r2 : r3);
+        r = (r == 0.0f) ? 0.0f : r;
+    } else {
+        float r1 = __builtin_rintf(a + a) * 0.5f;
+        float r2 = __builtin_rintf(a);
+        float r3 = 2.0f * __builtin_rintf(a * 0.5f);
+        r = a < 2.0f ? r1 : (a < 4.0f ? r2 : r3);
+    }
+    return r;
+}
+
+// Grid magnitude {0,.5,1,1.5,2,3,4,6,(8)} -> 3-bit code (8 for the overflow value).
+FOS_DEVICE uint32_t e2m1_mag_code(float r) {
+    float c = r < 2.0f ? (r + r) : (r < 4.0f ? r + 2.0f : r * 0.5f + 4.0f);
+    return (uint32_t)c;
+}
+
+template <bool SR>
+FOS_DEVICE float int4_round(float y, float u) {
+    if (SR) {
+        float t = fminf(fmaxf(fabsf(y) + u, -7.0f), 7.0f);
+        float r = __builtin_rintf(t);
+        r = (r == 0.0f) ? 0.0f : r;
+        return y < 0.0f ? -r : (y > 0.0f ? r : 0.0f * r);
+    }
+    return __builtin_rintf(fminf(fmaxf(y, -7.0f), 7.0f));
+}
+
+// torch.sum order over the 16 values of a 1x16 block.
+FOS_DEVICE float sum16(const float *e) {
+    float t = e[0] + e[8];
+#pragma unroll
+    for (int l = 1; l < 8; ++l) t = t + (e[l] + e[l + 8]);
+    return t;
+}
+
+// torch.sum order over a 16x16 tile flattened row-major, where this lane holds row
+// (lane & 15) of the tile in e[0..15] and the 16 rows lie along one DPP row.
+// Per column: even rows and odd rows are summed top to bottom (a chain of row_shr:2
+// adds; -0.0 is what lanes 0 and 1 receive, so they keep their own value), then
+// A[l] = ((E[l] + E[l+8]) + O[l]) + O[l+8] and the eight A[l] are summed left to right.
+// The result is valid in lane 14 of each row and broadcast from there.
+FOS_DEVICE float sum256_rows(const float *e) {
+    float t[16];
+#pragma unroll
+    for (int c = 0; c < 16; ++c) t[c] = e[c];
+#pragma unroll
+    for (int step = 0; step < 7; ++step) {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) t[c] = dpp_move<kDppRowShr + 2>(-0.0f, t[c]) + e[c];
+    }
+    float total = 0.0f;
+#pragma unroll
+    for (int l = 0; l < 8; ++l) {
+        float a = t[l] + t[l + 8];
+        a = a + dpp_move<kDppRowShl + 1>(0.0f, t[l]);
+        a = a + dpp_move<kDppRowShl + 1>(0.0f, t[l + 8]);
+        total = (l == 0) ? a : total + a;
+    }
+    const int lane = threadIdx.x & 63;
+    return __shfl(total, (lane & 48) | 14);
+}
+
+template <int RULE, bool TWO_D>
+FOS_DEVICE float reduce_error(const float *e) {
+    if (RULE == FOS_RULE_ABS_MAX) {
+        float m = e[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) m = fmaxf(m, e[i]);
+        return TWO_D ? row16_max(m) : m;
+    }
+    return TWO_D ? sum256_rows(e) : sum16(e);
+}
+
+template <int RULE>
+FOS_DEVICE float error_term(float deq, float x) {
+    float d = deq - x;
+    return RULE == FOS_RULE_MSE ? d * d : fabsf(d);
+}
+
+// Dither for the 16 elements of 1x16 block `blk`, candidate `cand`.
+FOS_DEVICE void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float *u) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        Philox4 p = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)(4 * cand + j),
+                                  (uint32_t)offset, (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) u[4 * j + i] = dither_from_word(p.v[i]);
+    }
+}
+
+// One 1x16 block (one row of a 16x16 tile when TWO_D): 8 input words -> 2 code words
+// and the scale byte.  `blk` = row * (cols_p / 16) + block column keys the dither.
+template <int DT, int RULE, int ROUND, bool TWO_D>
+FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t seed, uint64_t offset,
+                               uint64_t blk, uint32_t *codes, uint32_t &sbyte) {
+    constexpr bool SR = ROUND != FOS_ROUND_NEAREST;
+    constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        x[2 * i] = u2f(w[i] << 16);
+        x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+    }
+    float bmax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
+    if (TWO_D) bmax = row16_max(bmax);
+
+    uint32_t sA;
+    float sfA, invA;
+    block_scale(k, bmax, false, sA, sfA, invA);
+    float uA[16], uB[16];
+    if (SR) dither16(seed, offset, blk, 0, uA);
+
+    if (STATIC) {
+        uint32_t c0 = 0, c1 = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float xs = (sA != 0) ? x[i] * invA : 0.0f;
+            float r = e2m1_round<SR>(fabsf(xs), SR ? uA[i] : 0.0f);
+            uint32_t nib = e2m1_mag_code(r) | ((xs < 0.0f) ? 8u : 0u);
+            if (i < 8) c0 |= nib << (4 * i);
+            else c1 |= nib << (4 * (i - 8));
+        }
+        codes[0] = c0;
+        codes[1] = c1;
+        sbyte = sA;
+        return;
+    }
+
+    if (SR) dither16(seed, offset, blk, 1, uB);
+    float eA[16], eB[16];
+    uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+
+    if (DT == FOS_DTYPE_IF4) {
+        // select_intfloat (reference.py:328-425): candidate A = E2M1, candidate B = INT4
+        // on the same scale; B wins on a strictly smaller error.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float xs = (sA != 0) ? x[i] * invA : 0.0f;
+            float r = e2m1_round<SR>(fabsf(xs), SR ? uA[i] : 0.0f);
+            bool neg = xs < 0.0f;
+            float fq = neg ? -r : r;
+            uint32_t nibA = e2m1_mag_code(r) | (neg ? 8u : 0u);
+            float q = int4_round<SR>(xs * 1.16666666f, SR ? uB[i] : 0.0f);
+            uint32_t nibB = (uint32_t)((int)q) & 0xfu;
+            float deqA = ((fq * sfA) * k.amax) / k.errdiv;
+            float deqB = (((q * sfA) * k.amax) * 0.8571428571f) / k.errdiv;
+            eA[i] = error_term<RULE>(deqA, x[i]);
+            eB[i] = error_term<RULE>(deqB, x[i]);
+            if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
+            else { a1 |= nibA << (4 * (i - 8)); b1 |= nibB << (4 * (i - 8)); }
+        }
+        float errA = reduce_error<RULE, TWO_D>(eA);
+        float errB = reduce_error<RULE, TWO_D>(eB);
+        bool pickB = errB < errA;
+        codes[0] = pickB ? b0 : a0;
+        codes[1] = pickB ? b1 : a1;
+        sbyte = pickB ? (sA + 128u) : sA;
+        return;
+    }
+
+    // 4/6 (reference.py:262-325, 519-552): candidate A scales the block maximum to 6,
+    // candidate B to 4 (scale * 1.5); B wins on a strictly smaller error.
+    uint32_t sB;
+    float sfB, invB;
+    block_scale(k, bmax, true, sB, sfB, invB);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        float xsA = (sA != 0) ? x[i] * invA : 0.0f;
+        float xsB = (sB != 0) ? x[i] * invB : 0.0f;
+        float rA = e2m1_round<SR>(fabsf(xsA), SR ? uA[i] : 0.0f);
+        float rB = e2m1_round<SR>(fabsf(xsB), SR ? uB[i] : 0.0f);
+        bool negA = xsA < 0.0f, negB = xsB < 0.0f;
+        uint32_t nibA = e2m1_mag_code(rA) | (negA ? 8u : 0u);
+        uint32_t nibB = e2m1_mag_code(rB) | (negB ? 8u : 0u);
+        float deqA = (((negA ? -rA : rA) * sfA) * k.amax) / k.errdiv;
+        float deqB = (((negB ? -rB : rB) * sfB) * k.amax) / k.errdiv;
+        eA[i] = error_term<RULE>(deqA, x[i]);
+        eB[i] = error_term<RULE>(deqB, x[i]);
+        if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
+        else { a1 |= nibA << (4 * (i - 8)); b1 |= nibB << (4 * (i - 8)); }
+    }
+    float errA = reduce_error<RULE, TWO_D>(eA);
+    float errB = reduce_error<RULE, TWO_D>(eB);
+    bool pickB = errB < errA;
+    codes[0] = pickB ? b0 : a0;
+    codes[1] = pickB ? b1 : a1;
+    sbyte = pickB ? sB : sA;
+}
+
+// Offset of scale (r, c) inside the 128x4-tile layout (quantize/utils.py:88-96).
+FOS_DEVICE int64_t tiled_sf_offset(int64_t r, int64_t c, int64_t sf_cols) {
+    return ((r >> 7) * (sf_cols >> 2) + (c >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (c & 3);
+}
+
+
+}  // namespace fos

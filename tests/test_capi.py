@@ -55,13 +55,13 @@ def test_padding_and_workspace_queries(native):
 def test_argument_checks_need_no_device(native):
     """Every check below returns before the first HIP call."""
     L = native.lib()
-    buf = ctypes.create_string_buffer(4096)
+    buf = ctypes.create_string_buffer(1 << 16)
     p = ctypes.addressof(buf)
     p = (p + 255) & ~255
     q = lambda **kw: L.fos_quantize(  # noqa: E731
         kw.get("x", p), kw.get("x_type", 0), kw.get("rows", 128), kw.get("cols", 64), kw.get("ld", 64),
         kw.get("dtype", 0), kw.get("rule", 3), kw.get("round", 0), 0, 0, 0, kw.get("layout", 1),
-        kw.get("codes", p), kw.get("sf", p), kw.get("amax", p), 0, kw.get("ws", p), kw.get("ws_bytes", 4096), None)
+        kw.get("codes", p), kw.get("sf", p), kw.get("amax", p), 0, kw.get("ws", p), kw.get("ws_bytes", 1 << 15), None)
     assert q(x=None) == -4
     assert q(rows=0) == -1
     assert q(ld=32) == -1
