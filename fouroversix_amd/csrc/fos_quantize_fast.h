@@ -90,83 +90,253 @@ FOS_DEVICE float candidate_residual(float fq, const FastLutEntry &e, float x) {
     return __builtin_fmaf(p2, mult, -x);
 }
 
-// One 1x16 block on the fast path.  Returns false when the block must be redone by the
-// operation-by-operation path (sub-normal block scale).  `rq` = RN(1 / qdiv).
+// ---------------------------------------------------------------------------------------
+// 4/6-MSE with a certified shortcut
+// ---------------------------------------------------------------------------------------
+//
+// The exact decision compares E_k = sum_i fl(fl(deq_i - x_i)^2), k in {6, 4}, which costs
+// ~8 instructions per element and candidate.  In the block's scaled domain the same
+// quantity is h_k^2 * S_k with S_k = sum_i (fq_i - x_i / h_k)^2 and h_k = s_k * amax / 1536,
+// and S_k is 4 instructions per element (the scaled value x_i * inv_k is needed for the
+// rounding anyway).  With u = 2^-24, |x_i / h_k| <= 6.5 and |fq_i - x_i / h_k| <= 1, a
+// term-by-term bound of every rounding in both evaluations gives
+//     |E_k - h_k^2 S~_k| <= h_k^2 * u * (330 sqrt(S_k) + 40 S_k)        (16 elements)
+// (5 roundings from amax to x*inv: 33u absolute on the scaled value; 7u on the reference's
+// residual; 16u relative on either sum; 256-element tiles multiply the two coefficients by
+// 4 and 16).  The kernel uses 2^-14 (sqrt(n/16) sqrt(S) + (n/16) S), three times that, as
+// the tolerance: when the two intervals do not overlap the comparison E_4 < E_6 is
+// decided by the shortcut, otherwise (a few blocks in 10^4 on real data; every block of a
+// tensor whose candidates tie exactly) the exact evaluation runs.
+
+// max / sum over the 16 lanes of a DPP row; every lane gets lane 0's result so that the
+// whole row takes the same branch.
+FOS_DEVICE float row16_sum_lane0(float v) {
+    v = v + dpp_move<kDppRowRor + 8>(v, v);
+    v = v + dpp_move<kDppRowRor + 4>(v, v);
+    v = v + dpp_move<kDppRowRor + 2>(v, v);
+    v = v + dpp_move<kDppRowRor + 1>(v, v);
+    const int lane = threadIdx.x & 63;
+    return __shfl(v, lane & 48);
+}
+
+// The two rare paths are real function calls (arguments and results by value, in
+// registers) written as rolled loops over the eight column pairs (l, l + 8) -- the order
+// in which torch.sum consumes a block -- so that their register needs and code size stay
+// out of the hot loop.  Arrays indexed by the loop counter live in scratch memory.
+struct Block16 {
+    uint32_t w[8];
+};
+struct BlockOut {
+    uint32_t c0, c1, s;
+};
+
+FOS_DEVICE float block_element(const uint32_t *w, int idx) {
+    const uint32_t word = w[idx >> 1];
+    return (idx & 1) ? u2f(word & 0xffff0000u) : u2f(word << 16);
+}
+
+// Column sum of one value per lane down the 16 rows of a tile, even and odd rows apart
+// (lane 14 ends with the even-row sum, lane 15 with the odd-row sum).
+FOS_DEVICE float tile_column_chain(float e) {
+    float t = e;
+#pragma unroll
+    for (int step = 0; step < 7; ++step) t = dpp_move<kDppRowShr + 2>(-0.0f, t) + e;
+    return t;
+}
+
+// Running reduction of the selection error over the column pairs, in torch.sum's order.
 template <int RULE, bool TWO_D>
-FOS_DEVICE bool quantize_block_fast(const uint32_t *w, const QuantConsts &k, float enc, float rq, bool canon,
-                                    const FastLutEntry *lut, uint32_t *codes, uint32_t &sbyte) {
-    constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
-    float x[16];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        x[2 * i] = u2f(w[i] << 16);
-        x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+FOS_DEVICE void accumulate_pair(float e_lo, float e_hi, int l, float &total) {
+    if (RULE == FOS_RULE_ABS_MAX) {
+        total = fmaxf(total, fmaxf(e_lo, e_hi));  // errors are >= 0 and total starts at 0
+    } else if (!TWO_D) {
+        const float pair = e_lo + e_hi;
+        total = l == 0 ? pair : total + pair;
+    } else {
+        const float t_lo = tile_column_chain(e_lo), t_hi = tile_column_chain(e_hi);
+        float a = t_lo + t_hi;
+        a = a + dpp_move<kDppRowShl + 1>(0.0f, t_lo);
+        a = a + dpp_move<kDppRowShl + 1>(0.0f, t_hi);
+        total = l == 0 ? a : total + a;
     }
-    if (canon) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) x[i] = x[i] + 0.0f;
-    }
-    float bmax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
-    if (TWO_D) bmax = row16_max(bmax);
+}
 
-    const float s_hp6 = div_const(bmax, k.qdiv, rq) * enc;
-    const float s_hp4 = s_hp6 * 1.5f;
-    const uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp6, s_hp4, 0, false);
-    const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
-    if (s6 < 8u) {
-        if (bmax == 0.0f) {  // an all-zero block: zero codes, zero scale
-            codes[0] = 0;
-            codes[1] = 0;
-            sbyte = 0;
-            return true;
+template <int RULE, bool TWO_D>
+FOS_DEVICE float finish_error(float total) {
+    if (!TWO_D) return total;
+    if (RULE == FOS_RULE_ABS_MAX) return row16_max(total);
+    const int lane = threadIdx.x & 63;
+    return __shfl(total, (lane & 48) | 14);
+}
+
+FOS_DEVICE float e2m1_value(uint32_t code) {
+    const uint32_t e = (code >> 1) & 3u, m = code & 1u;
+    const float v = e == 0 ? 0.5f * (float)m : u2f((126u + e) << 23 | m << 22);
+    return (code & 8u) ? -v : v;
+}
+
+// Exact selection of a block whose shortcut was inconclusive: the residuals of both
+// candidates from their packed codes, with the reference's rounding and order.
+template <int RULE, bool TWO_D>
+__device__ __attribute__((noinline)) bool exact_pick_b(Block16 blk, bool canon, uint32_t a0, uint32_t a1, uint32_t b0,
+                                                       uint32_t b1, FastLutEntry A, FastLutEntry B) {
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = blk.w[i];
+    const uint64_t ca = ((uint64_t)a1 << 32) | a0, cb = ((uint64_t)b1 << 32) | b0;
+    float totA = 0.0f, totB = 0.0f;
+#pragma nounroll
+    for (int l = 0; l < 8; ++l) {
+        float e[2][2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int idx = l + 8 * h;
+            float x = block_element(w, idx);
+            if (canon) x = x + 0.0f;
+            const float dA = candidate_residual(e2m1_value((uint32_t)(ca >> (4 * idx)) & 0xfu), A, x);
+            const float dB = candidate_residual(e2m1_value((uint32_t)(cb >> (4 * idx)) & 0xfu), B, x);
+            e[0][h] = RULE == FOS_RULE_MSE ? dA * dA : fabsf(dA);
+            e[1][h] = RULE == FOS_RULE_MSE ? dB * dB : fabsf(dB);
         }
-        return false;
+        accumulate_pair<RULE, TWO_D>(e[0][0], e[0][1], l, totA);
+        accumulate_pair<RULE, TWO_D>(e[1][0], e[1][1], l, totB);
     }
+    return finish_error<RULE, TWO_D>(totB) < finish_error<RULE, TWO_D>(totA);
+}
 
-    const FastLutEntry A = lut[s6];
-    if (STATIC) {
-        uint32_t c0 = 0, c1 = 0;
-        static_for<0, 4>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            c0 = pack_fp4<j>(c0, x[2 * j] * A.inv, x[2 * j + 1] * A.inv);
-            c1 = pack_fp4<j>(c1, x[8 + 2 * j] * A.inv, x[9 + 2 * j] * A.inv);
-        });
-        codes[0] = c0;
-        codes[1] = c1;
-        sbyte = s6;
-        return true;
+// Operation-by-operation form (sub-normal block scales, out-of-range tensors): the
+// arithmetic of quantize_block in fos_quantize_common.h, rolled.
+template <int RULE, bool TWO_D>
+__device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantConsts k) {
+    constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = blk.w[i];
+    float bmax = 0.0f;
+#pragma nounroll
+    for (int i = 0; i < 16; ++i) bmax = fmaxf(bmax, fabsf(block_element(w, i)));
+    if (TWO_D) bmax = row16_max(bmax);
+    uint32_t sA, sB = 0;
+    float sfA, invA, sfB = 0.0f, invB = 0.0f;
+    block_scale(k, bmax, false, sA, sfA, invA);
+    if (!STATIC) block_scale(k, bmax, true, sB, sfB, invB);
+    uint64_t ca = 0, cb = 0;
+    float totA = 0.0f, totB = 0.0f;
+#pragma nounroll
+    for (int l = 0; l < 8; ++l) {
+        float e[2][2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int idx = l + 8 * h;
+            const float x = block_element(w, idx);
+            const float xsA = (sA != 0) ? x * invA : 0.0f;
+            const float rA = e2m1_round<false>(fabsf(xsA), 0.0f);
+            const bool negA = xsA < 0.0f;
+            ca |= (uint64_t)(e2m1_mag_code(rA) | (negA ? 8u : 0u)) << (4 * idx);
+            if (!STATIC) {
+                const float xsB = (sB != 0) ? x * invB : 0.0f;
+                const float rB = e2m1_round<false>(fabsf(xsB), 0.0f);
+                const bool negB = xsB < 0.0f;
+                cb |= (uint64_t)(e2m1_mag_code(rB) | (negB ? 8u : 0u)) << (4 * idx);
+                const float deqA = (((negA ? -rA : rA) * sfA) * k.amax) / k.errdiv;
+                const float deqB = (((negB ? -rB : rB) * sfB) * k.amax) / k.errdiv;
+                e[0][h] = error_term<RULE>(deqA, x);
+                e[1][h] = error_term<RULE>(deqB, x);
+            }
+        }
+        if (!STATIC) {
+            accumulate_pair<RULE, TWO_D>(e[0][0], e[0][1], l, totA);
+            accumulate_pair<RULE, TWO_D>(e[1][0], e[1][1], l, totB);
+        }
     }
+    bool pickB = false;
+    if (!STATIC) pickB = finish_error<RULE, TWO_D>(totB) < finish_error<RULE, TWO_D>(totA);
+    const uint64_t c = pickB ? cb : ca;
+    return BlockOut{(uint32_t)c, (uint32_t)(c >> 32), pickB ? sB : sA};
+}
 
-    const FastLutEntry B = lut[s4];
-    uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
-    static_for<0, 4>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
-        a0 = pack_fp4<j>(a0, x[2 * j] * A.inv, x[2 * j + 1] * A.inv);
-        a1 = pack_fp4<j>(a1, x[8 + 2 * j] * A.inv, x[9 + 2 * j] * A.inv);
-        b0 = pack_fp4<j>(b0, x[2 * j] * B.inv, x[2 * j + 1] * B.inv);
-        b1 = pack_fp4<j>(b1, x[8 + 2 * j] * B.inv, x[9 + 2 * j] * B.inv);
-    });
-    float eA[16], eB[16];
-    static_for<0, 8>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
-        const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
-        const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
-        const float dA0 = candidate_residual(fa.x, A, x[2 * j]), dA1 = candidate_residual(fa.y, A, x[2 * j + 1]);
-        const float dB0 = candidate_residual(fb.x, B, x[2 * j]), dB1 = candidate_residual(fb.y, B, x[2 * j + 1]);
-        eA[2 * j] = RULE == FOS_RULE_MSE ? dA0 * dA0 : fabsf(dA0);
-        eA[2 * j + 1] = RULE == FOS_RULE_MSE ? dA1 * dA1 : fabsf(dA1);
-        eB[2 * j] = RULE == FOS_RULE_MSE ? dB0 * dB0 : fabsf(dB0);
-        eB[2 * j + 1] = RULE == FOS_RULE_MSE ? dB1 * dB1 : fabsf(dB1);
-    });
-    const float errA = reduce_error<RULE, TWO_D>(eA);
-    const float errB = reduce_error<RULE, TWO_D>(eB);
-    const bool pickB = errB < errA;
-    codes[0] = pickB ? b0 : a0;
-    codes[1] = pickB ? b1 : a1;
-    sbyte = pickB ? s4 : s6;
-    return true;
+// One 1x16 block, NVFP4 round-to-nearest, any rule; falls back by itself.
+template <int RULE, bool TWO_D>
+FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
+                                             bool in_range, const FastLutEntry *lut) {
+    constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
+    if (in_range) {
+        float x[16];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            x[2 * i] = u2f(blk.w[i] << 16);
+            x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
+        }
+        if (canon) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) x[i] = x[i] + 0.0f;
+        }
+        float bmax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
+        if (TWO_D) bmax = row16_max(bmax);
+
+        const float s_hp6 = div_const(bmax, k.qdiv, rq) * enc;
+        const float s_hp4 = s_hp6 * 1.5f;
+        const uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp6, s_hp4, 0, false);
+        const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
+        if (s6 >= 8u) {
+            const FastLutEntry A = lut[s6];
+            if (STATIC) {
+                uint32_t c0 = 0, c1 = 0;
+                static_for<0, 4>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    c0 = pack_fp4<j>(c0, x[2 * j] * A.inv, x[2 * j + 1] * A.inv);
+                    c1 = pack_fp4<j>(c1, x[8 + 2 * j] * A.inv, x[9 + 2 * j] * A.inv);
+                });
+                return BlockOut{c0, c1, s6};
+            }
+            const FastLutEntry B = lut[s4];
+            uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+            float SA = 0.0f, SB = 0.0f;
+            static_for<0, 8>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const float xa0 = x[2 * j] * A.inv, xa1 = x[2 * j + 1] * A.inv;
+                const float xb0 = x[2 * j] * B.inv, xb1 = x[2 * j + 1] * B.inv;
+                if (j < 4) {
+                    a0 = pack_fp4<(j & 3)>(a0, xa0, xa1);
+                    b0 = pack_fp4<(j & 3)>(b0, xb0, xb1);
+                } else {
+                    a1 = pack_fp4<(j & 3)>(a1, xa0, xa1);
+                    b1 = pack_fp4<(j & 3)>(b1, xb0, xb1);
+                }
+                if (RULE == FOS_RULE_MSE) {
+                    const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+                    const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
+                    const float ra0 = fa.x - xa0, ra1 = fa.y - xa1, rb0 = fb.x - xb0, rb1 = fb.y - xb1;
+                    SA = __builtin_fmaf(ra0, ra0, SA);
+                    SA = __builtin_fmaf(ra1, ra1, SA);
+                    SB = __builtin_fmaf(rb0, rb0, SB);
+                    SB = __builtin_fmaf(rb1, rb1, SB);
+                }
+            });
+            bool pickB = false, certain = false;
+            if (RULE == FOS_RULE_MSE) {
+                if (TWO_D) {
+                    SA = row16_sum_lane0(SA);
+                    SB = row16_sum_lane0(SB);
+                }
+                constexpr float c_sqrt = TWO_D ? 4.0f : 1.0f, c_lin = TWO_D ? 16.0f : 1.0f;
+                const float hA = A.d1 * A.d1, hB = B.d1 * B.d1;
+                const float EA = hA * SA, EB = hB * SB;
+                const float tA = hA * (0x1p-14f * (c_sqrt * __builtin_sqrtf(SA) + c_lin * SA));
+                const float tB = hB * (0x1p-14f * (c_sqrt * __builtin_sqrtf(SB) + c_lin * SB));
+                const bool surely_b = EB + tB < EA - tA;
+                const bool surely_a = EB - tB > EA + tA;
+                certain = surely_a || surely_b;
+                pickB = surely_b;
+            }
+            if (!certain) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+            return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
+        }
+        if (bmax == 0.0f) return BlockOut{0, 0, 0};  // an all-zero block: zero codes, zero scale
+    }
+    return generic_block<RULE, TWO_D>(blk, k);
 }
 
 }  // namespace fos

@@ -1,14 +1,205 @@
-// Instantiations of the pass-2 kernel for NVFP4 with round-to-nearest (the fast
-// formulation of fos_quantize_fast.h), kept in their own translation unit so that the
-// library builds in parallel.
+// Pass 2 for NVFP4 with round-to-nearest, around the fast block formulation of
+// fos_quantize_fast.h.  Two lane mappings:
+//
+//  * 1x16 blocks (quantize_nvfp4_rtn_rows_kernel): a wavefront covers 4 rows x 16 blocks,
+//    i.e. 512 contiguous bytes per row.  Measured on MI355X, a wavefront that touches 16
+//    rows x 128 bytes streams at ~4.1 TB/s while 4 rows x 512 bytes reaches ~6 TB/s, so the
+//    row-contiguous mapping is what the HBM-bound path uses.  A 256-thread workgroup
+//    covers 128 rows x 256 columns in eight steps of 16 rows (the next step's loads are
+//    issued before the current step is processed), stages the 4 complete 128x4 scale
+//    tiles in LDS and writes them as one contiguous 2 KiB run.
+//  * 16x16 tiles (quantize_nvfp4_rtn_kernel): the 16 rows of a tile must lie along one DPP
+//    row for the tile reductions, so a wavefront covers 16 rows x 4 blocks; persistent
+//    workgroups walk over 128 x 64 tiles with the next tile prefetched.
+#include <cstdlib>
+
 #include "fos_quantize_kernel.h"
 
 namespace fos {
 
+struct TileRegs {
+    Block16 b[2];
+};
+
+FOS_DEVICE void load_tile(const QuantParams &p, uint32_t tile, int lane, int wave, TileRegs &t) {
+    const int64_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - (uint32_t)tile_y * (uint32_t)p.tiles_x;
+    const int64_t c0 = (tile_x * 4 + (lane >> 4)) * 16;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int64_t r = tile_y * 128 + h * 64 + wave * 16 + (lane & 15);
+        if (r < p.rows && c0 < p.cols) {
+            const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
+            const uint4 lo = src[0], hi = src[1];
+            t.b[h].w[0] = lo.x; t.b[h].w[1] = lo.y; t.b[h].w[2] = lo.z; t.b[h].w[3] = lo.w;
+            t.b[h].w[4] = hi.x; t.b[h].w[5] = hi.y; t.b[h].w[6] = hi.z; t.b[h].w[7] = hi.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) t.b[h].w[i] = 0;
+        }
+    }
+}
+
+template <int RULE, bool TWO_D>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_kernel(const QuantParams p) {
+    __shared__ uint32_t red[4];
+    __shared__ uint32_t sf_tile[2][128];
+    __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
+
+    uint32_t amax_bits;
+    bool maybe_negzero;
+    reduce_partials(p, red, amax_bits, maybe_negzero);
+    QuantConsts k;
+    k.amax = u2f(amax_bits);
+    k.enc = p.c / k.amax;
+    k.dec = 1.0f / (p.c / k.amax);
+    k.qdiv = p.qdiv;
+    k.errdiv = p.errdiv;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
+    const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
+    const float enc_fast = in_range ? k.enc : 0.0f;
+    const float rq = 1.0f / k.qdiv;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t sf_cols = p.cols_p >> 4;
+    const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
+    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+
+    auto process = [&](uint32_t tile, const TileRegs &t, uint32_t *stage) {
+        const int64_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - (uint32_t)tile_y * (uint32_t)p.tiles_x;
+        const int64_t cb = tile_x * 4 + (lane >> 4);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int rr = h * 64 + wave * 16 + (lane & 15);
+            const int64_t r = tile_y * 128 + rr;
+            const BlockOut o = quantize_block_nvfp4_rtn<RULE, TWO_D>(t.b[h], k, enc_fast, rq, maybe_negzero, in_range, lut);
+            *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(o.c0, o.c1);
+            if (tiled) reinterpret_cast<uint8_t *>(stage)[(rr & 31) * 16 + (rr >> 5) * 4 + (lane >> 4)] = (uint8_t)o.s;
+            else p.sf[r * sf_cols + cb] = (uint8_t)o.s;
+        }
+        if (tiled) {
+            __syncthreads();
+            if (threadIdx.x < 128)
+                reinterpret_cast<uint32_t *>(p.sf + (tile_y * (sf_cols >> 2) + tile_x) * 512)[threadIdx.x] = stage[threadIdx.x];
+        }
+    };
+
+    // two tiles per trip so that the prefetch registers alternate without copies
+    TileRegs ta, tb;
+    uint32_t tile = blockIdx.x;
+    const uint32_t step = gridDim.x;
+    if (tile < n_tiles) load_tile(p, tile, lane, wave, ta);
+    while (tile < n_tiles) {
+        if (tile + step < n_tiles) load_tile(p, tile + step, lane, wave, tb);
+        process(tile, ta, sf_tile[0]);
+        tile += step;
+        if (tile >= n_tiles) break;
+        if (tile + step < n_tiles) load_tile(p, tile + step, lane, wave, ta);
+        process(tile, tb, sf_tile[1]);
+        tile += step;
+    }
+}
+
+
+// 1x16 blocks, row-contiguous mapping: lane -> block column (lane & 15) of row (lane >> 4)
+// within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns.
+template <int RULE>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_rows_kernel(
+    const QuantParams p) {
+    __shared__ uint32_t red[4];
+    __shared__ uint32_t sf_stage[4 * 128];  // 4 scale tiles of 512 bytes
+    __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
+
+    uint32_t amax_bits;
+    bool maybe_negzero;
+    reduce_partials(p, red, amax_bits, maybe_negzero);
+    QuantConsts k;
+    k.amax = u2f(amax_bits);
+    k.enc = p.c / k.amax;
+    k.dec = 1.0f / (p.c / k.amax);
+    k.qdiv = p.qdiv;
+    k.errdiv = p.errdiv;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
+    const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
+    const float enc_fast = in_range ? k.enc : 0.0f;
+    const float rq = 1.0f / k.qdiv;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t tile_y = blockIdx.x / (uint32_t)p.tiles_x, tile_x = blockIdx.x - tile_y * (uint32_t)p.tiles_x;
+    const int64_t sf_cols = p.cols_p >> 4;
+    const int lb = lane & 15;                      // block column inside the tile
+    const int64_t cb = (int64_t)tile_x * 16 + lb;  // block column in the tensor
+    const int rr0 = wave * 4 + (lane >> 4);        // row inside a 16-row step
+    const bool col_ok = cb < sf_cols;
+    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    const uint16_t *src0 = p.x + ((int64_t)tile_y * 128 + rr0) * p.ld + cb * 16;
+    uint8_t *dst0 = p.codes + ((int64_t)tile_y * 128 + rr0) * (p.cols_p >> 1) + cb * 8;
+
+    auto load = [&](int g, Block16 &b) {
+        const int64_t r = (int64_t)tile_y * 128 + g * 16 + rr0;
+        if (col_ok && r < p.rows && cb * 16 < p.cols) {
+            const uint4 *src = reinterpret_cast<const uint4 *>(src0 + (int64_t)g * 16 * p.ld);
+            const uint4 lo = src[0], hi = src[1];
+            b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
+            b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) b.w[i] = 0;
+        }
+    };
+
+    Block16 cur, nxt;
+    load(0, cur);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        if (g + 1 < 8) load(g + 1, nxt);
+        if (col_ok) {
+            const int rr = g * 16 + rr0;
+            const BlockOut o = quantize_block_nvfp4_rtn<RULE, false>(cur, k, enc_fast, rq, maybe_negzero, in_range, lut);
+            *reinterpret_cast<uint2 *>(dst0 + (int64_t)g * 16 * (p.cols_p >> 1)) = make_uint2(o.c0, o.c1);
+            if (tiled)
+                reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)o.s;
+            else
+                p.sf[((int64_t)tile_y * 128 + rr) * sf_cols + cb] = (uint8_t)o.s;
+        }
+        cur = nxt;
+    }
+    if (tiled) {
+        __syncthreads();
+        // 4 scale tiles x 512 bytes, contiguous in the output; 8 bytes per thread
+        const int t = threadIdx.x >> 6;
+        const int64_t group = (int64_t)tile_x * 4 + t;
+        if (group < (sf_cols >> 2)) {
+            uint2 *dst = reinterpret_cast<uint2 *>(p.sf + ((int64_t)tile_y * (sf_cols >> 2) + group) * 512);
+            dst[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
+        }
+    }
+}
+
 template <int RULE>
 static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
-    if (two_d) launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
-    else launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
+    if (!aligned) {
+        if (two_d) launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
+        else launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
+        return;
+    }
+    if (!two_d) {
+        p.tiles_x = (int)((p.cols_p + 255) / 256);
+        const int64_t n = (p.rows_p / 128) * p.tiles_x;
+        hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE>), dim3((unsigned)n), dim3(kThreads), 0, s, p);
+        return;
+    }
+    p.tiles_x = (int)(p.cols_p / 64);
+    const int64_t n_tiles = (p.rows_p / 128) * p.tiles_x;
+    // Persistent grid: a few workgroups per compute unit (256 CUs), fewer when the tensor
+    // is small.  FOS_QUANT_GRID overrides the count for tuning runs.
+    int64_t grid = 256 * 6;
+    if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
+    if (grid > n_tiles) grid = n_tiles;
+    hipLaunchKernelGGL((quantize_nvfp4_rtn_kernel<RULE, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
 void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {

@@ -88,11 +88,15 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
         const int64_t cb = cb_base + (it >> 1) * 4;
         if (cb >= sf_cols) continue;  // whole wave-row group lies past the padded width
         uint32_t codes[2], sbyte;
-        bool done = false;
         if (FAST) {
-            if (in_range) done = quantize_block_fast<RULE, TWO_D>(w[it], k, enc_fast, rq, maybe_negzero, lut, codes, sbyte);
-        }
-        if (!done)
+            Block16 blk;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) blk.w[i] = w[it][i];
+            const BlockOut o = quantize_block_nvfp4_rtn<RULE, TWO_D>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut);
+            codes[0] = o.c0;
+            codes[1] = o.c1;
+            sbyte = o.s;
+        } else
             quantize_block<DT, RULE, ROUND, TWO_D>(w[it], k, p.seed, p.offset, (uint64_t)(r * sf_cols + cb), codes,
                                                    sbyte);
         *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(codes[0], codes[1]);
@@ -126,6 +130,13 @@ void launch_quantize(QuantParams &p, bool aligned, hipStream_t s) {
     // workgroups to fill the chip; narrow tiles for small or unaligned tensors.
     const int64_t tiles_y = p.rows_p / 128;
     const int64_t groups = p.cols_p / 64;
+    if constexpr (FAST) {
+        // aligned NVFP4 round-to-nearest inputs go to the persistent kernel instead
+        p.tiles_x = (int)groups;
+        hipLaunchKernelGGL((quantize_kernel<FAST, DT, RULE, ROUND, TWO_D, 1, false>),
+                           dim3((unsigned)(tiles_y * p.tiles_x)), dim3(kThreads), 0, s, p);
+        return;
+    }
     if (aligned && groups % 4 == 0 && tiles_y * (groups / 4) >= 1024) {
         p.tiles_x = (int)(groups / 4);
         hipLaunchKernelGGL((quantize_kernel<FAST, DT, RULE, ROUND, TWO_D, 4, true>),

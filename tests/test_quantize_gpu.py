@@ -91,6 +91,32 @@ def test_ragged_shapes_are_zero_padded(oracle, shape):
         assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), f"{shape} {cfg}")
 
 
+@pytest.mark.parametrize("scale", [2.0**-110, 2.0**-118, 2.0**105])
+@pytest.mark.parametrize("two_d", [False, True], ids=["1d", "2d"])
+def test_extreme_ranges_take_the_operation_by_operation_path(oracle, scale, two_d):
+    """Tensors whose maximum leaves [2^-100, 2^100] (fp32 intermediates of the scale math
+    go sub-normal or overflow) must still match the oracle bit for bit."""
+    x = (make_input("randn", (256, 128), 12).float() * scale).bfloat16()
+    for rule in ("mse", "static_6", "abs_max"):
+        q = hip_quantize(x, scale_rule=rule, block_scale_2d=two_d)
+        ref = oracle.quantize(x, scale_rule=rule, block_scale_2d=two_d)
+        assert_same_quantization(q, ref, f"scale {scale} {rule}")
+
+
+def test_negative_zero_inputs(oracle):
+    """-0.0 encodes as +0 (the reference multiplies by sign(x)); a small negative value
+    that rounds to zero keeps its sign bit."""
+    x = make_input("randn", (256, 256), 13)
+    x[::3, ::5] = -0.0
+    x[1::7, 3::11] = -1e-4
+    for cfg in (dict(scale_rule="mse"), dict(scale_rule="static_6"), dict(scale_rule="mse", block_scale_2d=True),
+                dict(dtype="if4", scale_rule="mse")):
+        assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), str(cfg))
+    x[:, :] = -0.0
+    q = hip_quantize(x, scale_rule="mse")
+    assert int(u8(q.values).max()) == 0 and int(u8(q.scale_factors).max()) == 0
+
+
 def test_strided_and_unaligned_inputs(oracle):
     base = make_input("randn", (256, 384), 4).cuda()
     view = base[:, 64:320]                      # ld 384, cols 256, 16-byte aligned
