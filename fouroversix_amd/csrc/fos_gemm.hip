@@ -7,8 +7,20 @@
 // src/fouroversix/quantize/backend.py:89-160), staged in LDS as fp16 and fed to
 // v_mfma_f32_32x32x16_f16 with FP32 accumulation; alpha is applied in the epilogue from
 // device memory (src/fouroversix/csrc/fp4_gemm.cu:143).
+//
+// Pipeline per workgroup (tile BM x BN x 64, BM = BN = threads / 2): every thread owns 32
+// codes of one A row and of one B row per K step.  Registers hold the packed data of step
+// k+2 (in flight from HBM) while step k+1 is dequantised into one LDS buffer and step k is
+// multiplied out of the other, so there is one barrier per K step and the VALU work of the
+// dequantisation issues in the shadow of the MFMAs.  The big tile (256 x 256, 8
+// wavefronts of 128 x 64) keeps LDS reads at ~75 % of their bandwidth; a 128 x 128 tile
+// serves shapes that are not multiples of 256 or too small to fill the chip otherwise.
+// Workgroups are numbered so that the tiles resident on one XCD (blockIdx % 8) form a
+// compact block of the output, which keeps their A/B panels in that XCD's L2.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <cstdlib>
 
 #include "fos_device.h"
 #include "fouroversix_hip.h"
@@ -25,7 +37,7 @@ struct GemmParams {
     const float *alpha;
     void *D;
     int64_t M, N, K, ldd;
-    int tiles_n;
+    int tiles_m, tiles_n;
 };
 
 // E4M3 byte (bits 0..6) -> fp16 pair {s, s}.  The byte at bit 7 of a half is the E4M3
@@ -47,106 +59,133 @@ FOS_DEVICE half8_t dequant8(uint32_t word, half2_t s) {
     return r;
 }
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int kGemmThreads = 256;
-constexpr int kPitch = BK + 8;  // halfs per LDS row (144 bytes: conflict-free 128-bit reads)
+constexpr int BK = 64;
+constexpr int kPitch = BK + 8;  // halfs per LDS row (144 bytes: conflict-free 128-bit accesses)
 
-// Tile 128 x 128 x 64, 4 wavefronts in a 2 x 2 arrangement, each 64 x 64 as 2 x 2 MFMA
-// 32x32x16 tiles.  The MFMA "A" operand is fed from the B matrix (rows n) and the "B"
-// operand from the A matrix (rows m), so that a lane's four consecutive accumulator
-// registers are four consecutive n of one output row and can be stored as 8 bytes.
-template <bool OUT_BF16>
-__global__ __launch_bounds__(kGemmThreads) void gemm_nvfp4_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) _Float16 lds_a[BM * kPitch];
-    __shared__ __attribute__((aligned(16))) _Float16 lds_b[BN * kPitch];
+// Packed operands of one K step as a thread holds them.
+struct Staged {
+    uint4 qa, qb;     // 32 codes of one A row / one B row
+    uint32_t sa, sb;  // the 4 scale bytes of that row's K step
+};
+
+// Output tile of workgroup `bid`: workgroups with equal bid % 8 share an XCD; give each
+// XCD a contiguous run of tiles, ordered in column bands of 8 tile rows.
+FOS_DEVICE void tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    int t = (bid & 7) * per_xcd + (bid >> 3);
+    if (t >= total || (total & 7) != 0) t = bid;  // ragged counts: plain order
+    constexpr int kBand = 8;
+    const int band = t / (kBand * tiles_n), in_band = t - band * kBand * tiles_n;
+    const int rows = (tiles_m - band * kBand) < kBand ? (tiles_m - band * kBand) : kBand;
+    tm = band * kBand + in_band % rows;
+    tn = in_band / rows;
+}
+
+// WAVES_M x WAVES_N wavefronts, each WM x WN MFMA tiles of 32 x 32.  The MFMA "A" operand
+// is fed from the B matrix (rows n) and the "B" operand from the A matrix (rows m), so
+// that a lane's four consecutive accumulator registers are four consecutive n of one
+// output row and can be stored as 8 bytes.
+template <int WAVES_M, int WAVES_N, int WM, int WN, bool OUT_BF16>
+__global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const GemmParams p) {
+    constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+    static_assert(BM == kThreadsG / 2 && BN == kThreadsG / 2, "one thread per half row of each operand");
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
+    _Float16 *lds_a[2] = {lds, lds + (BM + BN) * kPitch};
+    _Float16 *lds_b[2] = {lds + BM * kPitch, lds + (BM + BN) * kPitch + BM * kPitch};
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tile_n = blockIdx.x % p.tiles_n;
-    const int64_t tile_m = blockIdx.x / p.tiles_n;
-    const int64_t m0 = tile_m * BM, n0 = (int64_t)tile_n * BN;
-    const int64_t kbytes = p.K >> 1;      // packed bytes per row
-    const int64_t sf_groups = p.K >> 6;   // 4-block groups per row
+    int tile_m, tile_n;
+    tile_of(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int64_t kbytes = p.K >> 1;     // packed bytes per row
+    const int64_t sf_groups = p.K >> 6;  // 4-block groups per row
 
-    // global -> register staging: thread handles 32 codes (16 bytes) of one row of each operand
+    // global -> register staging: 32 codes (16 bytes) of one row of each operand
     const int ld_row = tid >> 1, ld_half = tid & 1;
     const uint8_t *a_ptr = p.A + (m0 + ld_row) * kbytes + ld_half * 16;
     const uint8_t *b_ptr = p.B + (n0 + ld_row) * kbytes + ld_half * 16;
-    const int sf_in_tile = (ld_row & 31) * 16 + (ld_row >> 5) * 4;
-    const uint8_t *sfa_ptr = p.sfA + tile_m * sf_groups * 512 + sf_in_tile;
-    const uint8_t *sfb_ptr = p.sfB + (int64_t)tile_n * sf_groups * 512 + sf_in_tile;
+    const int sf_in_tile = (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4;
+    const uint8_t *sfa_ptr = p.sfA + ((m0 + ld_row) >> 7) * sf_groups * 512 + sf_in_tile;
+    const uint8_t *sfb_ptr = p.sfB + ((n0 + ld_row) >> 7) * sf_groups * 512 + sf_in_tile;
+    const int64_t ksteps = p.K / BK;
 
-    const int wm = wave >> 1, wn = wave & 1;  // wave position in the 2 x 2 arrangement
-    float16_t acc[2][2];
+    auto fetch = [&](int64_t ks, Staged &s) {
+        s.qa = *reinterpret_cast<const uint4 *>(a_ptr + ks * 32);
+        s.qb = *reinterpret_cast<const uint4 *>(b_ptr + ks * 32);
+        s.sa = *reinterpret_cast<const uint32_t *>(sfa_ptr + ks * 512);
+        s.sb = *reinterpret_cast<const uint32_t *>(sfb_ptr + ks * 512);
+    };
+    // quarter q (0..3) of the staged data -> 8 halfs of each operand in LDS buffer `buf`
+    auto stage_quarter = [&](const Staged &s, int buf, int q) {
+        const uint32_t wa = q == 0 ? s.qa.x : q == 1 ? s.qa.y : q == 2 ? s.qa.z : s.qa.w;
+        const uint32_t wb = q == 0 ? s.qb.x : q == 1 ? s.qb.y : q == 2 ? s.qb.z : s.qb.w;
+        const int sh = 16 * ld_half + 8 * (q >> 1);
+        half8_t *da = reinterpret_cast<half8_t *>(lds_a[buf] + ld_row * kPitch + ld_half * 32);
+        half8_t *db = reinterpret_cast<half8_t *>(lds_b[buf] + ld_row * kPitch + ld_half * 32);
+        da[q] = dequant8(wa, e4m3_to_half2(s.sa >> sh));
+        db[q] = dequant8(wb, e4m3_to_half2(s.sb >> sh));
+    };
+
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    float16_t acc[WM][WN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < WM; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < WN; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    uint4 qa = *reinterpret_cast<const uint4 *>(a_ptr);
-    uint4 qb = *reinterpret_cast<const uint4 *>(b_ptr);
-    uint32_t sa = *reinterpret_cast<const uint32_t *>(sfa_ptr);
-    uint32_t sb = *reinterpret_cast<const uint32_t *>(sfb_ptr);
+    Staged st[2];
+    fetch(0, st[0]);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_quarter(st[0], 0, q);
+    if (ksteps > 1) fetch(1, st[1]);
+    __syncthreads();
 
-    const int64_t ksteps = p.K / BK;
-    for (int64_t ks = 0; ks < ksteps; ++ks) {
-        // dequantize the staged registers into LDS
-        {
-            half2_t s0 = e4m3_to_half2(sa >> (16 * ld_half));
-            half2_t s1 = e4m3_to_half2(sa >> (16 * ld_half + 8));
-            half8_t *dst = reinterpret_cast<half8_t *>(lds_a + ld_row * kPitch + ld_half * 32);
-            dst[0] = dequant8(qa.x, s0);
-            dst[1] = dequant8(qa.y, s0);
-            dst[2] = dequant8(qa.z, s1);
-            dst[3] = dequant8(qa.w, s1);
-            half2_t t0 = e4m3_to_half2(sb >> (16 * ld_half));
-            half2_t t1 = e4m3_to_half2(sb >> (16 * ld_half + 8));
-            half8_t *dstb = reinterpret_cast<half8_t *>(lds_b + ld_row * kPitch + ld_half * 32);
-            dstb[0] = dequant8(qb.x, t0);
-            dstb[1] = dequant8(qb.y, t0);
-            dstb[2] = dequant8(qb.z, t1);
-            dstb[3] = dequant8(qb.w, t1);
-        }
-        __syncthreads();
-        // prefetch the next K step while this one is multiplied
-        if (ks + 1 < ksteps) {
-            qa = *reinterpret_cast<const uint4 *>(a_ptr + (ks + 1) * 32);
-            qb = *reinterpret_cast<const uint4 *>(b_ptr + (ks + 1) * 32);
-            sa = *reinterpret_cast<const uint32_t *>(sfa_ptr + (ks + 1) * 512);
-            sb = *reinterpret_cast<const uint32_t *>(sfb_ptr + (ks + 1) * 512);
-        }
+    // body of one K step: multiply out of buffer `buf`, stage `nxt` (step ks+1) into the
+    // other buffer, refill `nxt`'s registers with step ks+2 afterwards
+    auto kstep = [&](int64_t ks, int buf, Staged &cur_regs, Staged &nxt) {
+        const bool have_next = ks + 1 < ksteps;
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
-            half8_t fa[2], fb[2];
+            half8_t fa[WM], fb[WN];
             const int kofs = kk * 16 + (lane >> 5) * 8;
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                fa[i] = *reinterpret_cast<const half8_t *>(lds_a + (wm * 64 + i * 32 + (lane & 31)) * kPitch + kofs);
+            for (int i = 0; i < WM; ++i)
+                fa[i] = *reinterpret_cast<const half8_t *>(lds_a[buf] + (wm * WM * 32 + i * 32 + (lane & 31)) * kPitch + kofs);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                fb[j] = *reinterpret_cast<const half8_t *>(lds_b + (wn * 64 + j * 32 + (lane & 31)) * kPitch + kofs);
+            for (int j = 0; j < WN; ++j)
+                fb[j] = *reinterpret_cast<const half8_t *>(lds_b[buf] + (wn * WN * 32 + j * 32 + (lane & 31)) * kPitch + kofs);
+            if (have_next) stage_quarter(nxt, buf ^ 1, kk);
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < WM; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < WN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
         }
+        if (ks + 2 < ksteps) fetch(ks + 2, cur_regs);
         __syncthreads();
+    };
+
+    for (int64_t ks = 0; ks < ksteps; ks += 2) {
+        kstep(ks, 0, st[0], st[1]);
+        if (ks + 1 < ksteps) kstep(ks + 1, 1, st[1], st[0]);
     }
 
-    // epilogue: acc[i][j][4*g + e] is D[m][n] with m = wm*64 + i*32 + (lane & 31),
-    // n = wn*64 + j*32 + 8*g + 4*(lane >> 5) + e
+    // epilogue: acc[i][j][4*g + e] is D[m][n] with m = wm*WM*32 + i*32 + (lane & 31),
+    // n = wn*WN*32 + j*32 + 8*g + 4*(lane >> 5) + e
     const float alpha = *p.alpha;
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int64_t m = m0 + wm * 64 + i * 32 + (lane & 31);
+    for (int i = 0; i < WM; ++i) {
+        const int64_t m = m0 + wm * WM * 32 + i * 32 + (lane & 31);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < WN; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn * 64 + j * 32 + 8 * g + 4 * (lane >> 5);
+                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * (lane >> 5);
                 uint16_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -166,6 +205,27 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_nvfp4_kernel(const GemmPara
     }
 }
 
+template <int WAVES_M, int WAVES_N, int WM, int WN>
+static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
+    constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+    constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
+    constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * kPitch * sizeof(_Float16);
+    p.tiles_m = (int)(p.M / BM);
+    p.tiles_n = (int)(p.N / BN);
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+    auto kbf = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, true>;
+    auto kh = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, false>;
+    if (lds_bytes > 64 * 1024) {
+        // more than the default dynamic LDS limit: opt in (idempotent, no device state besides the function attribute)
+        if (hipFuncSetAttribute((const void *)(out_type == FOS_T_BF16 ? kbf : kh), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes) != hipSuccess)
+            return FOS_E_LAUNCH;
+    }
+    if (out_type == FOS_T_BF16) hipLaunchKernelGGL(kbf, grid, dim3(kThreadsG), lds_bytes, s, p);
+    else hipLaunchKernelGGL(kh, grid, dim3(kThreadsG), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
 }  // namespace fos
 
 using namespace fos;
@@ -179,16 +239,15 @@ extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 3) || ((uintptr_t)sfB & 3) ||
         ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
         return FOS_E_BAD_ALIGNMENT;
-    if ((M / BM) * (N / BN) > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    if ((M / 128) * (N / 128) > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     GemmParams p;
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
-    p.tiles_n = (int)(N / BN);
-    dim3 grid((unsigned)((M / BM) * (N / BN)));
     hipStream_t s = (hipStream_t)stream;
-    if (out_type == FOS_T_BF16)
-        hipLaunchKernelGGL((gemm_nvfp4_kernel<true>), grid, dim3(kGemmThreads), 0, s, p);
-    else
-        hipLaunchKernelGGL((gemm_nvfp4_kernel<false>), grid, dim3(kGemmThreads), 0, s, p);
-    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+    // 256 x 256 tiles when they divide the problem and give every compute unit work;
+    // FOS_GEMM_TILE=128 forces the small tile (tuning / tests).
+    bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 128;
+    if (const char *e = getenv("FOS_GEMM_TILE")) big = big && atoi(e) != 128;
+    if (big) return launch_gemm<2, 4, 4, 2>(p, out_type, s);
+    return launch_gemm<2, 2, 2, 2>(p, out_type, s);
 }
