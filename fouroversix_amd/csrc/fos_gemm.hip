@@ -21,6 +21,7 @@
 #include <stdint.h>
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "fos_device.h"
 #include "fouroversix_hip.h"
@@ -62,6 +63,13 @@ FOS_DEVICE half8_t dequant8(uint32_t word, half2_t s) {
 constexpr int BK = 64;
 constexpr int kPitch = BK + 8;  // halfs per LDS row (144 bytes: conflict-free 128-bit accesses)
 
+// Buffer resource (V#) over [base, base + bytes): raw 32-bit offsets, no swizzle.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
 // Packed operands of one K step as a thread holds them.
 struct Staged {
     uint4 qa, qb;     // 32 codes of one A row / one B row
@@ -102,20 +110,24 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     const int64_t kbytes = p.K >> 1;     // packed bytes per row
     const int64_t sf_groups = p.K >> 6;  // 4-block groups per row
 
-    // global -> register staging: 32 codes (16 bytes) of one row of each operand
+    // global -> register staging: 32 codes (16 bytes) of one row of each operand, through
+    // buffer loads (wave-uniform base + per-thread 32-bit offset + scalar K offset), which
+    // keeps 64-bit address arithmetic out of the loop
     const int ld_row = tid >> 1, ld_half = tid & 1;
-    const uint8_t *a_ptr = p.A + (m0 + ld_row) * kbytes + ld_half * 16;
-    const uint8_t *b_ptr = p.B + (n0 + ld_row) * kbytes + ld_half * 16;
-    const int sf_in_tile = (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4;
-    const uint8_t *sfa_ptr = p.sfA + ((m0 + ld_row) >> 7) * sf_groups * 512 + sf_in_tile;
-    const uint8_t *sfb_ptr = p.sfB + ((n0 + ld_row) >> 7) * sf_groups * 512 + sf_in_tile;
+    const BufferRsrc ra = make_rsrc(p.A + m0 * kbytes, (uint32_t)(BM * kbytes));
+    const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(BN * kbytes));
+    const BufferRsrc rsa = make_rsrc(p.sfA + (m0 >> 7) * sf_groups * 512, (uint32_t)((BM >> 7) * sf_groups * 512));
+    const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)((BN >> 7) * sf_groups * 512));
+    const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_half * 16);
+    const uint32_t s_off = (uint32_t)((ld_row >> 7) * sf_groups * 512 + (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4);
     const int64_t ksteps = p.K / BK;
 
     auto fetch = [&](int64_t ks, Staged &s) {
-        s.qa = *reinterpret_cast<const uint4 *>(a_ptr + ks * 32);
-        s.qb = *reinterpret_cast<const uint4 *>(b_ptr + ks * 32);
-        s.sa = *reinterpret_cast<const uint32_t *>(sfa_ptr + ks * 512);
-        s.sb = *reinterpret_cast<const uint32_t *>(sfb_ptr + ks * 512);
+        const uint32_t kq = (uint32_t)ks * 32u, ksf = (uint32_t)ks * 512u;
+        s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
+        s.qb = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)q_off, (int)kq, 0));
+        s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
+        s.sb = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)s_off, (int)ksf, 0);
     };
     // quarter q (0..3) of the staged data -> 8 halfs of each operand in LDS buffer `buf`
     auto stage_quarter = [&](const Staged &s, int buf, int q) {
@@ -137,41 +149,75 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+    auto read_frags = [&](int buf, int kk, half8_t *fa, half8_t *fb) {
+        const int kofs = kk * 16 + (lane >> 5) * 8;
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+            fa[i] = *reinterpret_cast<const half8_t *>(lds_a[buf] + (wm * WM * 32 + i * 32 + (lane & 31)) * kPitch + kofs);
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+            fb[j] = *reinterpret_cast<const half8_t *>(lds_b[buf] + (wn * WN * 32 + j * 32 + (lane & 31)) * kPitch + kofs);
+    };
+
     Staged st[2];
+    half8_t fa[2][WM], fb[2][WN];  // MFMA fragments of the current and the next 16-wide K slice
     fetch(0, st[0]);
 #pragma unroll
     for (int q = 0; q < 4; ++q) stage_quarter(st[0], 0, q);
     if (ksteps > 1) fetch(1, st[1]);
     __syncthreads();
+    read_frags(0, 0, fa[0], fb[0]);
 
-    // body of one K step: multiply out of buffer `buf`, stage `nxt` (step ks+1) into the
-    // other buffer, refill `nxt`'s registers with step ks+2 afterwards
-    auto kstep = [&](int64_t ks, int buf, Staged &cur_regs, Staged &nxt) {
-        const bool have_next = ks + 1 < ksteps;
+    // Body of one K step: multiply out of buffer `buf` while staging `nxt` (step ks+1) into
+    // the other buffer.  Inside a 16-wide K slice the order is: issue the LDS reads of the
+    // NEXT slice, dequantise + write a quarter of the next step, then the MFMAs of the
+    // current slice, whose fragments are already in registers.  The step's barrier sits
+    // between the last quarter's writes and the last slice's MFMAs, and the first slice of
+    // the next step is read right after it, so the matrix pipe has work on both sides of
+    // the barrier and no LDS latency is exposed at the step boundary.
+    // The body is branch-free (the last step, which has nothing to stage, is a separate
+    // instantiation; the prefetch index is clamped instead of guarded): waits are then
+    // placed per register instead of conservatively at control-flow joins.
+    auto kstep = [&](auto have_next_c, int64_t ks, int buf, Staged &cur_regs, Staged &nxt) {
+        constexpr bool have_next = decltype(have_next_c)::value;
+        // `cur_regs` (step ks) went into LDS during the previous step: refill them now,
+        // two steps ahead of their use, so HBM / L2 latency has a whole K step to hide in
+        if (have_next) fetch(ks + 2 < ksteps ? ks + 2 : ksteps - 1, cur_regs);
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
-            half8_t fa[WM], fb[WN];
-            const int kofs = kk * 16 + (lane >> 5) * 8;
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-                fa[i] = *reinterpret_cast<const half8_t *>(lds_a[buf] + (wm * WM * 32 + i * 32 + (lane & 31)) * kPitch + kofs);
-#pragma unroll
-            for (int j = 0; j < WN; ++j)
-                fb[j] = *reinterpret_cast<const half8_t *>(lds_b[buf] + (wn * WN * 32 + j * 32 + (lane & 31)) * kPitch + kofs);
-            if (have_next) stage_quarter(nxt, buf ^ 1, kk);
+            if (kk + 1 < BK / 16) read_frags(buf, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+            if (have_next) {
+                stage_quarter(nxt, buf ^ 1, kk);
+                if (kk + 1 == BK / 16) {
+                    __syncthreads();
+                    read_frags(buf ^ 1, 0, fa[0], fb[0]);
+                    // keep this slice's MFMAs below the barrier (the scheduler would
+                    // otherwise hoist them and leave the matrix pipe idle behind it)
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < WM; ++i)
 #pragma unroll
                 for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+            // slices are scheduled one at a time: a wider window only raises register pressure
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (ks + 2 < ksteps) fetch(ks + 2, cur_regs);
-        __syncthreads();
     };
 
-    for (int64_t ks = 0; ks < ksteps; ks += 2) {
-        kstep(ks, 0, st[0], st[1]);
-        if (ks + 1 < ksteps) kstep(ks + 1, 1, st[1], st[0]);
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+    int64_t ks = 0;
+    for (; ks + 2 < ksteps; ks += 2) {
+        kstep(yes{}, ks, 0, st[0], st[1]);
+        kstep(yes{}, ks + 1, 1, st[1], st[0]);
+    }
+    if (ks + 2 == ksteps) {
+        kstep(yes{}, ks, 0, st[0], st[1]);
+        kstep(no{}, ks + 1, 1, st[1], st[0]);
+    } else {
+        kstep(no{}, ks, 0, st[0], st[1]);
     }
 
     // epilogue: acc[i][j][4*g + e] is D[m][n] with m = wm*WM*32 + i*32 + (lane & 31),
