@@ -103,8 +103,8 @@ FOS_DEVICE float candidate_residual(float fq, const FastLutEntry &e, float x) {
 //     |E_k - h_k^2 S~_k| <= h_k^2 * u * (330 sqrt(S_k) + 40 S_k)        (16 elements)
 // (5 roundings from amax to x*inv: 33u absolute on the scaled value; 7u on the reference's
 // residual; 16u relative on either sum; 256-element tiles multiply the two coefficients by
-// 4 and 16).  The kernel uses 2^-14 (sqrt(n/16) sqrt(S) + (n/16) S), three times that, as
-// the tolerance: when the two intervals do not overlap the comparison E_4 < E_6 is
+// 4 and 16).  The kernel uses 2^-14 (sqrt(n/16) (1 + S) / 2 + (n/16) S) >= three times that
+// (sqrt(S) <= (1 + S) / 2) as the tolerance: when the two intervals do not overlap the comparison E_4 < E_6 is
 // decided by the shortcut, otherwise (a few blocks in 10^4 on real data; every block of a
 // tensor whose candidates tie exactly) the exact evaluation runs.
 
@@ -321,11 +321,13 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
                     SA = row16_sum_lane0(SA);
                     SB = row16_sum_lane0(SB);
                 }
-                constexpr float c_sqrt = TWO_D ? 4.0f : 1.0f, c_lin = TWO_D ? 16.0f : 1.0f;
+                // tolerance 2^-14 (c1 sqrt(S) + c2 S) with sqrt(S) <= (1 + S) / 2
+                constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
+                constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
                 const float hA = A.d1 * A.d1, hB = B.d1 * B.d1;
                 const float EA = hA * SA, EB = hB * SB;
-                const float tA = hA * (0x1p-14f * (c_sqrt * __builtin_sqrtf(SA) + c_lin * SA));
-                const float tB = hB * (0x1p-14f * (c_sqrt * __builtin_sqrtf(SB) + c_lin * SB));
+                const float tA = hA * __builtin_fmaf(k1, SA, k0);
+                const float tB = hB * __builtin_fmaf(k1, SB, k0);
                 const bool surely_b = EB + tB < EA - tA;
                 const bool surely_a = EB - tB > EA + tA;
                 certain = surely_a || surely_b;

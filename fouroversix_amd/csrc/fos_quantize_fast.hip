@@ -103,12 +103,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
 
 // 1x16 blocks, row-contiguous mapping: lane -> block column (lane & 15) of row (lane >> 4)
-// within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns.
-template <int RULE>
+// within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns; workgroups stride
+// over the tiles so that the per-workgroup setup (tensor maximum, scale table) is paid
+// once for several tiles.  FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
+template <int RULE, bool FULL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
-    __shared__ uint32_t sf_stage[4 * 128];  // 4 scale tiles of 512 bytes
+    __shared__ uint32_t sf_stage[2][4 * 128];  // 4 scale tiles of 512 bytes, double-buffered
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
     uint32_t amax_bits;
@@ -128,53 +130,59 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t tile_y = blockIdx.x / (uint32_t)p.tiles_x, tile_x = blockIdx.x - tile_y * (uint32_t)p.tiles_x;
     const int64_t sf_cols = p.cols_p >> 4;
-    const int lb = lane & 15;                      // block column inside the tile
-    const int64_t cb = (int64_t)tile_x * 16 + lb;  // block column in the tensor
-    const int rr0 = wave * 4 + (lane >> 4);        // row inside a 16-row step
-    const bool col_ok = cb < sf_cols;
+    const int lb = lane & 15;                // block column inside the tile
+    const int rr0 = wave * 4 + (lane >> 4);  // row inside a 16-row step
     const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
-    const uint16_t *src0 = p.x + ((int64_t)tile_y * 128 + rr0) * p.ld + cb * 16;
-    uint8_t *dst0 = p.codes + ((int64_t)tile_y * 128 + rr0) * (p.cols_p >> 1) + cb * 8;
+    const int64_t row_pitch = p.ld, code_pitch = p.cols_p >> 1;
+    const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
+    int buf = 0;
 
-    auto load = [&](int g, Block16 &b) {
-        const int64_t r = (int64_t)tile_y * 128 + g * 16 + rr0;
-        if (col_ok && r < p.rows && cb * 16 < p.cols) {
-            const uint4 *src = reinterpret_cast<const uint4 *>(src0 + (int64_t)g * 16 * p.ld);
-            const uint4 lo = src[0], hi = src[1];
-            b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
-            b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) b.w[i] = 0;
-        }
-    };
+    for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
+        const uint32_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - tile_y * (uint32_t)p.tiles_x;
+        const int64_t cb = (int64_t)tile_x * 16 + lb;  // block column in the tensor
+        const bool col_ok = FULL || cb < sf_cols;
+        const int64_t row0 = (int64_t)tile_y * 128 + rr0;
+        const uint16_t *src = p.x + row0 * row_pitch + cb * 16;
+        uint8_t *dst = p.codes + row0 * code_pitch + cb * 8;
+        uint8_t *stage = reinterpret_cast<uint8_t *>(sf_stage[buf]) + (lb >> 2) * 512 + (lb & 3);
 
-    Block16 cur, nxt;
-    load(0, cur);
+        auto load = [&](int g, Block16 &b) {
+            if (FULL || (col_ok && row0 + g * 16 < p.rows && cb * 16 < p.cols)) {
+                const uint4 *q = reinterpret_cast<const uint4 *>(src + (int64_t)g * 16 * row_pitch);
+                const uint4 lo = q[0], hi = q[1];
+                b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
+                b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
+            } else {
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-        if (g + 1 < 8) load(g + 1, nxt);
-        if (col_ok) {
-            const int rr = g * 16 + rr0;
-            const BlockOut o = quantize_block_nvfp4_rtn<RULE, false>(cur, k, enc_fast, rq, maybe_negzero, in_range, lut);
-            *reinterpret_cast<uint2 *>(dst0 + (int64_t)g * 16 * (p.cols_p >> 1)) = make_uint2(o.c0, o.c1);
-            if (tiled)
-                reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)o.s;
-            else
-                p.sf[((int64_t)tile_y * 128 + rr) * sf_cols + cb] = (uint8_t)o.s;
+                for (int i = 0; i < 8; ++i) b.w[i] = 0;
+            }
+        };
+
+        Block16 blk[8];
+        load(0, blk[0]);
+        load(1, blk[1]);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g + 2 < 8) load(g + 2, blk[g + 2]);
+            if (col_ok) {
+                const int rr = g * 16 + rr0;
+                const BlockOut o = quantize_block_nvfp4_rtn<RULE, false>(blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut);
+                *reinterpret_cast<uint2 *>(dst + (int64_t)g * 16 * code_pitch) = make_uint2(o.c0, o.c1);
+                if (tiled) stage[(rr & 31) * 16 + (rr >> 5) * 4] = (uint8_t)o.s;
+                else p.sf[(row0 + g * 16) * sf_cols + cb] = (uint8_t)o.s;
+            }
         }
-        cur = nxt;
-    }
-    if (tiled) {
-        __syncthreads();
-        // 4 scale tiles x 512 bytes, contiguous in the output; 8 bytes per thread
-        const int t = threadIdx.x >> 6;
-        const int64_t group = (int64_t)tile_x * 4 + t;
-        if (group < (sf_cols >> 2)) {
-            uint2 *dst = reinterpret_cast<uint2 *>(p.sf + ((int64_t)tile_y * (sf_cols >> 2) + group) * 512);
-            dst[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
+        if (tiled) {
+            __syncthreads();
+            // 4 scale tiles x 512 bytes, contiguous in the output; 8 bytes per thread.  The
+            // other staging buffer is in use by the next tile, so one barrier per tile does.
+            const int t = threadIdx.x >> 6;
+            const int64_t group = (int64_t)tile_x * 4 + t;
+            if (FULL || group < (sf_cols >> 2)) {
+                uint2 *out = reinterpret_cast<uint2 *>(p.sf + ((int64_t)tile_y * (sf_cols >> 2) + group) * 512);
+                out[lane] = reinterpret_cast<const uint2 *>(sf_stage[buf])[threadIdx.x];
+            }
         }
     }
 }
@@ -189,7 +197,16 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     if (!two_d) {
         p.tiles_x = (int)((p.cols_p + 255) / 256);
         const int64_t n = (p.rows_p / 128) * p.tiles_x;
-        hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE>), dim3((unsigned)n), dim3(kThreads), 0, s, p);
+        // five resident workgroups per compute unit (256 CUs, <= 102 VGPRs); more tiles than
+        // that are walked by the same workgroups.  FOS_QUANT_GRID overrides for tuning runs.
+        int64_t grid = 1280;
+        if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
+        if (grid > n) grid = n;
+        const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
+        if (full)
+            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else
+            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, false>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         return;
     }
     p.tiles_x = (int)(p.cols_p / 64);
