@@ -55,6 +55,60 @@ def event_ms(fn, steps):
     return start.elapsed_time(stop) / steps
 
 
+def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv=1024, ffn=14336):
+    """Per layer: on-the-fly activation quantize (4/6-MSE, 1x16) + FP4 GEMM for q/k/v/o and
+    gate/up/down against weights pre-quantized 4/6-MSE with 16x16 blocks; each projection
+    re-quantizes its input, as the reference's linear layer does.  No attention, no
+    nonlinearity: the output of q feeds o, the output of gate feeds down."""
+    import torch
+
+    import fouroversix_amd as fos
+
+    wcfg = fos.QuantizationConfig(scale_rule="mse", block_scale_2d=True)
+    acfg = fos.QuantizationConfig(scale_rule="mse")
+    shapes = [("q", hidden, hidden), ("k", kv, hidden), ("v", kv, hidden), ("o", hidden, hidden),
+              ("gate", ffn, hidden), ("up", ffn, hidden), ("down", hidden, ffn)]
+    g = torch.Generator(device=dev).manual_seed(7)
+    weights = []
+    for _ in range(layers):
+        layer = {}
+        for name, n, k in shapes:
+            w = (0.02 * torch.randn(n, k, generator=g, device=dev)).bfloat16()
+            layer[name] = fos.quantize(w, wcfg)
+            del w
+        weights.append(layer)
+    x0 = torch.randn(tokens, hidden, generator=g, device=dev).bfloat16()
+
+    def step():
+        x = x0
+        for layer in weights:
+            q = fos.quantized_matmul(x, layer["q"], input_config=acfg)
+            fos.quantized_matmul(x, layer["k"], input_config=acfg)
+            fos.quantized_matmul(x, layer["v"], input_config=acfg)
+            h = fos.quantized_matmul(q, layer["o"], input_config=acfg)
+            gate = fos.quantized_matmul(h, layer["gate"], input_config=acfg)
+            fos.quantized_matmul(h, layer["up"], input_config=acfg)
+            x = fos.quantized_matmul(gate, layer["down"], input_config=acfg)
+        return x
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / steps
+    flops = 2.0 * tokens * sum(n * k for _, n, k in shapes) * layers
+    return {
+        "workload": f"{layers} layers x (q,k,v,o,gate,up,down) quantize+GEMM, {tokens} tokens, hidden {hidden}, "
+                    f"kv {kv}, ffn {ffn}",
+        "ms_per_step": round(sec * 1e3, 3),
+        "tokens_per_s": round(tokens / sec, 1),
+        "TFLOP/s": round(flops / sec / 1e12, 1),
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -64,6 +118,7 @@ def main() -> int:
     ap.add_argument("--cols", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-gemm", action="store_true")
+    ap.add_argument("--no-stack", action="store_true", help="skip the 32-layer quantized-linear stack")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -87,6 +142,10 @@ def main() -> int:
     # ---- quantize: whole step through the public API -------------------------------
     n_buf = 4
     xs = [make_activation(rows, cols, 100 + i).to(dev) for i in range(n_buf)]
+    # counter calibration for profiling runs: a plain elementwise kernel of known size
+    # (reads and writes rows*cols*2 bytes) appears once in every rocprofv3 trace of this script
+    calib = xs[0].view(torch.int16) + 1
+    del calib
     cfg = fos.QuantizationConfig(scale_rule="mse")
     for i in range(W):
         fos.quantize(xs[i % n_buf], cfg)
@@ -186,6 +245,11 @@ def main() -> int:
                          "unit": "TFLOP/s", "frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None},
         }
 
+    # ---- 32-layer quantized-linear stack (Llama-3-8B projection shapes, 8 x 2048 tokens) --
+    stack = None
+    if not args.no_stack and not args.no_gemm:
+        stack = linear_stack(dev, steps=3, warmup=1)
+
     # ---- CPU baseline: the C oracle on the host cores, bounded sample -----------------
     cpu = None
     if not args.no_cpu:
@@ -233,6 +297,7 @@ def main() -> int:
         "roofline": roofline,
         "cpu_baseline": cpu,
         "gemm": gemm,
+        "linear_stack": stack,
     }
     print(json.dumps(line))
     return 0

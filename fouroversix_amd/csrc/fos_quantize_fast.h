@@ -175,6 +175,24 @@ FOS_DEVICE float e2m1_value(uint32_t code) {
     return (code & 8u) ? -v : v;
 }
 
+// True when the two candidates of a block dequantise to identical values, element by
+// element, so that the reference's two error sums are bit-equal and "6" wins the tie.
+// With s4 = 1.5 * s6 exactly, fq6 * s6 == fq4 * s4 iff (fq6, fq4) is (0, 0), (1.5, 1),
+// (3, 2) or (6, 4) with equal signs: in codes, both magnitudes 0, or code4 in {2, 4, 6} and
+// code6 = code4 | 1.  That is the typical block with one dominant element: the outlier is
+// exact under both scales and everything else rounds to zero.  Nibble-parallel on a word
+// of 8 codes; `a` holds the "6" codes, `b` the "4" codes.
+FOS_DEVICE uint32_t tie_violations(uint32_t a, uint32_t b) {
+    const uint32_t d = a ^ b;
+    const uint32_t u = (a | b) & 0x77777777u;
+    const uint32_t nz = (u | (u >> 1) | (u >> 2)) & 0x11111111u;          // a magnitude is non-zero
+    const uint32_t nzb = ((b >> 1) | (b >> 2)) & 0x11111111u;             // code4 in {2..7}
+    return ((d & 0x77777777u) ^ nz)   // magnitudes differ exactly in bit 0 where non-zero, nowhere else
+           | (d & (nz << 3))          // equal signs where non-zero
+           | (~a & nz)                // the set bit 0 belongs to code6
+           | (nzb ^ nz);              // code4 is not 0 or 1 where non-zero
+}
+
 // Exact selection of a block whose shortcut was inconclusive: the residuals of both
 // candidates from their packed codes, with the reference's rounding and order.
 template <int RULE, bool TWO_D>
@@ -280,8 +298,13 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
         const float s_hp4 = s_hp6 * 1.5f;
         const uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp6, s_hp4, 0, false);
         const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
-        if (s6 >= 8u) {
-            const FastLutEntry A = lut[s6];
+        // The hardware convert saturates at 6 where the reference's unclamped rounding gives
+        // 8 for a scaled magnitude in [7, 9): that needs a sub-normal scale byte that was
+        // rounded down by more than 7/6 (only candidate "6" can get there).  A zero scale
+        // byte of a non-zero block has no scaled domain at all.  Everything else -- normal
+        // and sub-normal scales alike -- is exact on the fast path.
+        const FastLutEntry A = lut[s6];
+        if (s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f)) {
             if (STATIC) {
                 uint32_t c0 = 0, c1 = 0;
                 static_for<0, 4>([&](auto jc) {
@@ -333,7 +356,15 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
                 certain = surely_a || surely_b;
                 pickB = surely_b;
             }
-            if (!certain) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+            if (!certain) {
+                // exact ties by construction first (cheap), the full evaluation otherwise
+                bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
+                if (TWO_D) {
+                    // every row of the tile must agree
+                    tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
+                }
+                pickB = tie ? false : exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+            }
             return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
         }
         if (bmax == 0.0f) return BlockOut{0, 0, 0};  // an all-zero block: zero codes, zero scale

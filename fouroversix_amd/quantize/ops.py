@@ -37,6 +37,41 @@ def _padded(rows: int, cols: int) -> tuple[int, int]:
     return -(-rows // 128) * 128, -(-cols // 64) * 64
 
 
+# Pass-1 workspace (8 KiB), one per (device, stream): calls on one stream are ordered, so
+# they can share it; calls on different streams must not.
+_WORKSPACES: dict[tuple[int, int], torch.Tensor] = {}
+_WS_BYTES = 0
+
+
+def _workspace(dev: torch.device, stream: int) -> torch.Tensor:
+    global _WS_BYTES
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream)
+    ws = _WORKSPACES.get(key)
+    if ws is None:
+        if _WS_BYTES == 0:
+            _WS_BYTES = int(nat.lib().fos_quantize_workspace_bytes(1, 1))
+        ws = torch.empty(_WS_BYTES, dtype=torch.uint8, device=dev)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+class _on_device:
+    """`with torch.cuda.device(dev)` only when `dev` is not already current."""
+
+    def __init__(self, dev: torch.device) -> None:
+        self.ctx = None
+        if dev.index is not None and dev.index != torch.cuda.current_device():
+            self.ctx = torch.cuda.device(dev)
+
+    def __enter__(self) -> None:
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc) -> None:
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
 def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
     if x.dim() != 2:
         raise RuntimeError("quantize: x must be 2-D")
@@ -55,20 +90,20 @@ def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, s
         sf.view(torch.uint8).zero_()
         return values, sf, torch.zeros(1, dtype=torch.float32, device=dev)
     L = nat.lib()
-    ws_bytes = L.fos_quantize_workspace_bytes(rows, cols)
-    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     amax_is_input = amax is not None
     amax_buf = (
         amax.reshape(1).to(device=dev, dtype=torch.float32).contiguous()
         if amax_is_input
         else torch.empty(1, dtype=torch.float32, device=dev)
     )
-    with torch.cuda.device(dev):
+    with _on_device(dev):
+        stream = nat.current_stream(dev)
+        workspace = _workspace(dev, stream)
         rc = L.fos_quantize(
             x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), dtype, selection_rule, round_style, int(is_2d),
             seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, sf_layout,
             values.data_ptr(), sf.data_ptr(), amax_buf.data_ptr(), int(amax_is_input),
-            workspace.data_ptr(), ws_bytes, nat.current_stream(dev),
+            workspace.data_ptr(), workspace.numel(), stream,
         )
     nat.check(rc, "fouroversix::quantize")
     return values, sf, amax_buf
@@ -109,7 +144,7 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
     if b_sf.numel() * 16 != n * kb:
         raise RuntimeError("B_sf size mismatch")
     out = torch.empty(m, n, dtype=out_dtype, device=a.device)
-    with torch.cuda.device(a.device):
+    with _on_device(a.device):
         rc = nat.lib().fos_gemm_nvfp4(
             a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(),
             m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n, nat.current_stream(a.device),
@@ -125,7 +160,7 @@ def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, row
     if rows == 0 or cols == 0:
         return out
     amax32 = amax.reshape(1).to(device=values.device, dtype=torch.float32)
-    with torch.cuda.device(values.device):
+    with _on_device(values.device):
         rc = nat.lib().fos_dequantize(
             values.contiguous().data_ptr(), scale_factors.contiguous().data_ptr(), amax32.data_ptr(),
             dtype, sf_layout, divisor, rows, cols, rows_p, cols_p,
@@ -192,16 +227,29 @@ def quantize(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, r
 
 
 def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax=None):
+    """Extended quantize.  Real tensors go straight to the implementation (the dispatcher
+    costs more host time than a small quantize takes on the GPU); fake / meta tensors and
+    tracing go through the registered operator."""
+    if type(x) is torch.Tensor and x.device.type == "cuda" and not torch.compiler.is_compiling():
+        return _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax)
     return torch.ops.fouroversix.quantize_ex.default(
         x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax
     )
 
 
+def _direct(t: torch.Tensor) -> bool:
+    return type(t) is torch.Tensor and t.device.type == "cuda" and not torch.compiler.is_compiling()
+
+
 def gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha):
+    if _direct(a):
+        return _gemm_impl(a, b, a_sf, b_sf, alpha, torch.bfloat16)
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
 def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
+    if _direct(a):
+        return _gemm_impl(a, b, a_sf, b_sf, alpha, torch.float16)
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
