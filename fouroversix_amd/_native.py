@@ -29,6 +29,7 @@ EXPORTS = (
     "fos_amax",
     "fos_quantize",
     "fos_gemm_nvfp4",
+    "fos_gemm_workspace_bytes",
     "fos_dequantize",
 )
 
@@ -67,8 +68,10 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, i32,
                                vp, vp, vp, i32, vp, sz, vp]
     L.fos_quantize.restype = i32
-    L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp]
+    L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
+    L.fos_gemm_workspace_bytes.argtypes = [i64, i64, i64]
+    L.fos_gemm_workspace_bytes.restype = ctypes.c_size_t
     L.fos_dequantize.argtypes = [vp, vp, vp, i32, i32, dbl, i64, i64, i64, i64, vp, i32, i64, vp]
     L.fos_dequantize.restype = i32
     _lib = L

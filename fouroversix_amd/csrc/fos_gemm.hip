@@ -39,6 +39,10 @@ struct GemmParams {
     void *D;
     int64_t M, N, K, ldd;
     int tiles_m, tiles_n;
+    // split-K: workgroup (tile, blockIdx.y) contracts K steps [y * ksteps_per_split, ...) and
+    // writes its FP32 partial tile to partials[y][M][N]; splits == 1 writes D directly
+    float *partials;
+    int splits, ksteps_per_split;
 };
 
 // The two E4M3 bytes in the low 16 bits of `w` -> fp16 pair {s0, s1} (one hardware
@@ -91,8 +95,11 @@ FOS_DEVICE void tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
 // is fed from the B matrix (rows n) and the "B" operand from the A matrix (rows m), so
 // that a lane's four consecutive accumulator registers are four consecutive n of one
 // output row and can be stored as 8 bytes.
-template <int WAVES_M, int WAVES_N, int WM, int WN, bool OUT_BF16>
+enum { kOutF16 = 0, kOutBF16 = 1, kOutPartial = 2 };
+
+template <int WAVES_M, int WAVES_N, int WM, int WN, int OUT>
 __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const GemmParams p) {
+    constexpr bool OUT_BF16 = OUT == kOutBF16;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
     static_assert(BM == kThreadsG / 2 && BN == kThreadsG / 2, "one thread per half row of each operand");
@@ -117,10 +124,14 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)((BN >> 7) * sf_groups * 512));
     const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_half * 16);
     const uint32_t s_off = (uint32_t)((ld_row >> 7) * sf_groups * 512 + (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4);
-    const int64_t ksteps = p.K / BK;
+    // this workgroup's share of the K steps (all of them unless the launch splits K)
+    const int64_t ks0 = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
+    const int64_t ksteps_all = p.K / BK;
+    const int64_t ksteps =
+        OUT == kOutPartial ? (ksteps_all - ks0 < p.ksteps_per_split ? ksteps_all - ks0 : p.ksteps_per_split) : ksteps_all;
 
     auto fetch = [&](int64_t ks, Staged &s) {
-        const uint32_t kq = (uint32_t)ks * 32u, ksf = (uint32_t)ks * 512u;
+        const uint32_t kq = (uint32_t)(ks0 + ks) * 32u, ksf = (uint32_t)(ks0 + ks) * 512u;
         s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
         s.qb = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)q_off, (int)kq, 0));
         s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
@@ -222,6 +233,22 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 
     // epilogue: acc[i][j][4*g + e] is D[m][n] with m = wm*WM*32 + i*32 + (lane & 31),
     // n = wn*WN*32 + j*32 + 8*g + 4*(lane >> 5) + e
+    if (OUT == kOutPartial) {
+        float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < WM; ++i) {
+            const int64_t m = m0 + wm * WM * 32 + i * 32 + (lane & 31);
+#pragma unroll
+            for (int j = 0; j < WN; ++j)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * (lane >> 5);
+                    *reinterpret_cast<float4 *>(P + m * p.N + n) =
+                        make_float4(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]);
+                }
+        }
+        return;
+    }
     const float alpha = *p.alpha;
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
@@ -251,6 +278,255 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// M <= 128 ("skinny": decode-sized batches, one 128-row band of A).  The weight matrix B is
+// streamed once from HBM; a workgroup owns 32 * WN rows of B and the first 32 * MT rows of A,
+// and its 8 wavefronts split the K steps of 256 between them (wave w takes steps w, w + 8,
+// ...), so no data is shared between wavefronts and the main loop has no barrier.
+//
+// Per step a lane (r = lane & 31, h = lane >> 5) multiplies the 128 codes
+// k = 256 step + 128 h ... of B row n0 + 32 t + r with the same codes of A rows r + 32 i.
+// The MFMA contraction index is thereby permuted (slice x pairs codes 8x..8x+7 of both
+// lane halves); A and B use the same permutation, so the sum is unchanged.
+//  * B codes come straight from global memory (64 contiguous bytes per lane).
+//  * A codes are re-read by every workgroup, so their path through the vector cache
+//    matters: a wavefront loads its A step with 8 lanes per 128-byte row segment (whole
+//    cache lines) and transposes it through a private LDS region into the per-row
+//    fragment order (LDS operations of one wavefront execute in order: no barrier).
+//  * Scales: the 128x4 tiled layout puts the four blocks of a 64-wide K group of rows r,
+//    r + 32, r + 64, r + 96 next to each other, so one 128-bit load per group fetches the
+//    scales of all A rows of a lane; B takes one 32-bit word per group.
+// The 8 partial accumulators are tree-reduced through LDS at the end (fixed order).
+constexpr int kSkinnyPitch = 144;  // LDS bytes per A row (128 + 16: conflict-free 128-bit accesses)
+
+template <int MT, int WN>
+struct SkinnyRegs {
+    uint4 b[WN][4];     // 128 codes of each B row
+    uint32_t sb[WN][2]; // their 8 block scales (two groups)
+    uint4 sa[2];        // block scales of the A rows: [group] word i = row r + 32 i
+};
+
+template <int MT, int WN, int OUT>
+__global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
+    constexpr int kWaves = 8, kAcc = MT * WN * 16;
+    constexpr int kRegion = MT * 32 * kSkinnyPitch;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    // the wave index steers loops and scalar buffer offsets: make its uniformity known
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 31, h = lane >> 5;
+    uint8_t *region = smem + wave * kRegion;
+    const int64_t n0 = (int64_t)blockIdx.x * (32 * WN);
+    const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
+    const int64_t steps_all = p.K >> 8;
+    const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
+    const int64_t s_end = OUT == kOutPartial ? (s_begin + p.ksteps_per_split < steps_all ? s_begin + p.ksteps_per_split : steps_all)
+                                             : steps_all;
+
+    // rows of A past M read as zero codes (buffer range check), so A needs only M rows
+    const BufferRsrc ra = make_rsrc(p.A, (uint32_t)(p.M * kbytes));
+    const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(32 * WN * kbytes));
+    const BufferRsrc rsa = make_rsrc(p.sfA, (uint32_t)(sf_groups * 512));
+    const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
+    const uint32_t a_off = (uint32_t)((lane >> 3) * kbytes + (lane & 7) * 16);  // row 8 j + lane / 8, 16-byte column lane % 8
+    const uint32_t b_off = (uint32_t)(r * kbytes + h * 64);
+    const uint32_t sa_off = (uint32_t)(h * 1024 + r * 16);
+    const uint32_t sb_off = (uint32_t)(h * 1024 + r * 16 + (((uint32_t)n0 & 127u) >> 5) * 4);
+    const uint32_t lds_w = (uint32_t)((lane >> 3) * kSkinnyPitch + (lane & 7) * 16);
+    const uint32_t lds_r = (uint32_t)(r * kSkinnyPitch + h * 64);
+
+    uint4 a_stage[MT * 4];  // one A step in flight from global memory
+    auto fetch_a = [&](int64_t step) {
+#pragma unroll
+        for (int j = 0; j < MT * 4; ++j)
+            a_stage[j] = __builtin_bit_cast(
+                uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)(a_off + j * 8 * kbytes), (int)(step * 128), 0));
+    };
+    auto fetch_b = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
+        const int kq = (int)(step * 128), ksf = (int)(step * 2048);
+#pragma unroll
+        for (int t = 0; t < WN; ++t) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                s.b[t][q] = __builtin_bit_cast(
+                    uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
+#pragma unroll
+            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)(sb_off + t * 4 + u * 512), ksf, 0);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            s.sa[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsa, (int)(sa_off + u * 512), ksf, 0));
+    };
+
+    float16_t acc[MT][WN];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int t = 0; t < WN; ++t)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][t][e] = 0.0f;
+
+    auto word_of = [](const uint4 &v, int j) -> uint32_t { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; };
+    // scale of code word x (0..15) of a lane: block x >> 1 = byte (x >> 1) & 3 of group word x >> 3
+    auto scale_of = [](uint32_t w, int x) -> half2_t {
+        const half2_t s2 = e4m3x2_to_half2((x & 4) ? w >> 16 : w);
+        return ((x >> 1) & 1) ? __builtin_shufflevector(s2, s2, 1, 1) : __builtin_shufflevector(s2, s2, 0, 0);
+    };
+    auto read_frags = [&](int q, uint4 *fr) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) fr[i] = *reinterpret_cast<const uint4 *>(region + lds_r + i * 32 * kSkinnyPitch + q * 16);
+    };
+    // one step: A codes staged in `a_stage` go through LDS, the next step's A load is issued,
+    // then 16 K slices are multiplied
+    auto compute = [&](const SkinnyRegs<MT, WN> &s, int64_t next_step) {
+#pragma unroll
+        for (int j = 0; j < MT * 4; ++j) *reinterpret_cast<uint4 *>(region + lds_w + j * 8 * kSkinnyPitch) = a_stage[j];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        uint4 fr[2][MT];
+        read_frags(0, fr[0]);
+        if (next_step < s_end) fetch_a(next_step);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (q + 1 < 4) read_frags(q + 1, fr[(q + 1) & 1]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int x = q * 4 + j;
+                half8_t fb[WN], fa[MT];
+#pragma unroll
+                for (int t = 0; t < WN; ++t) fb[t] = dequant8(word_of(s.b[t][q], j), scale_of(s.sb[t][x >> 3], x));
+#pragma unroll
+                for (int i = 0; i < MT; ++i) fa[i] = dequant8(word_of(fr[q & 1][i], j), scale_of(word_of(s.sa[x >> 3], i), x));
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+#pragma unroll
+                    for (int t = 0; t < WN; ++t)
+                        acc[i][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[t], fa[i], acc[i][t], 0, 0, 0);
+            }
+        }
+        // the next step's LDS writes must not pass this step's reads
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    SkinnyRegs<MT, WN> st[2];
+    int64_t step = s_begin + wave;
+    if (step < s_end) {
+        fetch_a(step);
+        fetch_b(step, st[0]);
+    }
+    if (step + kWaves < s_end) fetch_b(step + kWaves, st[1]);
+    for (; step < s_end; step += 2 * kWaves) {
+        compute(st[0], step + kWaves);
+        if (step + 2 * kWaves < s_end) fetch_b(step + 2 * kWaves, st[0]);
+        if (step + kWaves < s_end) {
+            compute(st[1], step + 2 * kWaves);
+            if (step + 3 * kWaves < s_end) fetch_b(step + 3 * kWaves, st[1]);
+        }
+    }
+
+    // tree reduction of the 8 wavefronts' accumulators: waves [stride, 2 stride) hand theirs
+    // to waves [0, stride) through LDS slot (wave - stride); fixed order, hence deterministic.
+    // The slots overlay the staging regions, so every wavefront must have left the main loop.
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(smem);
+#pragma unroll
+    for (int stride = kWaves / 2; stride >= 1; stride >>= 1) {
+        if (wave >= stride && wave < 2 * stride) {
+            float *slot = red + (wave - stride) * (kAcc * 64);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int t = 0; t < WN; ++t)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) slot[((i * WN + t) * 16 + e) * 64 + lane] = acc[i][t][e];
+        }
+        __syncthreads();
+        if (wave < stride) {
+            const float *slot = red + wave * (kAcc * 64);
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int t = 0; t < WN; ++t)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[i][t][e] += slot[((i * WN + t) * 16 + e) * 64 + lane];
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+
+    // acc[i][t][4 g + e] is D[m][n], m = 32 i + r, n = n0 + 32 t + 8 g + 4 h + e; rows m >= M
+    // are padding of the band and are not written
+    if (OUT == kOutPartial) {
+        float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            if (32 * i + r >= p.M) continue;
+#pragma unroll
+            for (int t = 0; t < WN; ++t)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    *reinterpret_cast<float4 *>(P + (int64_t)(32 * i + r) * p.N + n0 + 32 * t + 8 * g + 4 * h) =
+                        make_float4(acc[i][t][4 * g], acc[i][t][4 * g + 1], acc[i][t][4 * g + 2], acc[i][t][4 * g + 3]);
+        }
+        return;
+    }
+    const float alpha = *p.alpha;
+    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        if (32 * i + r >= p.M) continue;
+#pragma unroll
+        for (int t = 0; t < WN; ++t)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint16_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = alpha * acc[i][t][4 * g + e];
+                    if (OUT == kOutBF16) {
+                        uint32_t u = f2u(v);
+                        u += 0x7fffu + ((u >> 16) & 1u);
+                        o[e] = (uint16_t)(u >> 16);
+                    } else {
+                        o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
+                    }
+                }
+                *reinterpret_cast<uint2 *>(D + (int64_t)(32 * i + r) * p.ldd + n0 + 32 * t + 8 * g + 4 * h) =
+                    make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+            }
+    }
+}
+
+// D = alpha * (sum of the split-K partial tiles, in split order), 4 consecutive n per thread.
+template <bool OUT_BF16>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
+    const int64_t quads = p.M * (p.N >> 2);
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= quads) return;
+    const int64_t m = t / (p.N >> 2), n = (t - m * (p.N >> 2)) << 2;
+    const float4 *P = reinterpret_cast<const float4 *>(p.partials + m * p.N + n);
+    const int64_t stride = (p.M * p.N) >> 2;
+    float4 s = P[0];
+    for (int y = 1; y < p.splits; ++y) {
+        const float4 v = P[y * stride];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const float alpha = *p.alpha;
+    const float v[4] = {alpha * s.x, alpha * s.y, alpha * s.z, alpha * s.w};
+    uint16_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (OUT_BF16) {
+            uint32_t u = f2u(v[e]);
+            u += 0x7fffu + ((u >> 16) & 1u);
+            o[e] = (uint16_t)(u >> 16);
+        } else {
+            o[e] = __builtin_bit_cast(uint16_t, (_Float16)v[e]);
+        }
+    }
+    *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.D) + m * p.ldd + n) =
+        make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+}
+
 template <int WAVES_M, int WAVES_N, int WM, int WN>
 static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
@@ -258,42 +534,136 @@ static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
     constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * kPitch * sizeof(_Float16);
     p.tiles_m = (int)(p.M / BM);
     p.tiles_n = (int)(p.N / BN);
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
-    auto kbf = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, true>;
-    auto kh = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, false>;
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.splits);
+    auto kbf = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutBF16>;
+    auto kh = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutF16>;
+    auto kp = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutPartial>;
+    auto kernel = p.splits > 1 ? kp : out_type == FOS_T_BF16 ? kbf : kh;
     if (lds_bytes > 64 * 1024) {
         // more than the default dynamic LDS limit: opt in (idempotent, no device state besides the function attribute)
-        if (hipFuncSetAttribute((const void *)(out_type == FOS_T_BF16 ? kbf : kh), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes) != hipSuccess)
+        if (hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
             return FOS_E_LAUNCH;
     }
-    if (out_type == FOS_T_BF16) hipLaunchKernelGGL(kbf, grid, dim3(kThreadsG), lds_bytes, s, p);
-    else hipLaunchKernelGGL(kh, grid, dim3(kThreadsG), lds_bytes, s, p);
+    hipLaunchKernelGGL(kernel, grid, dim3(kThreadsG), lds_bytes, s, p);
+    if (hipGetLastError() != hipSuccess) return FOS_E_LAUNCH;
+    if (p.splits > 1) {
+        const int64_t quads = p.M * (p.N >> 2);
+        dim3 rgrid((unsigned)((quads + 255) / 256));
+        if (out_type == FOS_T_BF16) hipLaunchKernelGGL(gemm_reduce_kernel<true>, rgrid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(gemm_reduce_kernel<false>, rgrid, dim3(256), 0, s, p);
+    }
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+template <int MT, int WN>
+static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
+    constexpr size_t stage_bytes = (size_t)8 * MT * 32 * kSkinnyPitch, red_bytes = (size_t)4 * (MT * WN * 16) * 64 * sizeof(float);
+    constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
+    dim3 grid((unsigned)(p.N / (32 * WN)), (unsigned)p.splits);
+    auto kernel = p.splits > 1 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutPartial>
+                  : out_type == FOS_T_BF16 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutBF16> : gemm_nvfp4_skinny_kernel<MT, WN, kOutF16>;
+    if (lds_bytes > 64 * 1024 &&
+        hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+        return FOS_E_LAUNCH;
+    hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
+    if (hipGetLastError() != hipSuccess) return FOS_E_LAUNCH;
+    if (p.splits > 1) {
+        const int64_t quads = p.M * (p.N >> 2);
+        dim3 rgrid((unsigned)((quads + 255) / 256));
+        if (out_type == FOS_T_BF16) hipLaunchKernelGGL(gemm_reduce_kernel<true>, rgrid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(gemm_reduce_kernel<false>, rgrid, dim3(256), 0, s, p);
+    }
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+// Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
+// caller's workspace for splits * M * N FP32 partials).
+enum { kPlanBig, kPlanSmall, kPlanSkinny };
+struct GemmPlan {
+    int kind, splits, ksteps_per_split;
+};
+constexpr int kTargetWorkgroups = 256;
+static int env_int(const char *name, int fallback) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : fallback;
+}
+static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
+    GemmPlan g;
+    const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no skinny kernel
+    int64_t steps, tiles;
+    if (M <= 128 && K % 256 == 0 && tile == 0) {
+        // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
+        g.kind = kPlanSkinny;
+        steps = K / 256;
+        tiles = N / 32;
+    } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
+        // 256 x 256 tiles once they give each of the 256 compute units a workgroup
+        g.kind = kPlanBig;
+        g.splits = 1;
+        g.ksteps_per_split = (int)(K / BK);
+        return g;
+    } else {
+        g.kind = kPlanSmall;
+        steps = K / BK;
+        tiles = ((M + 127) / 128) * (N / 128);
+    }
+    // split so that about kTargetWorkgroups workgroups run, each with a useful share of K
+    const int64_t min_steps = g.kind == kPlanSkinny ? 8 : 4;
+    int64_t want = tiles >= kTargetWorkgroups / 2 ? 1 : (kTargetWorkgroups + tiles - 1) / tiles;
+    if (want > steps / min_steps) want = steps / min_steps;
+    want = env_int("FOS_GEMM_SPLITK", (int)want);  // tuning / tests
+    if (want > steps) want = steps;
+    if (want > 32) want = 32;
+    if (want < 1) want = 1;
+    g.ksteps_per_split = (int)((steps + want - 1) / want);
+    g.splits = (int)((steps + g.ksteps_per_split - 1) / g.ksteps_per_split);
+    return g;
 }
 
 }  // namespace fos
 
 using namespace fos;
 
+extern "C" size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || (M < 128 && K % 256 != 0) || N % 128 != 0 || K % 64 != 0)
+        return 0;
+    const GemmPlan g = plan_gemm(M, N, K);
+    return g.splits > 1 ? (size_t)g.splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
 extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
                               const float *alpha, int64_t M, int64_t N, int64_t K,
-                              void *D, int out_type, int64_t ldd, fos_stream_t stream) {
+                              void *D, int out_type, int64_t ldd,
+                              void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!A || !B || !sfA || !sfB || !alpha || !D) return FOS_E_NULL_POINTER;
-    if (M <= 0 || N <= 0 || K <= 0 || M % 128 != 0 || N % 128 != 0 || K % 64 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
+    if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || N % 128 != 0 || K % 64 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
+    if (M < 128 && K % 256 != 0) return FOS_E_BAD_SHAPE;  // partial bands only through the weight-streaming kernel
     if (out_type != FOS_T_BF16 && out_type != FOS_T_F16) return FOS_E_UNSUPPORTED;
-    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 3) || ((uintptr_t)sfB & 3) ||
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 15) || ((uintptr_t)sfB & 15) ||
         ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
         return FOS_E_BAD_ALIGNMENT;
-    if ((M / 128) * (N / 128) > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 24)) return FOS_E_BAD_SHAPE;
     GemmParams p;
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
-    // 256 x 256 tiles when they divide the problem and give every compute unit work;
-    // FOS_GEMM_TILE=128 forces the small tile (tuning / tests).
-    bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 128;
-    if (const char *e = getenv("FOS_GEMM_TILE")) big = big && atoi(e) != 128;
-    if (big) return launch_gemm<2, 4, 4, 2>(p, out_type, s);
-    return launch_gemm<2, 2, 2, 2>(p, out_type, s);
+    GemmPlan g = plan_gemm(M, N, K);
+    if (M < 128 && g.kind != kPlanSkinny) return FOS_E_BAD_SHAPE;  // partial bands only through the weight-streaming kernel
+    if (g.splits > 1 && !(workspace && !((uintptr_t)workspace & 15) &&
+                          workspace_bytes >= (size_t)g.splits * (size_t)M * (size_t)N * sizeof(float))) {
+        // no (or too small a) workspace: run unsplit
+        g.splits = 1;
+        g.ksteps_per_split = (int)(K / (g.kind == kPlanSkinny ? 256 : BK));
+    }
+    p.partials = g.splits > 1 ? static_cast<float *>(workspace) : nullptr;
+    p.splits = g.splits;
+    p.ksteps_per_split = g.ksteps_per_split;
+    switch (g.kind) {
+        case kPlanBig: return launch_gemm<2, 4, 4, 2>(p, out_type, s);
+        case kPlanSkinny:
+            if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
+            if (M <= 64) return launch_skinny<2, 1>(p, out_type, s);
+            return launch_skinny<4, 1>(p, out_type, s);
+        default: return launch_gemm<2, 2, 2, 2>(p, out_type, s);
+    }
 }

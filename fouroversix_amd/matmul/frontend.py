@@ -80,7 +80,12 @@ def quantized_matmul(
         if out_dtype == DataType.bfloat16
         else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
     )
-    out = gemm(input.values, other.values, input.scale_factors, other.scale_factors, alpha)
+    a_values = input.values
+    m_orig = input.original_shape[0]
+    if m_orig < 128 and a_values.shape[0] == 128 and a_values.shape[1] % 128 == 0:
+        # small batch: hand over only the real rows, so the kernel skips the padding
+        a_values = a_values[:m_orig]
+    out = gemm(a_values, other.values, input.scale_factors, other.scale_factors, alpha)
     out_shape = (input.original_shape[0], other.original_shape[0])
     if tuple(out.shape) != out_shape:
         out = out[: out_shape[0], : out_shape[1]]

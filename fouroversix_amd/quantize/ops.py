@@ -139,15 +139,25 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
         raise RuntimeError("K-dim must be >= 16")
     if ka != kb:
         raise RuntimeError(f"Inner dims mismatch: {ka} vs {kb}")
-    if a_sf.numel() * 16 != m * ka:
+    # A may be the first m < 128 rows of a quantized tensor whose scales cover the whole
+    # padded 128-row band (small batches: the kernel then skips the padding rows)
+    if a_sf.numel() * 16 != (m if m >= 128 else 128) * ka:
         raise RuntimeError("A_sf size mismatch")
+    if m < 128 and ka % 256 != 0:
+        raise RuntimeError("A with fewer than 128 rows needs K to be a multiple of 256")
     if b_sf.numel() * 16 != n * kb:
         raise RuntimeError("B_sf size mismatch")
     out = torch.empty(m, n, dtype=out_dtype, device=a.device)
+    L = nat.lib()
+    ws_bytes = int(L.fos_gemm_workspace_bytes(m, n, ka))
     with _on_device(a.device):
-        rc = nat.lib().fos_gemm_nvfp4(
+        # split-K partial tiles of small-M shapes; from torch's caching allocator, which
+        # keeps the block tied to the current stream
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+        rc = L.fos_gemm_nvfp4(
             a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(),
-            m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n, nat.current_stream(a.device),
+            m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n,
+            ws.data_ptr() if ws is not None else None, ws_bytes, nat.current_stream(a.device),
         )
     nat.check(rc, "fouroversix::gemm_nvfp4nvfp4_accum_fp32")
     return out

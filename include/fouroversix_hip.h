@@ -102,12 +102,24 @@ int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t 
  *   A  u8 [M, K/2], B u8 [N, K/2]: packed E2M1, low nibble = even k
  *   sfA, sfB  E4M3 bytes in the FOS_SF_TILED_128X4 layout of [M, K/16] / [N, K/16]
  *   alpha f32[1] on the device
- * M and N must be multiples of 128 and K a multiple of 64 (the padded shapes that
- * fos_quantize produces).
+ * N must be a multiple of 128 and K of 64, and M a multiple of 128 (the padded shapes that
+ * fos_quantize produces).  M < 128 is also accepted when K is a multiple of 256: A then
+ * holds M rows, sfA the full 128-row band of the tiled layout, and only M rows of D are
+ * written (decode-sized batches skip the work on the padding rows).
+ *   workspace  optional (may be NULL): fos_gemm_workspace_bytes(M, N, K) bytes, 16-byte
+ *              aligned.  With it, shapes with few output tiles (small M) split the K
+ *              dimension over several workgroups and reduce FP32 partial tiles in a fixed
+ *              order (deterministic); without it they run unsplit, only slower.
  */
 int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
                    const float *alpha, int64_t M, int64_t N, int64_t K,
-                   void *D, int out_type, int64_t ldd, fos_stream_t stream);
+                   void *D, int out_type, int64_t ldd,
+                   void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/* Bytes of workspace with which fos_gemm_nvfp4 runs this shape fastest (0 = none needed).
+ * The reference's op runs CUTLASS without a workspace
+ * (src/fouroversix/csrc/fp4_gemm.cu:148-151), so this has no counterpart there. */
+size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
  * out[rows, cols] = dequantized values of a quantized tensor, cropped to (rows, cols).

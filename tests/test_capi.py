@@ -75,9 +75,12 @@ def test_argument_checks_need_no_device(native):
     assert q(codes=p + 1) == -2
     g = lambda **kw: L.fos_gemm_nvfp4(  # noqa: E731
         kw.get("A", p), p, p, p, p, kw.get("M", 128), kw.get("N", 128), kw.get("K", 64), p, kw.get("out", 0),
-        kw.get("ldd", 128), None)
+        kw.get("ldd", 128), None, 0, None)
     assert g(A=None) == -4
-    assert g(M=100) == -1
+    assert g(M=100) == -1  # fewer than 128 rows need K % 256 == 0
+    assert L.fos_gemm_workspace_bytes(100, 128, 64) == 0
+    assert L.fos_gemm_workspace_bytes(128, 1024, 4096) == 2 * 128 * 1024 * 4
+    assert L.fos_gemm_workspace_bytes(8192, 8192, 8192) == 0
     assert g(K=32) == -1
     assert g(ldd=64) == -1
     assert g(out=2) == -3

@@ -68,7 +68,8 @@ def test_gemm_fp16_output_and_mixed_rules(oracle):
     assert float((got.float() - expect.float()).abs().max() / expect.float().abs().max()) <= MAX_REL
 
 
-@pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), (16, 4096, 4096), (128, 14336, 4096), (2048, 4096, 14336)])
+@pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), (16, 4096, 4096), (128, 14336, 4096), (2048, 4096, 14336),
+                                           (128, 4096, 14336), (256, 384, 2368)])
 def test_gemm_full_size_sampled(oracle, m, n, k):
     """Headline and Llama-3-8B shapes: 192 sampled rows of each operand are multiplied by
     the oracle (fp64 accumulation) and compared with the same entries of the GPU result."""
@@ -88,6 +89,63 @@ def test_gemm_full_size_sampled(oracle, m, n, k):
     ref, _ = oracle.gemm_nvfp4(va[rows.numpy()], sa[rows.numpy()], vb[cols.numpy()], sb[cols.numpy()], alpha)
     got = bits16(out[rows.cuda()][:, cols.cuda()])
     check(got, ref, oracle, f"{m}x{n}x{k}")
+
+
+@pytest.mark.parametrize(
+    ("m", "n", "k", "env"),
+    [
+        (128, 1024, 4096, {}),                                  # weight-streaming kernel, split 2
+        (128, 4096, 4096, {"FOS_GEMM_SPLITK": "3"}),            # ... ragged last split
+        (100, 2048, 3328, {"FOS_GEMM_SPLITK": "5"}),            # ... 13 steps, idle waves, 100 of 128 rows
+        (16, 1024, 4096, {}),                                   # ... one 32-row A tile
+        (48, 512, 2048, {"FOS_GEMM_SPLITK": "2"}),              # ... two
+        (128, 512, 1088, {}),                                   # K % 128 != 0: 128 x 128 tiles
+        (384, 256, 14336, {}),
+    ],
+)
+def test_gemm_split_k_matches_unsplit(monkeypatch, m, n, k, env):
+    """Small-M shapes split K when the caller lends a workspace.  Through the C ABI: the
+    split result equals the unsplit one and the 128 x 128-tile kernel's up to FP32
+    re-association (one bf16 ulp on a few outputs), two split runs are bit-identical
+    (fixed reduction order), and too small a workspace is ignored."""
+    from fouroversix_amd import _native as nat
+
+    for key, val in env.items():
+        monkeypatch.setenv(key, val)
+    L = nat.lib()
+    ws_bytes = int(L.fos_gemm_workspace_bytes(m, n, k))
+    assert ws_bytes > 0 and ws_bytes % (m * n * 4) == 0
+    cfg = fos.QuantizationConfig(scale_rule="mse")
+    qa = fos.quantize(make_input("randn", (m, k), 11).cuda(), cfg)
+    qb = fos.quantize(make_input("randn", (n, k), 12).cuda(), cfg)
+    alpha = fos.matmul.frontend.gemm_alpha(qa, qb).reshape(1).float().cuda()
+    stream = nat.current_stream(qa.values.device)
+
+    def run(ws, out_dtype=torch.bfloat16, rows=m):
+        out = torch.full((rows, n), 7.0, dtype=out_dtype, device="cuda")
+        rc = L.fos_gemm_nvfp4(qa.values.data_ptr(), qb.values.data_ptr(), qa.scale_factors.data_ptr(),
+                              qb.scale_factors.data_ptr(), alpha.data_ptr(), rows, n, k, out.data_ptr(),
+                              nat.TORCH_TO_T[out_dtype], n,
+                              ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        return out
+
+    def close(x, y):
+        diff = (x.float() - y.float()).abs()
+        assert float((diff > 0).float().mean()) <= 2e-2
+        assert float((diff / y.float().abs().clamp_min(1e-2)).max()) <= 2.0 ** -7
+
+    ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device="cuda")  # NaN patterns: every partial must be written
+    unsplit, split, again = run(None), run(ws), run(ws)
+    assert torch.equal(split, again)
+    assert not torch.isnan(split.float()).any()
+    close(split, unsplit)
+    assert torch.equal(run(ws[: ws_bytes - 16]), unsplit)
+    close(run(ws, torch.float16), run(None, torch.float16))
+    monkeypatch.setenv("FOS_GEMM_TILE", "1")  # the general kernel on the same operands
+    monkeypatch.delenv("FOS_GEMM_SPLITK", raising=False)
+    close(unsplit, run(None, rows=qa.values.shape[0])[:m])
 
 
 def test_linear_layer_forward(oracle):
