@@ -28,6 +28,7 @@ EXPORTS = (
     "fos_quantize_workspace_bytes",
     "fos_amax",
     "fos_quantize",
+    "fos_pseudo_quantize",
     "fos_gemm_nvfp4",
     "fos_gemm_workspace_bytes",
     "fos_dequantize",
@@ -68,6 +69,8 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, i32,
                                vp, vp, vp, i32, vp, sz, vp]
     L.fos_quantize.restype = i32
+    L.fos_pseudo_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i32, vp, sz, vp]
+    L.fos_pseudo_quantize.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
     L.fos_gemm_workspace_bytes.argtypes = [i64, i64, i64]

@@ -170,12 +170,15 @@ extern "C" int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, i
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
-extern "C" int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
-                            int dtype, int rule, int round_style, int block2d,
-                            uint64_t seed, uint64_t offset, int sf_layout,
-                            uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
-                            void *workspace, size_t workspace_bytes, fos_stream_t stream) {
-    if (!x || !codes || !sf || !amax) return FOS_E_NULL_POINTER;
+// Shared body of fos_quantize and fos_pseudo_quantize (pseudo_out != null: bf16 round trip
+// instead of codes / scales).
+static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                         int dtype, int rule, int round_style, int block2d,
+                         uint64_t seed, uint64_t offset, int sf_layout,
+                         uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                         void *workspace, size_t workspace_bytes, fos_stream_t stream,
+                         uint16_t *pseudo_out, int64_t ldo) {
+    if (!x || !amax || (!pseudo_out && (!codes || !sf))) return FOS_E_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if (x_type != FOS_T_BF16) return FOS_E_UNSUPPORTED;
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;
@@ -193,8 +196,16 @@ extern "C" int fos_quantize(const void *x, int x_type, int64_t rows, int64_t col
     hipStream_t s = (hipStream_t)stream;
     uint32_t *partials = (uint32_t *)workspace;
     const bool aligned = (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0);
+    if (pseudo_out) {
+        // only the NVFP4 round-to-nearest kernels have the fused epilogue
+        if (dtype != FOS_DTYPE_NVFP4 || round_style != FOS_ROUND_NEAREST || !aligned) return FOS_E_UNSUPPORTED;
+        if (ldo < cols) return FOS_E_BAD_SHAPE;
+        if (((uintptr_t)pseudo_out & 15) || (ldo % 8 != 0)) return FOS_E_BAD_ALIGNMENT;
+    }
 
     QuantParams p;
+    p.pseudo_out = pseudo_out;
+    p.ldo = ldo;
     p.x = (const uint16_t *)x;
     p.rows = rows; p.cols = cols; p.ld = ld;
     p.rows_p = rows_p; p.cols_p = cols_p;
@@ -241,4 +252,22 @@ extern "C" int fos_quantize(const void *x, int x_type, int64_t rows, int64_t col
         }
     }
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+extern "C" int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                            int dtype, int rule, int round_style, int block2d,
+                            uint64_t seed, uint64_t offset, int sf_layout,
+                            uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                            void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, seed, offset, sf_layout, codes, sf,
+                         amax, amax_is_input, workspace, workspace_bytes, stream, nullptr, 0);
+}
+
+extern "C" int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                                   int dtype, int rule, int round_style, int block2d,
+                                   void *out, int64_t ldo, float *amax, int amax_is_input,
+                                   void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!out) return FOS_E_NULL_POINTER;
+    return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, 0, 0, FOS_SF_LINEAR, nullptr, nullptr,
+                         amax, amax_is_input, workspace, workspace_bytes, stream, static_cast<uint16_t *>(out), ldo);
 }

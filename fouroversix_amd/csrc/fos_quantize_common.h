@@ -29,6 +29,8 @@ struct QuantParams {
     int sf_layout;
     int tiles_x;                 // workgroup tiles along the columns
     float c, qdiv, errdiv;       // f32(qmax*smax*adj), f32(qmax*adj), selection divisor
+    uint16_t *pseudo_out;        // fused quantize -> dequantize: bf16 [rows, cols] output instead of codes / sf
+    int64_t ldo;                 // its leading dimension
 };
 
 // ---- workgroup reductions ------------------------------------------------------------

@@ -372,4 +372,27 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
     return generic_block<RULE, TWO_D>(blk, k);
 }
 
+// The 16 dequantised values of a quantised NVFP4 block as bf16 pairs, with the operations
+// of the reference's dequantize (src/fouroversix/quantize/backend.py:141-155):
+// bf16(((value * scale) * amax) / c); value * scale is exact.  FASTDIV replaces the IEEE
+// division by the exact 3-operation form (quotient normal or zero) and restores the sign
+// of a zero quotient.
+template <bool FASTDIV>
+FOS_DEVICE void dequant_block_bf16(const BlockOut &o, float amax, float c, float rc, uint32_t *w) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const float sf = e4m3_decode(o.s & 0x7fu);
+    static_for<0, 8>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const float2_t v = unpack_fp4<(j & 3)>(j < 4 ? o.c0 : o.c1);
+        float2_t q;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float f = (v[e] * sf) * amax;
+            if (FASTDIV) q[e] = u2f((f2u(div_const(f, c, rc)) & 0x7fffffffu) | (f2u(f) & 0x80000000u));
+            else q[e] = f / c;
+        }
+        w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_t));
+    });
+}
+
 }  // namespace fos

@@ -39,7 +39,7 @@ FOS_DEVICE void load_tile(const QuantParams &p, uint32_t tile, int lane, int wav
     }
 }
 
-template <int RULE, bool TWO_D>
+template <int RULE, bool TWO_D, bool PSEUDO>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_kernel(const QuantParams p) {
     __shared__ uint32_t red[4];
     __shared__ uint32_t sf_tile[2][128];
@@ -57,14 +57,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
-    const float rq = 1.0f / k.qdiv;
+    const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t sf_cols = p.cols_p >> 4;
     const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
-    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    const bool tiled = !PSEUDO && p.sf_layout == FOS_SF_TILED_128X4;
 
     auto process = [&](uint32_t tile, const TileRegs &t, uint32_t *stage) {
         const int64_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - (uint32_t)tile_y * (uint32_t)p.tiles_x;
@@ -74,6 +74,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const int rr = h * 64 + wave * 16 + (lane & 15);
             const int64_t r = tile_y * 128 + rr;
             const BlockOut o = quantize_block_nvfp4_rtn<RULE, TWO_D>(t.b[h], k, enc_fast, rq, maybe_negzero, in_range, lut);
+            if (PSEUDO) {
+                uint32_t w[8];
+                if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+                else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
+                if (r < p.rows && cb * 16 < p.cols) {
+                    uint4 *d = reinterpret_cast<uint4 *>(p.pseudo_out + r * p.ldo + cb * 16);
+                    d[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                    d[1] = make_uint4(w[4], w[5], w[6], w[7]);
+                }
+                continue;
+            }
             *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(o.c0, o.c1);
             if (tiled) reinterpret_cast<uint8_t *>(stage)[(rr & 31) * 16 + (rr >> 5) * 4 + (lane >> 4)] = (uint8_t)o.s;
             else p.sf[r * sf_cols + cb] = (uint8_t)o.s;
@@ -106,7 +117,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 // within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns; workgroups stride
 // over the tiles so that the per-workgroup setup (tensor maximum, scale table) is paid
 // once for several tiles.  FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
-template <int RULE, bool FULL>
+template <int RULE, bool FULL, bool PSEUDO>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
@@ -125,7 +136,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
-    const float rq = 1.0f / k.qdiv;
+    const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
     __syncthreads();
 
@@ -133,7 +144,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     const int64_t sf_cols = p.cols_p >> 4;
     const int lb = lane & 15;                // block column inside the tile
     const int rr0 = wave * 4 + (lane >> 4);  // row inside a 16-row step
-    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    const bool tiled = !PSEUDO && p.sf_layout == FOS_SF_TILED_128X4;
     const int64_t row_pitch = p.ld, code_pitch = p.cols_p >> 1;
     const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
     int buf = 0;
@@ -168,6 +179,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             if (col_ok) {
                 const int rr = g * 16 + rr0;
                 const BlockOut o = quantize_block_nvfp4_rtn<RULE, false>(blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut);
+                if (PSEUDO) {
+                    uint32_t w[8];
+                    if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+                    else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
+                    if (FULL || (row0 + g * 16 < p.rows && cb * 16 < p.cols)) {
+                        uint4 *d = reinterpret_cast<uint4 *>(p.pseudo_out + (row0 + g * 16) * p.ldo + cb * 16);
+                        d[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                        d[1] = make_uint4(w[4], w[5], w[6], w[7]);
+                    }
+                    continue;
+                }
                 *reinterpret_cast<uint2 *>(dst + (int64_t)g * 16 * code_pitch) = make_uint2(o.c0, o.c1);
                 if (tiled) stage[(rr & 31) * 16 + (rr >> 5) * 4] = (uint8_t)o.s;
                 else p.sf[(row0 + g * 16) * sf_cols + cb] = (uint8_t)o.s;
@@ -187,9 +209,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     }
 }
 
-template <int RULE>
+template <int RULE, bool PSEUDO>
 static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     if (!aligned) {
+        if (PSEUDO) return;  // rejected by the entry point
         if (two_d) launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
         else launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
         return;
@@ -204,9 +227,9 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         if (grid > n) grid = n;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
         if (full)
-            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else
-            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, false>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, false, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         return;
     }
     p.tiles_x = (int)(p.cols_p / 64);
@@ -216,20 +239,26 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     int64_t grid = 256 * 6;
     if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
     if (grid > n_tiles) grid = n_tiles;
-    hipLaunchKernelGGL((quantize_nvfp4_rtn_kernel<RULE, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((quantize_nvfp4_rtn_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
-void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {
+template <bool PSEUDO>
+static void by_rule(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {
     switch (rule) {
         case FOS_RULE_STATIC_6:
         case FOS_RULE_STATIC_4:
             // the two static rules differ only in the host-computed constants
-            by_dim<FOS_RULE_STATIC_6>(p, two_d, aligned, s);
+            by_dim<FOS_RULE_STATIC_6, PSEUDO>(p, two_d, aligned, s);
             break;
-        case FOS_RULE_MAE: by_dim<FOS_RULE_MAE>(p, two_d, aligned, s); break;
-        case FOS_RULE_MSE: by_dim<FOS_RULE_MSE>(p, two_d, aligned, s); break;
-        default: by_dim<FOS_RULE_ABS_MAX>(p, two_d, aligned, s); break;
+        case FOS_RULE_MAE: by_dim<FOS_RULE_MAE, PSEUDO>(p, two_d, aligned, s); break;
+        case FOS_RULE_MSE: by_dim<FOS_RULE_MSE, PSEUDO>(p, two_d, aligned, s); break;
+        default: by_dim<FOS_RULE_ABS_MAX, PSEUDO>(p, two_d, aligned, s); break;
     }
+}
+
+void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {
+    if (p.pseudo_out) by_rule<true>(p, rule, two_d, aligned, s);
+    else by_rule<false>(p, rule, two_d, aligned, s);
 }
 
 }  // namespace fos

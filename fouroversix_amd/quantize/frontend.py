@@ -68,6 +68,13 @@ def quantize(
         raise ValueError(msg)
 
     if config.pseudo_quantize:
+        # one fused kernel where the library has it, else the two-step round trip
+        # (QuantizeBackendBase.pseudo_quantize, src/fouroversix/quantize/backend.py:213-234)
+        fmt, style = NATIVE_FORMAT_IDS[config.dtype.value], config.round_style.native_id
+        if ops.pseudo_quantize_is_fused(x, fmt, style):
+            return ops.pseudo_quantize(
+                x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax")
+            )
         plain = QuantizationConfig(**{**config.__dict__, "pseudo_quantize": False})
         return dequantize(quantize(x, plain), dtype=x.dtype)
 

@@ -25,6 +25,9 @@ _LIB.define(
     "quantize_ex(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, int seed, int offset, "
     "int sf_layout, Tensor? amax) -> (Tensor, Tensor, Tensor)"
 )
+_LIB.define(
+    "pseudo_quantize(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, Tensor? amax) -> Tensor"
+)
 _LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
 _LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
 _LIB.define(
@@ -109,6 +112,46 @@ def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, s
     return values, sf, amax_buf
 
 
+def pseudo_quantize_is_fused(x: torch.Tensor, dtype: int, round_style: int) -> bool:
+    """True when the library has a fused quantize->dequantize kernel for this call."""
+    return (
+        dtype == 0
+        and round_style == 0
+        and x.dim() == 2
+        and x.dtype == torch.bfloat16
+        and x.numel() > 0
+        and x.stride(-1) == 1
+        and x.shape[1] % 16 == 0
+        and x.stride(0) % 8 == 0
+        and x.data_ptr() % 16 == 0
+    )
+
+
+def _pseudo_quantize_impl(x, dtype, selection_rule, round_style, is_2d, amax):
+    if not pseudo_quantize_is_fused(x, dtype, round_style):
+        raise RuntimeError("pseudo_quantize: no fused kernel for these arguments (quantize, then dequantize)")
+    nat.require_gpu_tensor(x, "x")
+    rows, cols = x.shape
+    dev = x.device
+    out = torch.empty(rows, cols, dtype=torch.bfloat16, device=dev)
+    amax_is_input = amax is not None
+    amax_buf = (
+        amax.reshape(1).to(device=dev, dtype=torch.float32).contiguous()
+        if amax_is_input
+        else torch.empty(1, dtype=torch.float32, device=dev)
+    )
+    with _on_device(dev):
+        stream = nat.current_stream(dev)
+        workspace = _workspace(dev, stream)
+        rc = nat.lib().fos_pseudo_quantize(
+            x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), dtype, selection_rule, round_style, int(is_2d),
+            out.data_ptr(), cols, amax_buf.data_ptr(), int(amax_is_input),
+            workspace.data_ptr(), workspace.numel(), stream,
+        )
+    nat.check(rc, "fouroversix::pseudo_quantize")
+    return out
+
+
 def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
     if not is_nvfp4:
         raise RuntimeError("quantize: only the NVFP4 format is implemented by this op (use quantize_ex for IF4)")
@@ -182,6 +225,7 @@ def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, row
 
 _LIB.impl("quantize", _quantize_ref_schema, "CUDA")
 _LIB.impl("quantize_ex", _quantize_impl, "CUDA")
+_LIB.impl("pseudo_quantize", _pseudo_quantize_impl, "CUDA")
 _LIB.impl(
     "gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt",
     lambda a, b, a_sf, b_sf, alpha: _gemm_impl(a, b, a_sf, b_sf, alpha, torch.bfloat16),
@@ -212,6 +256,11 @@ def _(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
 @torch.library.register_fake("fouroversix::quantize_ex")
 def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
     return _fake_quantize_shapes(x)
+
+
+@torch.library.register_fake("fouroversix::pseudo_quantize")
+def _(x, dtype, selection_rule, round_style, is_2d, amax):
+    return torch.empty_like(x, memory_format=torch.contiguous_format)
 
 
 @torch.library.register_fake("fouroversix::gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt")
@@ -245,6 +294,13 @@ def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_l
     return torch.ops.fouroversix.quantize_ex.default(
         x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax
     )
+
+
+def pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax=None):
+    """Fused quantize -> dequantize (bf16 in, bf16 out); see ``pseudo_quantize_is_fused``."""
+    if type(x) is torch.Tensor and x.device.type == "cuda" and not torch.compiler.is_compiling():
+        return _pseudo_quantize_impl(x, dtype, selection_rule, round_style, is_2d, amax)
+    return torch.ops.fouroversix.pseudo_quantize.default(x, dtype, selection_rule, round_style, is_2d, amax)
 
 
 def _direct(t: torch.Tensor) -> bool:

@@ -95,6 +95,21 @@ int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t 
                  void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * Fused quantize -> dequantize round trip: out[rows, cols] (bf16, leading dimension ldo) =
+ * the values fos_dequantize would return for fos_quantize's result, without materialising
+ * codes or scales.  Stands in for QuantizeBackendBase.pseudo_quantize
+ * (src/fouroversix/quantize/backend.py:213-234; fused Triton kernel
+ * src/fouroversix/kernels/triton/ops.py:212-374).  Arguments as fos_quantize.  Fused
+ * kernels exist for FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST, x and out 16-byte aligned,
+ * ld and ldo multiples of 8 and cols a multiple of 16; anything else returns
+ * FOS_E_UNSUPPORTED (compose fos_quantize and fos_dequantize instead).
+ */
+int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                        int dtype, int rule, int round_style, int block2d,
+                        void *out, int64_t ldo, float *amax, int amax_is_input,
+                        void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * D[M, N] = alpha * sum_k (A[m,k] * sfA[m,k/16]) * (B[n,k] * sfB[n,k/16]), FP32
  * accumulation, written as out_type (FOS_T_BF16 or FOS_T_F16) with leading dimension ldd.
  * Stands in for torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_{bf16,fp16}_tnt

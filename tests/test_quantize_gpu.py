@@ -212,13 +212,72 @@ def test_dequantize_bit_exact(oracle, dtype, rule, out):
                        expect.view(torch.int16 if out != torch.float32 else torch.int32))
 
 
-def test_pseudo_quantize_is_the_round_trip():
-    """quantize(pseudo_quantize=True) == dequantize(quantize(x), dtype=x.dtype)
-    (reference tests/test_quantize.py:391-458)."""
-    x = make_input("randn", (512, 1024), 10).cuda()
-    for rule in ("mse", "static_6", "abs_max"):
-        r = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, pseudo_quantize=True))
-        e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(scale_rule=rule)), dtype=x.dtype,
-                           intermediate_dtype=torch.float32)
-        assert isinstance(r, torch.Tensor) and r.dtype == torch.bfloat16 and r.shape == x.shape
-        assert torch.equal(r, e)
+@pytest.mark.parametrize("two_d", [False, True])
+@pytest.mark.parametrize("rule", ["mse", "mae", "abs_max", "static_6", "static_4"])
+@pytest.mark.parametrize(
+    ("kind", "shape", "scale"),
+    [
+        ("randn", (512, 1024), 1.0),
+        ("outlier", (256, 512), 1.0),
+        ("tiny_blocks", (200, 144), 1.0),   # ragged rows, cols % 64 != 0, sub-normal block scales
+        ("rand01", (128, 256), 1.0),
+        ("zeros", (128, 64), 1.0),
+        ("randn", (130, 272), 2.0 ** -110),  # outside the fast range: IEEE division path
+        ("randn", (128, 256), 2.0 ** 105),
+    ],
+)
+def test_pseudo_quantize_is_the_round_trip(kind, shape, scale, rule, two_d):
+    """quantize(pseudo_quantize=True), one fused kernel, is bit-identical to
+    dequantize(quantize(x), dtype=x.dtype) (reference tests/test_quantize.py:391-458;
+    QuantizeBackendBase.pseudo_quantize, quantize/backend.py:213-234), signs of zeros
+    included."""
+    x = (make_input(kind, shape, 10).float() * scale).bfloat16()
+    x[0, :16] = -x[0, :16].abs()
+    x[1, 3] = -0.0
+    x = x.cuda()
+    assert fos.quantize.__module__ and fos.quantize  # public entry
+    from fouroversix_amd.quantize import ops
+
+    assert ops.pseudo_quantize_is_fused(x, 0, 0)
+    r = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, block_scale_2d=two_d, pseudo_quantize=True))
+    e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, block_scale_2d=two_d)), dtype=x.dtype)
+    assert isinstance(r, torch.Tensor) and r.dtype == torch.bfloat16 and r.shape == x.shape
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+
+
+def test_pseudo_quantize_unfused_cases_and_amax():
+    """Configurations without a fused kernel take the two-step path (same result type);
+    a caller-supplied amax is honoured by the fused kernel."""
+    from fouroversix_amd.quantize import ops
+
+    x = make_input("randn", (256, 200), 3).cuda()  # cols % 16 != 0
+    assert not ops.pseudo_quantize_is_fused(x, 0, 0)
+    r = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True))
+    e = fos.dequantize(fos.quantize(x), dtype=x.dtype)
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+    x = make_input("randn", (256, 256), 4).cuda()
+    cfg = dict(scale_rule="mse", round_style="stochastic", kwargs={"seed": 5})
+    r = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True, **cfg))
+    e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(**cfg)), dtype=x.dtype)
+    assert torch.equal(r, e)
+    r = fos.quantize(x, fos.QuantizationConfig(dtype="if4", pseudo_quantize=True))
+    assert torch.equal(r, fos.dequantize(fos.quantize(x, fos.QuantizationConfig(dtype="if4")), dtype=x.dtype))
+    amax = torch.tensor(8.0, device="cuda")
+    r = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True, kwargs={"amax": amax}))
+    e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(kwargs={"amax": amax})), dtype=x.dtype)
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+
+
+def test_pseudo_quantize_full_size():
+    """North-star shape: the fused kernel against the two-step path, and idempotence (a
+    dequantised tensor re-quantises to itself with the same tensor maximum)."""
+    x = make_input("randn", (8192, 8192), 1).cuda()
+    cfg = fos.QuantizationConfig(scale_rule="mse", pseudo_quantize=True)
+    r = fos.quantize(x, cfg)
+    e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(scale_rule="mse")), dtype=x.dtype)
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+    del e
+    s6 = fos.QuantizationConfig(scale_rule="static_6", pseudo_quantize=True)
+    once = fos.quantize(x, s6)
+    # by value: a -0.0 (a negative input that rounded to zero) re-quantizes to +0.0
+    assert torch.equal(fos.quantize(once, s6), once)
