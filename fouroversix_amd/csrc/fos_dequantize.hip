@@ -5,7 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "fos_device.h"
+#include "fos_quantize_fast.h"
 #include "fouroversix_hip.h"
 
 namespace fos {
@@ -17,56 +17,95 @@ struct DequantParams {
     int64_t rows, cols, rows_p, cols_p, ldo;
     float divisor;
     int sf_layout;
+    int fast_div;       // divisor is 1536, 1792 or 2688 (exact 3-operation division)
+    int vector_stores;  // out and ldo allow 16-byte stores of whole blocks
 };
 
-FOS_DEVICE float e2m1_value(uint32_t code) {
-    // magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6: (e, m) = (code >> 1 & 3, code & 1)
-    const uint32_t e = (code >> 1) & 3u, m = code & 1u;
-    float v = e == 0 ? 0.5f * (float)m : u2f((126u + e) << 23 | m << 22);
-    return (code & 8u) ? -v : v;
-}
-
+// One thread per 1x16 block (consecutive threads = consecutive blocks of a row: 512
+// contiguous bytes of codes in, 2 KiB of bf16 out per wavefront).  `p.fast_div`: the divisor
+// is one of the constants for which the 3-operation division is exact; it is used when amax
+// is far enough from the ends of the float range for every quotient to be normal or zero.
 template <int DT, int OUT>
 __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) {
     const int64_t sf_cols = p.cols_p >> 4;
     const int64_t blk = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t n_blocks = p.rows * ((p.cols + 15) >> 4);
-    if (blk >= n_blocks) return;
     const int64_t bpr = (p.cols + 15) >> 4;
-    const int64_t r = blk / bpr, cb = blk % bpr;
+    const int64_t n_blocks = p.rows * bpr;
+    if (blk >= n_blocks) return;
+    const int64_t r = blk / bpr, cb = blk - r * bpr;
     const uint2 q = *reinterpret_cast<const uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8);
     const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
                              ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
                              : r * sf_cols + cb;
     const uint32_t sb = p.sf[sofs];
-    const bool is_int = DT == FOS_DTYPE_IF4 && (sb & 0x80u);
-    const _Float16 s16 = (_Float16)e4m3_decode(sb & 0x7fu);
     const float amax = *p.amax;
-    const float six_sevenths = (float)(6.0 / 7.0);
+    const float sf = e4m3_decode(sb & 0x7fu);
+
+    // value * scale, as the fp16 product of the reference (exact for E2M1 values)
+    float f[16];
+    if (DT == FOS_DTYPE_IF4 && (sb & 0x80u)) {
+        const _Float16 s16 = (_Float16)sf;
+        const float six_sevenths = (float)(6.0 / 7.0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const int64_t c = cb * 16 + i;
-        if (c >= p.cols) break;
-        const uint32_t word = i < 8 ? q.x : q.y;
-        const uint32_t code = (word >> (4 * (i & 7))) & 0xfu;
-        _Float16 v16;
-        if (is_int) {
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t code = ((i < 8 ? q.x : q.y) >> (4 * (i & 7))) & 0xfu;
             const int iv = ((int)(code << 28)) >> 28;
-            v16 = (_Float16)((float)iv * six_sevenths);
-        } else {
-            v16 = (_Float16)e2m1_value(code);
+            f[i] = (float)((_Float16)((float)iv * six_sevenths) * s16);
         }
-        const _Float16 r16 = v16 * s16;
-        const float f = ((float)r16 * amax) / p.divisor;
-        if (OUT == FOS_T_F32) {
-            reinterpret_cast<float *>(p.out)[r * p.ldo + c] = f;
-        } else if (OUT == FOS_T_F16) {
-            reinterpret_cast<_Float16 *>(p.out)[r * p.ldo + c] = (_Float16)f;
-        } else {
-            uint32_t u = f2u(f);
-            u += 0x7fffu + ((u >> 16) & 1u);
-            reinterpret_cast<uint16_t *>(p.out)[r * p.ldo + c] = (uint16_t)(u >> 16);
+    } else {
+        static_for<0, 8>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const float2_t v = unpack_fp4<(j & 3)>(j < 4 ? q.x : q.y);
+            f[2 * j] = v.x * sf;
+            f[2 * j + 1] = v.y * sf;
+        });
+    }
+    if (p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f) {
+        const float rc = 1.0f / p.divisor;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float t = f[i] * amax;
+            f[i] = u2f((f2u(div_const(t, p.divisor, rc)) & 0x7fffffffu) | (f2u(t) & 0x80000000u));
         }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) f[i] = (f[i] * amax) / p.divisor;
+    }
+
+    const int64_t c0 = cb * 16;
+    const bool whole = p.vector_stores && c0 + 16 <= p.cols;
+    if (OUT == FOS_T_F32) {
+        float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
+        if (whole) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) reinterpret_cast<float4 *>(o)[v] = make_float4(f[4 * v], f[4 * v + 1], f[4 * v + 2], f[4 * v + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (c0 + i < p.cols) o[i] = f[i];
+        }
+        return;
+    }
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float2_t v = {f[2 * j], f[2 * j + 1]};
+        if (OUT == FOS_T_F16) {
+            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2_t));
+        } else {
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+        }
+    }
+    uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
+    if (whole) {
+        reinterpret_cast<uint4 *>(o)[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        reinterpret_cast<uint4 *>(o)[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
     }
 }
 
@@ -99,6 +138,9 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
     p.divisor = (float)divisor;
     p.sf_layout = sf_layout;
+    p.fast_div = p.divisor == 1536.0f || p.divisor == 1792.0f || p.divisor == 2688.0f;
+    const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
+    p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
     const int64_t n_blocks = rows * ((cols + 15) / 16);
     if ((n_blocks + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     dim3 grid((unsigned)((n_blocks + 255) / 256));
