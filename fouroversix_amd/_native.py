@@ -29,6 +29,7 @@ EXPORTS = (
     "fos_amax",
     "fos_quantize",
     "fos_pseudo_quantize",
+    "fos_transform",
     "fos_gemm_nvfp4",
     "fos_gemm_workspace_bytes",
     "fos_dequantize",
@@ -71,6 +72,8 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize.restype = i32
     L.fos_pseudo_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i32, vp, sz, vp]
     L.fos_pseudo_quantize.restype = i32
+    L.fos_transform.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, i64, vp, vp, sz, vp]
+    L.fos_transform.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
     L.fos_gemm_workspace_bytes.argtypes = [i64, i64, i64]

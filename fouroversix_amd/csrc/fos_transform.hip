@@ -1,0 +1,202 @@
+// gfx950 pre-transform of the training-side quantize options: y = x^T and / or the 16-point
+// random Hadamard transform of every group of 16 consecutive elements of a row, together
+// with the tensor maximum of y -- the steps the reference performs before it scales
+// (src/fouroversix/quantize/pytorch/reference.py:567-578; sign vector and matrix
+// src/fouroversix/quantize/utils.py:19-85; CUDA form src/fouroversix/csrc/include/
+// hadamard_transform.h:16-37).  The result is a plain bf16 matrix that fos_quantize then
+// reads with `amax_is_input`, so the whole option costs one extra write and read of x.
+//
+// RHT arithmetic: the reference multiplies bf16 [.., 16] by the bf16 matrix
+// diag(signs) * H16 / 4 with fp32 accumulation and one rounding to bf16.  All products are
+// exact, so the sum is evaluated here as a fast Walsh-Hadamard butterfly in fp32 (64 adds
+// instead of 256 multiply-adds) and scaled by 1/4 at the end; the two orders of summation
+// agree unless the fp32 partial sums themselves round, i.e. unless a group spans more
+// than ~12 binades, and then only when the last fp32 bit decides a bf16 rounding.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fos_quantize_common.h"
+#include "fouroversix_hip.h"
+
+namespace fos {
+
+struct TransformParams {
+    const uint16_t *x;
+    int64_t rows, cols, ld;  // input
+    uint16_t *y;
+    int64_t ldy;             // output [cols, rows] if transposed else [rows, cols]
+    uint32_t *partials;      // pairs {max |y| as f32 bits, 1 if a -0.0 was written}
+    int64_t n_units;         // tiles (transpose) or 16-element groups (rows)
+    int tiles_x;
+};
+
+typedef float float2_tt __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_tt __attribute__((ext_vector_type(2)));
+
+// signs of the reference's fixed vector as a bit mask (bit i set: element i is negated)
+constexpr uint32_t kRhtNegMask = (1u << 3) | (1u << 5) | (1u << 6) | (1u << 7) | (1u << 8) | (1u << 9) | (1u << 10) |
+                                 (1u << 12) | (1u << 14) | (1u << 15);
+
+// w[0..7]: 16 bf16 (element 2j in the low half of w[j]) -> RHT -> 16 bf16, same packing.
+FOS_DEVICE void rht16(uint32_t *w) {
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        v[2 * j] = u2f((w[j] << 16) ^ (((kRhtNegMask >> (2 * j)) & 1u) << 31));
+        v[2 * j + 1] = u2f((w[j] & 0xffff0000u) ^ (((kRhtNegMask >> (2 * j + 1)) & 1u) << 31));
+    }
+#pragma unroll
+    for (int len = 1; len < 16; len <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if ((i & len) == 0) {
+                const float a = v[i], b = v[i + len];
+                v[i] = a + b;
+                v[i + len] = a - b;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        // + 0.0f: a dot product accumulated from +0 never yields -0
+        const float2_tt q = {v[2 * j] * 0.25f + 0.0f, v[2 * j + 1] * 0.25f + 0.0f};
+        w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_tt));
+    }
+}
+
+FOS_DEVICE void track(const uint32_t *w, uint32_t &m, uint32_t &z) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        m = pk_max_u16(m, w[j] & 0x7fff7fffu);
+        z = pk_min_i16(z, w[j]);
+    }
+}
+
+FOS_DEVICE void write_partials(uint32_t m, uint32_t z, uint32_t *partials) {
+    __shared__ uint32_t smem[4];
+    uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    mm = block_max_u32(mm, smem);
+    const uint32_t zz = block_max_u32(((z & 0xffffu) == 0x8000u || (z >> 16) == 0x8000u) ? 1u : 0u, smem);
+    if (threadIdx.x == 0) {
+        partials[2 * blockIdx.x] = mm << 16;
+        partials[2 * blockIdx.x + 1] = zz;
+    }
+}
+
+// RHT without transposition: one thread per group of 16, grid-stride.
+__global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParams p) {
+    const int64_t groups_per_row = p.cols >> 4;
+    uint32_t m = 0, z = 0;
+    for (int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x; g < p.n_units; g += (int64_t)gridDim.x * kThreads) {
+        const int64_t r = g / groups_per_row, cb = g - r * groups_per_row;
+        const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + cb * 16);
+        const uint4 lo = src[0], hi = src[1];
+        uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        rht16(w);
+        track(w, m, z);
+        uint4 *dst = reinterpret_cast<uint4 *>(p.y + r * p.ldy + cb * 16);
+        dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+        dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+    write_partials(m, z, p.partials);
+}
+
+// Transposition (optionally followed by the RHT along the new rows) through a 64 x 64 LDS
+// tile: rows of x come in as 128-byte runs, rows of y leave as 128-byte runs.  rows and
+// cols are multiples of 16, so 16-element groups are either inside or outside the matrix.
+template <bool RHT>
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformParams p) {
+    constexpr int kPitchT = 66;  // halfs per LDS row: 33 dwords, odd, so a column walk changes bank every row
+    __shared__ uint16_t tile[64 * kPitchT];
+    const int t = threadIdx.x;
+    uint32_t m = 0, z = 0;
+    for (int64_t u = blockIdx.x; u < p.n_units; u += gridDim.x) {
+        const int64_t ty = u / p.tiles_x, tx = u - ty * p.tiles_x;
+        const int64_t r0 = ty * 64, c0 = tx * 64;
+        {
+            const int row = t >> 2, chunk = t & 3;
+            uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (r0 + row < p.rows && c0 + chunk * 16 < p.cols) {
+                const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (r0 + row) * p.ld + c0 + chunk * 16);
+                const uint4 lo = src[0], hi = src[1];
+                w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
+                w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
+            }
+            uint32_t *d = reinterpret_cast<uint32_t *>(tile + row * kPitchT + chunk * 16);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) d[j] = w[j];
+        }
+        __syncthreads();
+        {
+            const int rb = t & 3, c = t >> 2;  // output row c0 + c, output columns r0 + 16 rb ...
+            if (c0 + c < p.cols && r0 + rb * 16 < p.rows) {
+                uint32_t w[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t a = tile[(rb * 16 + 2 * j) * kPitchT + c], b = tile[(rb * 16 + 2 * j + 1) * kPitchT + c];
+                    w[j] = a | (b << 16);
+                }
+                if (RHT) rht16(w);
+                track(w, m, z);
+                uint4 *dst = reinterpret_cast<uint4 *>(p.y + (c0 + c) * p.ldy + r0 + rb * 16);
+                dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+            }
+        }
+        __syncthreads();
+    }
+    write_partials(m, z, p.partials);
+}
+
+__global__ __launch_bounds__(kThreads) void transform_amax_kernel(const uint32_t *__restrict__ partials, int n,
+                                                                  float *__restrict__ amax) {
+    __shared__ uint32_t smem[4];
+    uint32_t m = 0;
+    for (int i = threadIdx.x; i < n; i += kThreads) m = m > partials[2 * i] ? m : partials[2 * i];
+    m = block_max_u32(m, smem);
+    if (threadIdx.x == 0) *amax = u2f(m);
+}
+
+}  // namespace fos
+
+using namespace fos;
+
+extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                             int transpose, int rht, void *y, int64_t ldy, float *amax,
+                             void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!x || !y || !amax) return FOS_E_NULL_POINTER;
+    if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
+    if (x_type != FOS_T_BF16 || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
+    const int64_t out_cols = transpose ? rows : cols;
+    if (ldy < out_cols) return FOS_E_BAD_SHAPE;
+    // whole 16-element groups in both orientations
+    if (cols % 16 != 0 || (transpose && rows % 16 != 0)) return FOS_E_UNSUPPORTED;
+    if (!workspace || workspace_bytes < fos_quantize_workspace_bytes(rows, cols)) return FOS_E_WORKSPACE;
+    if (((uintptr_t)x & 15) || ((uintptr_t)y & 15) || (ld % 8 != 0) || (ldy % 8 != 0) || ((uintptr_t)workspace & 7) ||
+        ((uintptr_t)amax & 3))
+        return FOS_E_BAD_ALIGNMENT;
+    TransformParams p;
+    p.x = static_cast<const uint16_t *>(x);
+    p.rows = rows; p.cols = cols; p.ld = ld;
+    p.y = static_cast<uint16_t *>(y);
+    p.ldy = ldy;
+    p.partials = static_cast<uint32_t *>(workspace);
+    hipStream_t s = (hipStream_t)stream;
+    int64_t grid;
+    constexpr int64_t kMaxGrid = 1024;  // pairs the workspace holds
+    if (transpose) {
+        p.tiles_x = (int)((cols + 63) / 64);
+        p.n_units = ((rows + 63) / 64) * p.tiles_x;
+        grid = p.n_units < kMaxGrid ? p.n_units : kMaxGrid;
+        if (rht) hipLaunchKernelGGL(transpose_kernel<true>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL(transpose_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    } else {
+        p.tiles_x = 0;
+        p.n_units = rows * (cols / 16);
+        grid = (p.n_units + kThreads - 1) / kThreads;
+        if (grid > kMaxGrid) grid = kMaxGrid;
+        hipLaunchKernelGGL(rht_rows_kernel, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    }
+    hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s, p.partials, (int)grid, amax);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}

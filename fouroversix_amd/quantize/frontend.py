@@ -30,14 +30,12 @@ def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | Non
         return f"scale rule {config.scale_rule.value} is not defined for {config.dtype.value}"
     if config.dtype.value not in NATIVE_FORMAT_IDS:
         return f"format {config.dtype.value} has no gfx950 kernel"
-    if config.rht:
-        return "the random Hadamard transform is not implemented"
-    if config.transpose:
-        return "transposed quantization is not implemented"
     if x.device.type != "cuda":
         return f"input must live on the GPU, got {x.device}"
     if x.dtype != torch.bfloat16:
         return f"input must be bfloat16, got {x.dtype}"
+    if config.rht or config.transpose:
+        return ops.transform_unsupported_reason(x, config.transpose, config.rht)
     return None
 
 
@@ -66,6 +64,19 @@ def quantize(
         else:
             msg = f"Backend {config.backend} does not support the given parameters ({reason})"
         raise ValueError(msg)
+
+    if config.transpose or config.rht:
+        # x.T and / or the random Hadamard transform first (reference
+        # quantize/pytorch/reference.py:567-571), as one pass that also yields the tensor
+        # maximum; the rest is the plain path on the transformed tensor
+        if "amax" in config.kwargs:
+            msg = "kwargs['amax'] cannot be combined with transpose / rht (the maximum is that of the transformed tensor)"
+            raise ValueError(msg)
+        y, amax = ops.transform(x, config.transpose, config.rht)
+        plain = QuantizationConfig(
+            **{**config.__dict__, "transpose": False, "rht": False, "kwargs": {**config.kwargs, "amax": amax}}
+        )
+        return quantize(y, plain)
 
     if config.pseudo_quantize:
         # one fused kernel where the library has it, else the two-step round trip

@@ -152,15 +152,49 @@ def _pseudo_quantize_impl(x, dtype, selection_rule, round_style, is_2d, amax):
     return out
 
 
+def transform_unsupported_reason(x: torch.Tensor, transpose: bool, rht: bool) -> str | None:
+    """Why the transpose / random-Hadamard pre-transform cannot run on ``x``, or None."""
+    rows, cols = x.shape
+    if cols % 16 != 0 or (transpose and rows % 16 != 0):
+        return "transpose / rht need dimensions that are multiples of 16"
+    return None
+
+
+def _transform_impl(x, transpose, rht):
+    """``(y, amax)``: y = RHT(x^T) as the reference forms it before scaling, amax = max|y|."""
+    if x.dim() != 2 or x.dtype != torch.bfloat16:
+        raise RuntimeError("transform: x must be a 2-D bfloat16 tensor")
+    nat.require_gpu_tensor(x, "x")
+    reason = transform_unsupported_reason(x, transpose, rht)
+    if reason is not None:
+        raise RuntimeError(f"transform: {reason}")
+    if x.stride(-1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+        x = x.contiguous()
+    rows, cols = x.shape
+    dev = x.device
+    y = torch.empty((cols, rows) if transpose else (rows, cols), dtype=torch.bfloat16, device=dev)
+    amax = torch.empty(1, dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        stream = nat.current_stream(dev)
+        workspace = _workspace(dev, stream)
+        rc = nat.lib().fos_transform(
+            x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), int(transpose), int(rht),
+            y.data_ptr(), y.stride(0), amax.data_ptr(), workspace.data_ptr(), workspace.numel(), stream,
+        )
+    nat.check(rc, "fouroversix::transform")
+    return y, amax
+
+
 def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
     if not is_nvfp4:
         raise RuntimeError("quantize: only the NVFP4 format is implemented by this op (use quantize_ex for IF4)")
-    if is_rht or is_transpose:
-        raise RuntimeError("quantize: rht / transpose are not implemented")
     if not 0 <= selection_rule <= 4:
         raise RuntimeError(f"Invalid selection_rule: {selection_rule}")
     seed = 0 if rbits < 0 else rbits
-    return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, None)
+    amax = None
+    if is_rht or is_transpose:
+        x, amax = _transform_impl(x, is_transpose, is_rht)
+    return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, amax)
 
 
 def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
@@ -294,6 +328,11 @@ def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_l
     return torch.ops.fouroversix.quantize_ex.default(
         x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax
     )
+
+
+def transform(x, transpose, rht):
+    """Pre-transform of the ``transpose`` / ``rht`` quantize options: ``(y, amax)``."""
+    return _transform_impl(x, transpose, rht)
 
 
 def pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax=None):

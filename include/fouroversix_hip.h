@@ -95,6 +95,22 @@ int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t 
                  void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * Pre-transform of the training-side quantize options: y = x^T (transpose != 0) and / or
+ * the 16-point random Hadamard transform of every group of 16 consecutive row elements
+ * (rht != 0; fixed sign vector), written as a row-major bf16 matrix y ([cols, rows] when
+ * transposed, else [rows, cols]; leading dimension ldy), and amax[0] = max |y|.  Stands in
+ * for the `x.T` / `x.reshape(-1, 16) @ had` / `abs().max()` steps of the reference
+ * quantizer (src/fouroversix/quantize/pytorch/reference.py:567-578,
+ * quantize/utils.py:19-85; CUDA: csrc/include/hadamard_transform.h:16-37).  Follow it with
+ * fos_quantize(y, ..., amax, amax_is_input = 1).  x and y 16-byte aligned, ld and ldy
+ * multiples of 8, cols (and rows when transposing) multiples of 16; same workspace as
+ * fos_quantize.
+ */
+int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                  int transpose, int rht, void *y, int64_t ldy, float *amax,
+                  void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * Fused quantize -> dequantize round trip: out[rows, cols] (bf16, leading dimension ldo) =
  * the values fos_dequantize would return for fos_quantize's result, without materialising
  * codes or scales.  Stands in for QuantizeBackendBase.pseudo_quantize

@@ -137,10 +137,48 @@ def pad_bits(xb: np.ndarray) -> np.ndarray:
     return out
 
 
+# Hard-coded sign vector and Sylvester-ordered 16-point Hadamard matrix of the reference's
+# random Hadamard transform (src/fouroversix/quantize/utils.py:19-85): RHT = diag(signs) @ H / 4.
+RHT_SIGNS = np.array([1, 1, 1, -1, 1, -1, -1, -1, -1, -1, -1, 1, -1, 1, -1, -1], dtype=np.float32)
+
+
+def rht_matrix() -> np.ndarray:
+    idx = np.arange(16)
+    had = np.array([[(-1.0) ** bin(i & j).count("1") for j in idx] for i in idx], dtype=np.float32)
+    return (RHT_SIGNS[:, None] * had * np.float32(0.25)).astype(np.float32)
+
+
+def f32_to_bf16_bits(f: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(f, dtype=np.float32).view(np.uint32)
+    return ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+
+
+def transform(xb: np.ndarray, *, transpose=False, rht=False) -> np.ndarray:
+    """bf16 bits of the tensor the reference quantizes when ``transpose`` / ``rht`` are set
+    (src/fouroversix/quantize/pytorch/reference.py:567-571): ``x.T``, then every group of 16
+    consecutive elements of a row times the RHT matrix as a bf16 matmul, i.e. exact
+    products, fp32 accumulation (here in the order i = 0..15), one rounding to bf16."""
+    xb = np.asarray(xb, dtype=np.uint16)
+    if transpose:
+        xb = np.ascontiguousarray(xb.T)
+    if rht:
+        assert xb.shape[1] % 16 == 0
+        g = bf16_bits_to_f32(xb).reshape(-1, 16)
+        h = rht_matrix()
+        acc = np.zeros_like(g)
+        for i in range(16):
+            acc = acc + g[:, i:i + 1] * h[i][None, :]
+        xb = f32_to_bf16_bits(acc).reshape(xb.shape)
+    return xb
+
+
 def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
-             block_scale_2d=False, seed=0, offset=0, threads=None) -> OracleQuantized:
+             block_scale_2d=False, seed=0, offset=0, threads=None,
+             transpose=False, rht=False) -> OracleQuantized:
     xb = bf16_bits(x)
     assert xb.ndim == 2
+    if transpose or rht:
+        xb = transform(xb, transpose=transpose, rht=rht)
     orig = tuple(int(v) for v in xb.shape)
     xp = np.ascontiguousarray(pad_bits(xb))
     mp, np_ = xp.shape

@@ -97,15 +97,56 @@ QUANT_CONFIGS = [
 ] + [("if4", rule, two_d) for rule in ("mse", "mae", "abs_max") for two_d in (False, True)]
 
 
+def write_transform_vectors() -> None:
+    """transpose / random-Hadamard options of the reference quantizer
+    (quantize/pytorch/reference.py:567-571).  Its backend wrapper builds the Hadamard
+    matrix on "cuda" (quantize/utils.py:68-85 default), which this container lacks, so the
+    reference function is called directly with the CPU matrix; shapes are multiples of
+    (128, 64) in both orientations, for which the wrapper adds no padding."""
+    from fouroversix.quantize.pytorch.reference import quantize as ref_quantize  # noqa: PLC0415
+    from fouroversix.quantize.utils import get_rht_matrix  # noqa: PLC0415
+    from fouroversix.utils import DataType, RoundStyle, ScaleRule  # noqa: PLC0415
+
+    had = get_rht_matrix(device="cpu")
+    out: dict[str, np.ndarray] = {"had": bits(had)}
+    for name, kind, shape, seed in [
+        ("randn_256x128", "randn", (256, 128), 31),
+        ("outlier_128x256", "outlier", (128, 256), 32),
+        ("tiny_blocks_128x128", "tiny_blocks", (128, 128), 33),
+    ]:
+        x = make_input(kind, shape, seed)
+        out[f"{name}.x"] = bits(x)
+        for transpose in (False, True):
+            for rht in (False, True):
+                if not transpose and not rht:
+                    continue
+                for rule, two_d in (("mse", False), ("static_6", False), ("mse", True)):
+                    v, sf, amax = ref_quantize(
+                        x.clone(), had=had if rht else None, fp4_format=DataType.nvfp4,
+                        round_style=RoundStyle.nearest, scale_rule=ScaleRule(rule), block_scale_2d=two_d,
+                        transpose=transpose, use_blackwell_scale_layout=True,
+                    )
+                    key = f"{name}.t{int(transpose)}.h{int(rht)}.{rule}.{'2d' if two_d else '1d'}"
+                    out[key + ".values"] = u8(v)
+                    out[key + ".sf"] = u8(sf)
+                    out[key + ".amax"] = np.array([float(amax)], dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "transform.npz"), **out)
+    print("wrote transform", len(out))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
+    ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
     args = ap.parse_args()
 
     fos = import_reference()
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_transform_vectors()
+    if args.only_transform:
+        return
 
     # ---- quantize + dequantize ------------------------------------------------------
     for name, kind, shape, seed in QUANT_INPUTS:

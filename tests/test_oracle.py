@@ -52,6 +52,30 @@ def test_quantize_config1_digest(oracle, golden_dir):
         assert hashlib.sha256(q.scale_factors.tobytes()).hexdigest() == str(d[f"{rule}.sf_sha"])
 
 
+def test_transform_options_match_reference_vectors(oracle, golden_dir):
+    """transpose / random-Hadamard options (reference quantize/pytorch/reference.py:567-571):
+    vectors written by the reference function on CPU, all three combinations, 1-D and 2-D;
+    the RHT matrix itself is pinned against the reference's bf16 matrix."""
+    d = np.load(os.path.join(golden_dir, "transform.npz"))
+    assert np.array_equal(oracle.f32_to_bf16_bits(oracle.rht_matrix()), d["had"])
+    # symmetric up to the sign vector, orthonormal: H H^T = I
+    h = oracle.rht_matrix()
+    assert np.array_equal(h @ h.T, np.eye(16, dtype=np.float32))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        name, t, hh, rule, dim = key[: -len(".values")].split(".")
+        x = d[f"{name}.x"]
+        q = oracle.quantize(x, scale_rule=rule, block_scale_2d=(dim == "2d"), transpose=(t == "t1"), rht=(hh == "h1"))
+        base = key[: -len(".values")]
+        assert np.array_equal(q.values, d[base + ".values"]), base
+        assert np.array_equal(q.scale_factors, d[base + ".sf"].reshape(-1)), base
+        assert q.amax == d[base + ".amax"][0], base
+        n += 1
+    assert n == 27
+
+
 def test_dequantize_matches_reference_vectors(oracle, golden_dir):
     for name in ("randn_256x128", "ragged_100x80", "tiny_blocks_128x128"):
         d = np.load(os.path.join(golden_dir, f"quantize_{name}.npz"))

@@ -281,3 +281,67 @@ def test_pseudo_quantize_full_size():
     once = fos.quantize(x, s6)
     # by value: a -0.0 (a negative input that rounded to zero) re-quantizes to +0.0
     assert torch.equal(fos.quantize(once, s6), once)
+
+
+# ---- transpose / random Hadamard transform ------------------------------------------------
+
+def test_transform_options_match_reference_vectors(golden_dir):
+    """config.transpose / config.rht against the vectors the reference function wrote
+    (quantize/pytorch/reference.py:567-571): codes, scales and amax, bit for bit."""
+    d = np.load(os.path.join(golden_dir, "transform.npz"))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        base = key[: -len(".values")]
+        name, t, hh, rule, dim = base.split(".")
+        x = torch.from_numpy(d[f"{name}.x"].view(np.int16).copy()).view(torch.bfloat16).cuda()
+        q = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, block_scale_2d=(dim == "2d"),
+                                                   transpose=(t == "t1"), rht=(hh == "h1")))
+        assert tuple(q.original_shape) == (tuple(x.shape)[::-1] if t == "t1" else tuple(x.shape))
+        assert np.array_equal(u8(q.values), d[base + ".values"]), base
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), d[base + ".sf"].reshape(-1)), base
+        assert float(q.amax) == float(d[base + ".amax"][0]), base
+        n += 1
+    assert n == 27
+
+
+@pytest.mark.parametrize(("transpose", "rht"), [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize(("kind", "shape"), [("randn", (1024, 2048)), ("outlier", (272, 144)), ("tiny_blocks", (48, 400)),
+                                             ("zeros", (64, 64))])
+def test_transform_matches_oracle(oracle, kind, shape, transpose, rht):
+    """fos_transform (through ops.transform) and the quantization that follows it, against
+    the oracle's restatement, on shapes that are not multiples of (128, 64) or of the
+    64 x 64 transposition tile."""
+    from fouroversix_amd.quantize import ops
+
+    x = make_input(kind, shape, 21)
+    y, amax = ops.transform(x.cuda(), transpose, rht)
+    ref_y = oracle.transform(bits16(x), transpose=transpose, rht=rht)
+    assert np.array_equal(bits16(y), ref_y)
+    assert float(amax) == float(np.abs(oracle.bf16_bits_to_f32(ref_y)).max())
+    for rule, two_d in (("mse", False), ("static_6", True)):
+        q = hip_quantize(x, scale_rule=rule, block_scale_2d=two_d, transpose=transpose, rht=rht)
+        ref = oracle.quantize(x, scale_rule=rule, block_scale_2d=two_d, transpose=transpose, rht=rht)
+        assert_same_quantization(q, ref, f"{kind} t={transpose} h={rht} {rule}")
+
+
+def test_transform_properties_full_size():
+    """8192 x 8192: the RHT matrix is orthonormal up to bf16 rounding (energy preserved to
+    1e-3), transposing twice is the identity, and unsupported shapes are refused."""
+    from fouroversix_amd.quantize import ops
+
+    x = make_input("randn", (8192, 8192), 2).cuda()
+    y, amax = ops.transform(x, False, True)
+    assert abs(float(y.float().pow(2).sum() / x.float().pow(2).sum()) - 1.0) < 1e-3
+    assert float(amax) == float(y.abs().max())
+    t, amax_t = ops.transform(x, True, False)
+    assert torch.equal(t, x.T) and float(amax_t) == float(x.abs().max())
+    tt, _ = ops.transform(t, True, False)
+    assert torch.equal(tt, x)
+    th, _ = ops.transform(x, True, True)
+    assert torch.equal(th, ops.transform(t, False, True)[0])
+    with pytest.raises(ValueError, match="multiples of 16"):
+        fos.quantize(x[:, :200], fos.QuantizationConfig(rht=True))
+    with pytest.raises(ValueError, match="multiples of 16"):
+        fos.quantize(x[:100], fos.QuantizationConfig(transpose=True))
