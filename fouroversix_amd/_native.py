@@ -31,6 +31,8 @@ EXPORTS = (
     "fos_pseudo_quantize",
     "fos_transform",
     "fos_gemm_nvfp4",
+    "fos_gemm_mxfp4",
+    "fos_padded_cols_for",
     "fos_gemm_workspace_bytes",
     "fos_dequantize",
 )
@@ -76,6 +78,10 @@ def lib() -> ctypes.CDLL:
     L.fos_transform.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
+    L.fos_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp]
+    L.fos_gemm_mxfp4.restype = i32
+    L.fos_padded_cols_for.argtypes = [i32, i64]
+    L.fos_padded_cols_for.restype = i64
     L.fos_gemm_workspace_bytes.argtypes = [i64, i64, i64]
     L.fos_gemm_workspace_bytes.restype = ctypes.c_size_t
     L.fos_dequantize.argtypes = [vp, vp, vp, i32, i32, dbl, i64, i64, i64, i64, vp, i32, i64, vp]

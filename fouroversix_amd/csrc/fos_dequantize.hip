@@ -111,6 +111,12 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
 
 }  // namespace fos
 
+namespace fos {
+// MXFP4 (fos_mxfp4.hip)
+int launch_dequantize_mxfp4(const uint8_t *codes, const uint8_t *sf, int sf_layout, int64_t rows, int64_t cols,
+                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, hipStream_t s);
+}  // namespace fos
+
 using namespace fos;
 
 namespace {
@@ -126,7 +132,14 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
                               int dtype, int sf_layout, double divisor,
                               int64_t rows, int64_t cols, int64_t rows_p, int64_t cols_p,
                               void *out, int out_type, int64_t ldo, fos_stream_t stream) {
-    if (!codes || !sf || !amax || !out) return FOS_E_NULL_POINTER;
+    if (!codes || !sf || !out || (!amax && dtype != FOS_DTYPE_MXFP4)) return FOS_E_NULL_POINTER;
+    if (dtype == FOS_DTYPE_MXFP4) {
+        if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || ldo < cols) return FOS_E_BAD_SHAPE;
+        if (sf_layout == FOS_SF_TILED_128X4 && rows_p % 128 != 0) return FOS_E_BAD_SHAPE;
+        if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
+        if (out_type != FOS_T_BF16 && out_type != FOS_T_F16 && out_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
+        return launch_dequantize_mxfp4(codes, sf, sf_layout, rows, cols, rows_p, cols_p, out, out_type, ldo, (hipStream_t)stream);
+    }
     if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || cols_p % 16 != 0 || ldo < cols) return FOS_E_BAD_SHAPE;
     if (sf_layout == FOS_SF_TILED_128X4 && (rows_p % 128 != 0 || cols_p % 64 != 0)) return FOS_E_BAD_SHAPE;
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;

@@ -1,0 +1,506 @@
+// gfx950 MXFP4: E2M1 codes with one E8M0 (power-of-two) scale per 1x32 block, no tensor
+// scale (OCP microscaling).  Three kernels:
+//
+//  * quantize: one streaming pass (there is no tensor maximum to find first) with the
+//    arithmetic of quantize_to_mxfp4 + fake_quantize_to_e2m1
+//    (src/fouroversix/quantize/pytorch/reference.py:30-51, 149-181): scale = the block
+//    maximum over qmax rounded UP to a power of two, values divided by it (exact) and
+//    rounded to the E2M1 grid, half to even.
+//  * dequantize: the mx branch of QuantizeBackendBase.dequantize
+//    (src/fouroversix/quantize/backend.py:89-160): value and scale meet in fp16.
+//  * GEMM: this is the one format the matrix cores take natively --
+//    v_mfma_scale_f32_32x32x64_f8f6f4 multiplies packed FP4 operands and applies one E8M0
+//    scale per row and 32-wide K block, exactly the MX block -- so packed codes go
+//    global -> LDS -> MFMA without any conversion, at four times the fp16 MFMA rate.
+//    Stands in for gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt
+//    (src/fouroversix/csrc/bindings.cpp:26-35, src/fouroversix/matmul/cutlass/backend.py:79-110).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fos_quantize_fast.h"
+#include "fouroversix_hip.h"
+
+namespace fos {
+
+// ---------------------------------------------------------------------------------------
+// quantize
+// ---------------------------------------------------------------------------------------
+
+struct MxQuantParams {
+    const uint16_t *x;
+    int64_t rows, cols, ld;
+    int64_t rows_p, cols_p;  // rows to 128, cols to 128
+    uint8_t *codes;          // [rows_p, cols_p / 2]
+    uint8_t *sf;             // rows_p * cols_p / 32 E8M0 bytes
+    float qmax;              // 6 or 4
+    int sf_layout;
+    int tiles_x;
+    int vector_loads;        // x 16-byte aligned, ld % 8 == 0
+};
+
+struct Block32 {
+    uint32_t w[16];
+};
+
+// Codes (4 words) and scale byte of one 1x32 block.
+FOS_DEVICE void quantize_block_mxfp4(const Block32 &b, float qmax, uint4 &codes, uint32_t &e) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) m = pk_max_u16(m, b.w[i] & 0x7fff7fffu);
+    const uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    const float s_hp = u2f(mm << 16) / qmax;
+    const uint32_t u = f2u(s_hp);
+    e = (u >> 23) & 0xffu;
+    if (u & 0x7fffffu) e = (e + 1u) & 0xffu;  // round up to the next power of two
+    // 1 / 2^(e - 127); e == 0 marks an all-zero block (values become 0), 255 is inf / NaN
+    const float inv = e == 0u || e == 255u ? 0.0f : (e == 254u ? u2f(0x00400000u) : u2f((254u - e) << 23));
+    uint32_t c[4] = {0, 0, 0, 0};
+    static_for<0, 16>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        // + 0: the reference multiplies by sign(x) with sign(-0.0) = 0, so a negative zero
+        // (also one produced by underflow) must not keep its sign; a negative value that
+        // rounds to zero does
+        const float lo = __builtin_fmaf(u2f(b.w[j] << 16), inv, 0.0f);
+        const float hi = __builtin_fmaf(u2f(b.w[j] & 0xffff0000u), inv, 0.0f);
+        c[j >> 2] = pack_fp4<(j & 3)>(c[j >> 2], lo, hi);
+    });
+    codes = make_uint4(c[0], c[1], c[2], c[3]);
+}
+
+// Workgroup tile 128 rows x 512 columns (16 blocks): a wavefront covers 4 rows x 16
+// blocks = 1 KiB contiguous per row; eight steps of 16 rows; the four complete 128x4 scale
+// tiles are staged in LDS and leave as one contiguous 2 KiB run.
+__global__ __launch_bounds__(kThreads) void quantize_mxfp4_kernel(const MxQuantParams p) {
+    __shared__ uint32_t sf_stage[4 * 128];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lb = lane & 15, rr0 = wave * 4 + (lane >> 4);
+    const int64_t sf_cols = p.cols_p >> 5;
+    const int64_t tile_y = blockIdx.x / p.tiles_x, tile_x = blockIdx.x - tile_y * p.tiles_x;
+    const int64_t cb = tile_x * 16 + lb;
+    const bool col_ok = cb < sf_cols;
+    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    const int64_t row0 = tile_y * 128 + rr0;
+
+    auto load = [&](int g, Block32 &b) {
+        const int64_t r = row0 + g * 16, c0 = cb * 32;
+        if (r < p.rows && c0 + 32 <= p.cols && p.vector_loads) {
+            const uint4 *q = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint4 t = q[v];
+                b.w[4 * v] = t.x; b.w[4 * v + 1] = t.y; b.w[4 * v + 2] = t.z; b.w[4 * v + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                uint32_t lo = 0, hi = 0;
+                if (r < p.rows && c0 + 2 * i < p.cols) lo = p.x[r * p.ld + c0 + 2 * i];
+                if (r < p.rows && c0 + 2 * i + 1 < p.cols) hi = p.x[r * p.ld + c0 + 2 * i + 1];
+                b.w[i] = lo | (hi << 16);
+            }
+        }
+    };
+
+    Block32 blk[2];
+    load(0, blk[0]);
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        if (g + 1 < 8) load(g + 1, blk[(g + 1) & 1]);
+        if (col_ok) {
+            uint4 codes;
+            uint32_t e;
+            quantize_block_mxfp4(blk[g & 1], p.qmax, codes, e);
+            const int rr = g * 16 + rr0;
+            *reinterpret_cast<uint4 *>(p.codes + (row0 + g * 16) * (p.cols_p >> 1) + cb * 16) = codes;
+            if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
+            else p.sf[(row0 + g * 16) * sf_cols + cb] = (uint8_t)e;
+        }
+    }
+    if (tiled) {
+        __syncthreads();
+        const int t = threadIdx.x >> 6;  // scale tile of this wavefront: 512 bytes, 8 per lane
+        const int64_t group = tile_x * 4 + t;
+        if (group < (sf_cols >> 2)) {
+            uint2 *out = reinterpret_cast<uint2 *>(p.sf + (tile_y * (sf_cols >> 2) + group) * 512);
+            out[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
+        }
+    }
+}
+
+__global__ void set_one_kernel(float *amax) { *amax = 1.0f; }
+
+int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
+                          uint8_t *sf, float *amax, hipStream_t s) {
+    MxQuantParams p;
+    p.x = static_cast<const uint16_t *>(x);
+    p.rows = rows; p.cols = cols; p.ld = ld;
+    p.rows_p = (rows + 127) / 128 * 128;
+    p.cols_p = (cols + 127) / 128 * 128;
+    p.codes = codes; p.sf = sf;
+    p.qmax = rule == FOS_RULE_STATIC_4 ? 4.0f : 6.0f;
+    p.sf_layout = sf_layout;
+    p.tiles_x = (int)((p.cols_p + 511) / 512);
+    p.vector_loads = (((uintptr_t)x & 15) == 0) && (ld % 8 == 0);
+    const int64_t grid = (p.rows_p / 128) * p.tiles_x;
+    if (grid > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    hipLaunchKernelGGL(quantize_mxfp4_kernel, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    // the format has no tensor scale; the reference reports amax = 1 (reference.py:573-578)
+    hipLaunchKernelGGL(set_one_kernel, dim3(1), dim3(1), 0, s, amax);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------
+// dequantize
+// ---------------------------------------------------------------------------------------
+
+struct MxDequantParams {
+    const uint8_t *codes, *sf;
+    void *out;
+    int64_t rows, cols, rows_p, cols_p, ldo;
+    int sf_layout;
+    int vector_stores;
+};
+
+typedef _Float16 mx_half2_t __attribute__((ext_vector_type(2)));
+
+// One thread per 1x32 block.  value (fp16) * fp16(2^(e - 127)), product in fp16: scales
+// outside fp16's range turn into 0 / inf there, as in the reference.
+template <int OUT>
+__global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantParams p) {
+    const int64_t sf_cols = p.cols_p >> 5;
+    const int64_t bpr = (p.cols + 31) >> 5;
+    const int64_t blk = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (blk >= p.rows * bpr) return;
+    const int64_t r = blk / bpr, cb = blk - r * bpr;
+    const uint4 q = *reinterpret_cast<const uint4 *>(p.codes + r * (p.cols_p >> 1) + cb * 16);
+    const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
+                             ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
+                             : r * sf_cols + cb;
+    const uint32_t e = p.sf[sofs];
+    const _Float16 s16 = (_Float16)(e == 0u ? u2f(0x00400000u) : u2f(e << 23));
+    const mx_half2_t s2 = {s16, s16};
+    const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+    float f[32];
+    static_for<0, 16>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const mx_half2_t v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(words[j >> 2], 1.0f, j & 3) * s2;
+        f[2 * j] = (float)v.x;
+        f[2 * j + 1] = (float)v.y;
+    });
+    const int64_t c0 = cb * 32;
+    const bool whole = p.vector_stores && c0 + 32 <= p.cols;
+    if (OUT == FOS_T_F32) {
+        float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
+        if (whole) {
+#pragma unroll
+            for (int v = 0; v < 8; ++v) reinterpret_cast<float4 *>(o)[v] = make_float4(f[4 * v], f[4 * v + 1], f[4 * v + 2], f[4 * v + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                if (c0 + i < p.cols) o[i] = f[i];
+        }
+        return;
+    }
+    uint32_t w[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const float2_t v = {f[2 * j], f[2 * j + 1]};
+        if (OUT == FOS_T_F16) {
+            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
+        } else {
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+        }
+    }
+    uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
+    if (whole) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) reinterpret_cast<uint4 *>(o)[v] = make_uint4(w[4 * v], w[4 * v + 1], w[4 * v + 2], w[4 * v + 3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 32; ++i)
+            if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+    }
+}
+
+int launch_dequantize_mxfp4(const uint8_t *codes, const uint8_t *sf, int sf_layout, int64_t rows, int64_t cols,
+                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, hipStream_t s) {
+    if (cols_p % 32 != 0 || (sf_layout == FOS_SF_TILED_128X4 && cols_p % 128 != 0)) return FOS_E_BAD_SHAPE;
+    if ((uintptr_t)codes & 15) return FOS_E_BAD_ALIGNMENT;
+    MxDequantParams p;
+    p.codes = codes; p.sf = sf; p.out = out;
+    p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
+    p.sf_layout = sf_layout;
+    const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
+    p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
+    const int64_t n_blocks = rows * ((cols + 31) / 32);
+    if ((n_blocks + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    dim3 grid((unsigned)((n_blocks + 255) / 256));
+    if (out_type == FOS_T_F32) hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_F32>, grid, dim3(256), 0, s, p);
+    else if (out_type == FOS_T_F16) hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_F16>, grid, dim3(256), 0, s, p);
+    else hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_BF16>, grid, dim3(256), 0, s, p);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+// ---------------------------------------------------------------------------------------
+// GEMM on the scaled FP4 matrix instruction
+// ---------------------------------------------------------------------------------------
+//
+// D[M, N] = alpha * sum_k (A[m,k] 2^(sfA[m,k/32]-127)) (B[n,k] 2^(sfB[n,k/32]-127)).
+// Operand layout of v_mfma_scale_f32_32x32x64_f8f6f4 with FP4 inputs (probed on the
+// device): lane (r = lane & 31, h = lane >> 5) supplies the 32 codes k = 32 h .. 32 h + 31 of
+// row r (16 bytes, low nibble = even k) and, in one byte of a scale register, that row's
+// E8M0 scale for its K block; accumulator register 4 g + e of lane l is
+// C[8 g + 4 (l >> 5) + e][l & 31] with rows taken from the first operand.  B (rows n) is
+// fed as the first operand so that a lane's consecutive registers are consecutive n.
+//
+// Tile 256 x 256 x 128 (BK = 128 codes = 64 bytes per row = one scale chunk), 8 wavefronts
+// of 128 x 64, LDS pitch 80 bytes (conflict-free 128-bit accesses), two stages; the
+// pipeline is the one of the NVFP4 kernel minus the dequantisation: registers hold step
+// k+2 in flight, step k+1 goes to LDS in halves while step k is multiplied.  Scales bypass
+// LDS: the 128x4 tiled layout holds the four scale bytes of a 128-wide K chunk of rows r,
+// r+32, r+64, r+96 next to each other, so a wavefront's lanes fetch one 32-bit word per
+// row tile and chunk straight from global memory.
+
+typedef int mx_v8i __attribute__((ext_vector_type(8)));
+typedef float mx_v16f __attribute__((ext_vector_type(16)));
+typedef __amdgpu_buffer_rsrc_t MxRsrc;
+
+struct MxGemmParams {
+    const uint8_t *A, *B, *sfA, *sfB;
+    const float *alpha;
+    void *D;
+    int64_t M, N, K, ldd;
+    int tiles_m, tiles_n;
+};
+
+constexpr int kMxBK = 128;    // codes per K step
+constexpr int kMxPitch = 80;  // LDS bytes per row (64 + 16)
+
+FOS_DEVICE MxRsrc mx_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+FOS_DEVICE mx_v8i frag_of(const uint4 &q) {
+    mx_v8i v = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};  // FP4 operands use the first four registers
+    return v;
+}
+
+FOS_DEVICE void mx_tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
+    // workgroups with equal bid % 8 share an XCD: give each XCD a compact run of tiles,
+    // ordered in column bands of 8 tile rows
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    int t = (bid & 7) * per_xcd + (bid >> 3);
+    if (t >= total || (total & 7) != 0) t = bid;
+    constexpr int kBand = 8;
+    const int band = t / (kBand * tiles_n), in_band = t - band * kBand * tiles_n;
+    const int rows = (tiles_m - band * kBand) < kBand ? (tiles_m - band * kBand) : kBand;
+    tm = band * kBand + in_band % rows;
+    tn = in_band / rows;
+}
+
+template <int WAVES_M, int WAVES_N, int WM, int WN, bool OUT_BF16>
+__global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const MxGemmParams p) {
+    constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
+    constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+    constexpr int kRowsPerPass = kThreadsG / 4;  // 4 lanes cover the 64 bytes of a row
+    constexpr int PA = BM / kRowsPerPass, PB = BN / kRowsPerPass;
+    static_assert(PA == 2 && PB == 2 && WM * 32 <= 128 && WN * 32 <= 128, "tile shape: staged in two halves");
+    extern __shared__ __attribute__((aligned(16))) uint8_t mx_lds[];
+    uint8_t *lds_a[2] = {mx_lds, mx_lds + (BM + BN) * kMxPitch};
+    uint8_t *lds_b[2] = {mx_lds + BM * kMxPitch, mx_lds + (BM + BN) * kMxPitch + BM * kMxPitch};
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    int tile_m, tile_n;
+    mx_tile_of(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int64_t kbytes = p.K >> 1;
+    const int64_t ksteps = p.K / kMxBK;  // = 128-wide K chunks = scale groups per band
+
+    const MxRsrc ra = mx_rsrc(p.A + m0 * kbytes, (uint32_t)(BM * kbytes));
+    const MxRsrc rb = mx_rsrc(p.B + n0 * kbytes, (uint32_t)(BN * kbytes));
+    const int ld_row = tid >> 2, ld_col = (tid & 3) * 16;
+    const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_col);
+    const uint32_t lds_off = (uint32_t)(ld_row * kMxPitch + ld_col);
+
+    // scales of this wavefront's rows, straight from global memory
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int64_t a_row0 = m0 + wm * WM * 32, b_row0 = n0 + wn * WN * 32;
+    const MxRsrc rsa = mx_rsrc(p.sfA + (a_row0 >> 7) * ksteps * 512, (uint32_t)(ksteps * 512));
+    const MxRsrc rsb = mx_rsrc(p.sfB + (b_row0 >> 7) * ksteps * 512, (uint32_t)(ksteps * 512));
+    const uint32_t sa_off = (uint32_t)(r * 16 + ((a_row0 & 127) >> 5) * 4);
+    const uint32_t sb_off = (uint32_t)(r * 16 + ((b_row0 & 127) >> 5) * 4);
+
+    struct Staged {
+        uint4 a[PA], b[PB];
+    };
+    struct Scales {
+        uint32_t a[WM], b[WN];  // scale bytes of the step's four K blocks, per row tile
+    };
+    auto fetch = [&](int64_t ks, Staged &s) {
+        const int kq = (int)(ks * (kMxBK / 2));
+#pragma unroll
+        for (int i = 0; i < PA; ++i)
+            s.a[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)(q_off + i * kRowsPerPass * kbytes), kq, 0));
+#pragma unroll
+        for (int i = 0; i < PB; ++i)
+            s.b[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(q_off + i * kRowsPerPass * kbytes), kq, 0));
+    };
+    // lanes of the upper half shift their word by one byte, so that byte 0 / byte 2 of every
+    // lane's register are the scales of the K blocks it feeds in slice 0 / slice 1
+    auto fetch_scales = [&](int64_t ks, Scales &s) {
+        const int ksf = (int)(ks * 512);
+#pragma unroll
+        for (int i = 0; i < WM; ++i) s.a[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)(sa_off + i * 4), ksf, 0) >> (8 * h);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) s.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)(sb_off + j * 4), ksf, 0) >> (8 * h);
+    };
+    // half q of the staged registers -> LDS stage `buf`
+    auto stage_part = [&](const Staged &s, int buf, int q) {
+        *reinterpret_cast<uint4 *>(lds_a[buf] + lds_off + q * kRowsPerPass * kMxPitch) = s.a[q];
+        *reinterpret_cast<uint4 *>(lds_b[buf] + lds_off + q * kRowsPerPass * kMxPitch) = s.b[q];
+    };
+
+    mx_v16f acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    auto read_frags = [&](int buf, int kk, uint4 *fa, uint4 *fb) {
+        const int kofs = kk * 32 + h * 16;
+#pragma unroll
+        for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const uint4 *>(lds_a[buf] + (wm * WM * 32 + i * 32 + r) * kMxPitch + kofs);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const uint4 *>(lds_b[buf] + (wn * WN * 32 + j * 32 + r) * kMxPitch + kofs);
+    };
+
+    Staged st[2];
+    Scales sc[2];
+    uint4 fa[2][WM], fb[2][WN];
+    fetch(0, st[0]);
+    fetch_scales(0, sc[0]);
+    stage_part(st[0], 0, 0);
+    stage_part(st[0], 0, 1);
+    if (ksteps > 1) fetch(1, st[1]);
+    __syncthreads();
+    read_frags(0, 0, fa[0], fb[0]);
+
+    // One K step: multiply out of stage `buf` (fragments of slice 0 are in registers) while
+    // step ks+1 (`nxt`) goes to the other stage; the barrier sits between the last staging
+    // write and the last slice's MFMAs, and the next step's first fragments are read right
+    // after it.  Branch-free; the last step is its own instantiation.
+    auto kstep = [&](auto have_next_c, int64_t ks, int buf, Staged &cur_regs, Staged &nxt, const Scales &s_cur, Scales &s_nxt) {
+        constexpr bool have_next = decltype(have_next_c)::value;
+        if (have_next) {
+            fetch(ks + 2 < ksteps ? ks + 2 : ksteps - 1, cur_regs);
+            fetch_scales(ks + 1, s_nxt);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+            if (kk == 0) read_frags(buf, 1, fa[1], fb[1]);
+            if (have_next) {
+                stage_part(nxt, buf ^ 1, kk);
+                if (kk == 1) {
+                    __syncthreads();
+                    read_frags(buf ^ 1, 0, fa[0], fb[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j) {
+                    if (kk == 1)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            frag_of(fb[1][j]), frag_of(fa[1][i]), acc[i][j], 4, 4, 2, (int)s_cur.b[j], 2, (int)s_cur.a[i]);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            frag_of(fb[0][j]), frag_of(fa[0][i]), acc[i][j], 4, 4, 0, (int)s_cur.b[j], 0, (int)s_cur.a[i]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    using yes = std::integral_constant<bool, true>;
+    using no = std::integral_constant<bool, false>;
+    int64_t ks = 0;
+    for (; ks + 2 < ksteps; ks += 2) {
+        kstep(yes{}, ks, 0, st[0], st[1], sc[0], sc[1]);
+        kstep(yes{}, ks + 1, 1, st[1], st[0], sc[1], sc[0]);
+    }
+    if (ks + 2 == ksteps) {
+        kstep(yes{}, ks, 0, st[0], st[1], sc[0], sc[1]);
+        kstep(no{}, ks + 1, 1, st[1], st[0], sc[1], sc[0]);
+    } else {
+        kstep(no{}, ks, 0, st[0], st[1], sc[0], sc[1]);
+    }
+
+    const float alpha = *p.alpha;
+    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int64_t m = m0 + wm * WM * 32 + i * 32 + r;
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * h;
+                uint32_t w[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float2_t v = {alpha * acc[i][j][4 * g + 2 * e], alpha * acc[i][j][4 * g + 2 * e + 1]};
+                    if (OUT_BF16) {
+                        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+                    } else {
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
+                    }
+                }
+                *reinterpret_cast<uint2 *>(D + m * p.ldd + n) = make_uint2(w[0], w[1]);
+            }
+        }
+    }
+}
+
+template <int WAVES_M, int WAVES_N, int WM, int WN>
+static int launch_gemm_mxfp4(MxGemmParams &p, int out_type, hipStream_t s) {
+    constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
+    constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * kMxPitch;
+    p.tiles_m = (int)(p.M / BM);
+    p.tiles_n = (int)(p.N / BN);
+    auto kernel = out_type == FOS_T_BF16 ? gemm_mxfp4_kernel<WAVES_M, WAVES_N, WM, WN, true>
+                                         : gemm_mxfp4_kernel<WAVES_M, WAVES_N, WM, WN, false>;
+    if (lds_bytes > 64 * 1024 &&
+        hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+        return FOS_E_LAUNCH;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(64 * WAVES_M * WAVES_N), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+}  // namespace fos
+
+using namespace fos;
+
+extern "C" int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                              const float *alpha, int64_t M, int64_t N, int64_t K,
+                              void *D, int out_type, int64_t ldd, fos_stream_t stream) {
+    if (!A || !B || !sfA || !sfB || !alpha || !D) return FOS_E_NULL_POINTER;
+    if (M <= 0 || N <= 0 || K <= 0 || M % 128 != 0 || N % 128 != 0 || K % 128 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
+    if (out_type != FOS_T_BF16 && out_type != FOS_T_F16) return FOS_E_UNSUPPORTED;
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 15) || ((uintptr_t)sfB & 15) ||
+        ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
+        return FOS_E_BAD_ALIGNMENT;
+    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 24)) return FOS_E_BAD_SHAPE;
+    MxGemmParams p;
+    p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
+    p.M = M; p.N = N; p.K = K; p.ldd = ldd;
+    hipStream_t s = (hipStream_t)stream;
+    const bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256;
+    if (big) return launch_gemm_mxfp4<2, 4, 4, 2>(p, out_type, s);
+    return launch_gemm_mxfp4<2, 2, 2, 2>(p, out_type, s);
+}

@@ -110,6 +110,10 @@ using namespace fos;
 
 extern "C" int64_t fos_padded_rows(int64_t rows) { return (rows + 127) / 128 * 128; }
 extern "C" int64_t fos_padded_cols(int64_t cols) { return (cols + 63) / 64 * 64; }
+extern "C" int64_t fos_padded_cols_for(int dtype, int64_t cols) {
+    const int64_t mult = dtype == FOS_DTYPE_MXFP4 ? 128 : 64;  // four blocks of 32 / of 16
+    return (cols + mult - 1) / mult * mult;
+}
 
 extern "C" size_t fos_quantize_workspace_bytes(int64_t, int64_t) { return 2 * kMaxPartials * sizeof(uint32_t); }
 
@@ -179,6 +183,16 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
                          void *workspace, size_t workspace_bytes, fos_stream_t stream,
                          uint16_t *pseudo_out, int64_t ldo) {
     if (!x || !amax || (!pseudo_out && (!codes || !sf))) return FOS_E_NULL_POINTER;
+    if (dtype == FOS_DTYPE_MXFP4) {
+        // one streaming kernel; no tensor maximum, no workspace
+        if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
+        if (x_type != FOS_T_BF16 || pseudo_out || block2d || round_style != FOS_ROUND_NEAREST || amax_is_input ||
+            (rule != FOS_RULE_STATIC_6 && rule != FOS_RULE_STATIC_4))
+            return FOS_E_UNSUPPORTED;
+        if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
+        if (((uintptr_t)x & 1) || ((uintptr_t)codes & 15) || ((uintptr_t)sf & 7) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
+        return launch_quantize_mxfp4(x, rows, cols, ld, rule, sf_layout, codes, sf, amax, (hipStream_t)stream);
+    }
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if (x_type != FOS_T_BF16) return FOS_E_UNSUPPORTED;
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;

@@ -155,4 +155,8 @@ void launch_quantize(QuantParams &p, bool aligned, hipStream_t s) {
 // Defined in fos_quantize_fast.hip: NVFP4, round to nearest, any rule.
 void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s);
 
+// MXFP4 (fos_mxfp4.hip)
+int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
+                          uint8_t *sf, float *amax, hipStream_t s);
+
 }  // namespace fos

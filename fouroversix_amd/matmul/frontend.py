@@ -31,7 +31,7 @@ def is_supported(input: QuantizedTensor, other: QuantizedTensor, *, out_dtype: D
         raise ValueError(msg)
     return (
         input.dtype == other.dtype
-        and input.dtype == DataType.nvfp4
+        and input.dtype in (DataType.nvfp4, DataType.mxfp4)
         and input.device.type == "cuda"
         and out_dtype in (DataType.bfloat16, DataType.float16)
         and input.scale_factors_are_in_blackwell_layout
@@ -73,6 +73,16 @@ def quantized_matmul(
         else:
             msg = f"Backend {backend} does not support the given parameters"
         raise ValueError(msg)
+
+    out_shape = (input.original_shape[0], other.original_shape[0])
+    if input.dtype == DataType.mxfp4:
+        # no tensor scale: alpha = 1 (src/fouroversix/matmul/cutlass/backend.py:79-85)
+        alpha = torch.ones(1, dtype=torch.float32, device=input.values.device)
+        out = ops.gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(
+            input.values, other.values, input.scale_factors, other.scale_factors, alpha,
+            torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16,
+        )
+        return out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
 
     alpha = gemm_alpha(input, other)
     gemm = (

@@ -34,6 +34,8 @@ def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | Non
         return f"input must live on the GPU, got {x.device}"
     if x.dtype != torch.bfloat16:
         return f"input must be bfloat16, got {x.dtype}"
+    if config.dtype == DataType.mxfp4 and (config.block_scale_2d or config.round_style.is_stochastic):
+        return "mxfp4 has kernels for 1x32 blocks with round-to-nearest only"
     if config.rht or config.transpose:
         return ops.transform_unsupported_reason(x, config.transpose, config.rht)
     return None
@@ -107,7 +109,7 @@ def quantize(
         seed,
         offset,
         nat.SF_LINEAR if linear else nat.SF_TILED,
-        config.kwargs.get("amax"),
+        None if config.dtype == DataType.mxfp4 else config.kwargs.get("amax"),  # mxfp4 has no tensor scale
     )
     return QuantizedTensor(
         values,
@@ -144,10 +146,10 @@ def dequantize(
     scaled by ``amax / (qmax * smax * adjustment)`` and cast to ``dtype``.
     """
     del backend
-    if tensor.dtype.value not in NATIVE_FORMAT_IDS or tensor.dtype.scale_type == ScaleType.mx:
+    if tensor.dtype.value not in NATIVE_FORMAT_IDS:
         msg = f"No backend can dequantize {tensor.dtype.value}"
         raise ValueError(msg)
-    if tensor.amax is None:
+    if tensor.amax is None and tensor.dtype.scale_type != ScaleType.mx:
         msg = "dequantize needs the tensor-wide amax"
         raise ValueError(msg)
     if intermediate_dtype != torch.float16 and tensor.dtype != DataType.nvfp4:
@@ -157,13 +159,14 @@ def dequantize(
         msg = f"unsupported output dtype {dtype}"
         raise ValueError(msg)
     rows, cols = tensor.original_shape
+    amax = tensor.amax if tensor.amax is not None else torch.ones(1, dtype=torch.float32, device=tensor.values.device)
     return ops.dequantize(
         tensor.values,
         tensor.scale_factors,
-        tensor.amax,
+        amax,
         NATIVE_FORMAT_IDS[tensor.dtype.value],
         nat.SF_TILED if tensor.scale_factors_are_in_blackwell_layout else nat.SF_LINEAR,
-        float(dequantize_divisor(tensor)),
+        1.0 if tensor.dtype.scale_type == ScaleType.mx else float(dequantize_divisor(tensor)),
         rows,
         cols,
         dtype,

@@ -30,14 +30,19 @@ _LIB.define(
 )
 _LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
 _LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
+_LIB.define("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
 _LIB.define(
     "dequantize(Tensor values, Tensor scale_factors, Tensor amax, int dtype, int sf_layout, float divisor, "
     "int rows, int cols, ScalarType out_dtype) -> Tensor"
 )
 
 
-def _padded(rows: int, cols: int) -> tuple[int, int]:
-    return -(-rows // 128) * 128, -(-cols // 64) * 64
+MXFP4 = 2  # format id at the native boundary (blocks of 32, E8M0 scales)
+
+
+def _padded(rows: int, cols: int, dtype: int = 0) -> tuple[int, int]:
+    col_multiple = 128 if dtype == MXFP4 else 64  # four blocks
+    return -(-rows // 128) * 128, -(-cols // col_multiple) * col_multiple
 
 
 # Pass-1 workspace (8 KiB), one per (device, stream): calls on one stream are ordered, so
@@ -84,14 +89,17 @@ def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, s
         raise RuntimeError("quantize: x must be contiguous on the last dim")
     nat.require_gpu_tensor(x, "x")
     rows, cols = x.shape
-    rows_p, cols_p = _padded(rows, cols)
+    rows_p, cols_p = _padded(rows, cols, dtype)
     dev = x.device
     values = torch.empty(rows_p, cols_p // 2, dtype=torch.uint8, device=dev)
-    sf = torch.empty(rows_p * cols_p // 16, dtype=torch.float8_e4m3fn, device=dev)
+    if dtype == MXFP4:
+        sf = torch.empty(rows_p * cols_p // 32, dtype=torch.float8_e8m0fnu, device=dev)
+    else:
+        sf = torch.empty(rows_p * cols_p // 16, dtype=torch.float8_e4m3fn, device=dev)
     if rows == 0 or cols == 0:
         values.zero_()
         sf.view(torch.uint8).zero_()
-        return values, sf, torch.zeros(1, dtype=torch.float32, device=dev)
+        return values, sf, torch.full((1,), 1.0 if dtype == MXFP4 else 0.0, dtype=torch.float32, device=dev)
     L = nat.lib()
     amax_is_input = amax is not None
     amax_buf = (
@@ -240,6 +248,35 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
     return out
 
 
+def _gemm_mxfp4_impl(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):
+    """MXFP4 x MXFP4 GEMM on the scaled FP4 matrix instruction; checks as the NVFP4 op
+    (reference csrc/include/element_traits.hpp:122-170 with blocks of 32, E8M0 scales)."""
+    for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), ("alpha", alpha)):
+        nat.require_gpu_tensor(t, name)
+        if not t.is_contiguous():
+            raise RuntimeError(f"gemm: {name} must be contiguous")
+        if t.device != a.device:
+            raise RuntimeError("gemm: all operands must be on the same GPU")
+    if a.dtype != torch.uint8 or b.dtype != torch.uint8 or a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError("A and B must be 2D uint8")
+    if a_sf.dtype != torch.float8_e8m0fnu or b_sf.dtype != torch.float8_e8m0fnu:
+        raise RuntimeError("A_sf and B_sf must be Float8_e8m0fnu")
+    m, ka = a.shape[0], a.shape[1] * 2
+    n, kb = b.shape[0], b.shape[1] * 2
+    if ka != kb:
+        raise RuntimeError(f"Inner dims mismatch: {ka} vs {kb}")
+    if a_sf.numel() * 32 != m * ka or b_sf.numel() * 32 != n * kb:
+        raise RuntimeError("scale factor size mismatch")
+    out = torch.empty(m, n, dtype=out_dtype, device=a.device)
+    with _on_device(a.device):
+        rc = nat.lib().fos_gemm_mxfp4(
+            a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(),
+            m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n, nat.current_stream(a.device),
+        )
+    nat.check(rc, "fouroversix::gemm_mxfp4mxfp4_accum_fp32")
+    return out
+
+
 def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
     nat.require_gpu_tensor(values, "values")
     rows_p, cols_p = values.shape[0], values.shape[1] * 2
@@ -270,14 +307,16 @@ _LIB.impl(
     lambda a, b, a_sf, b_sf, alpha: _gemm_impl(a, b, a_sf, b_sf, alpha, torch.float16),
     "CUDA",
 )
+_LIB.impl("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt", _gemm_mxfp4_impl, "CUDA")
 _LIB.impl("dequantize", _dequantize_impl, "CUDA")
 
 
-def _fake_quantize_shapes(x):
-    rows_p, cols_p = _padded(x.shape[0], x.shape[1])
+def _fake_quantize_shapes(x, dtype=0):
+    rows_p, cols_p = _padded(x.shape[0], x.shape[1], dtype)
+    block, sf_dtype = (32, torch.float8_e8m0fnu) if dtype == MXFP4 else (16, torch.float8_e4m3fn)
     return (
         torch.empty(rows_p, cols_p // 2, dtype=torch.uint8, device=x.device),
-        torch.empty(rows_p * cols_p // 16, dtype=torch.float8_e4m3fn, device=x.device),
+        torch.empty(rows_p * cols_p // block, dtype=sf_dtype, device=x.device),
         torch.empty(1, dtype=torch.float32, device=x.device),
     )
 
@@ -289,7 +328,7 @@ def _(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
 
 @torch.library.register_fake("fouroversix::quantize_ex")
 def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
-    return _fake_quantize_shapes(x)
+    return _fake_quantize_shapes(x, dtype)
 
 
 @torch.library.register_fake("fouroversix::pseudo_quantize")
@@ -305,6 +344,11 @@ def _(a, b, a_sf, b_sf, alpha):
 @torch.library.register_fake("fouroversix::gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt")
 def _(a, b, a_sf, b_sf, alpha):
     return torch.empty(a.shape[0], b.shape[0], dtype=torch.float16, device=a.device)
+
+
+@torch.library.register_fake("fouroversix::gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt")
+def _(a, b, a_sf, b_sf, alpha):
+    return torch.empty(a.shape[0], b.shape[0], dtype=torch.bfloat16, device=a.device)
 
 
 @torch.library.register_fake("fouroversix::dequantize")
@@ -356,6 +400,13 @@ def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
     if _direct(a):
         return _gemm_impl(a, b, a_sf, b_sf, alpha, torch.float16)
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
+
+
+def gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):
+    """Same call as the reference's ``matmul/cutlass/ops.py:6-20`` (fp16 output as an extension)."""
+    if _direct(a):
+        return _gemm_mxfp4_impl(a, b, a_sf, b_sf, alpha, out_dtype)
+    return torch.ops.fouroversix.gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
 def dequantize(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):

@@ -245,4 +245,4 @@ DataType.supported_scale_rules = property(_rules)
 DataType.torch_dtype = property(_torch_dtype)
 
 # Formats that have a gfx950 kernel, with their id at the native boundary.
-NATIVE_FORMAT_IDS = {"nvfp4": 0, "if4": 1}
+NATIVE_FORMAT_IDS = {"nvfp4": 0, "if4": 1, "mxfp4": 2}

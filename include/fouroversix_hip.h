@@ -33,7 +33,7 @@ enum {
 };
 
 /* formats, mirroring DataType members of src/fouroversix/utils.py:13-41 */
-enum { FOS_DTYPE_NVFP4 = 0, FOS_DTYPE_IF4 = 1 };
+enum { FOS_DTYPE_NVFP4 = 0, FOS_DTYPE_IF4 = 1, FOS_DTYPE_MXFP4 = 2 };
 /* scale rules with the ids of ScaleRule.cuda_id, src/fouroversix/utils.py:271-280 and
  * csrc/quantize/fp4_quant.cu:111-119 */
 enum { FOS_RULE_STATIC_6 = 0, FOS_RULE_STATIC_4 = 1, FOS_RULE_MAE = 2, FOS_RULE_MSE = 3, FOS_RULE_ABS_MAX = 4 };
@@ -55,6 +55,8 @@ const char *fos_error_string(int code);
  * multiple of 64 (QuantizedTensor, src/fouroversix/quantize/quantized_tensor.py:65-78). */
 int64_t fos_padded_rows(int64_t rows);
 int64_t fos_padded_cols(int64_t cols);
+/* Same for a given format: FOS_DTYPE_MXFP4 (blocks of 32) pads columns to a multiple of 128. */
+int64_t fos_padded_cols_for(int dtype, int64_t cols);
 
 /* Bytes of device workspace fos_quantize needs for an [rows, cols] input (never 0). */
 size_t fos_quantize_workspace_bytes(int64_t rows, int64_t cols);
@@ -87,6 +89,12 @@ int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, 
  *   sf          u8 [rows_p * cols_p / 16] E4M3 bytes (IF4: bit 7 marks integer blocks)
  *   amax        f32[1]; written with max|x| unless amax_is_input, in which case it is read
  *   workspace   >= fos_quantize_workspace_bytes(rows, cols) bytes, 256-byte aligned
+ *
+ * FOS_DTYPE_MXFP4 (src/fouroversix/quantize/pytorch/reference.py:149-181): E2M1 codes with
+ * one E8M0 scale per 1x32 block, static rules and FOS_ROUND_NEAREST only, 1x32 blocks only;
+ * columns are padded to a multiple of 128 (fos_padded_cols_for), `sf` holds
+ * rows_p * cols_p / 32 bytes, amax is written with 1 (the format has no tensor scale) and
+ * the workspace is not used.
  */
 int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
                  int dtype, int rule, int round_style, int block2d,
@@ -153,11 +161,24 @@ int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const
 size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * MXFP4 counterpart of fos_gemm_nvfp4: D = alpha * sum_k (A 2^(sfA-127)) (B 2^(sfB-127)) on
+ * the native scaled FP4 matrix instruction.  Stands in for
+ * torch.ops.fouroversix.gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt
+ * (src/fouroversix/csrc/bindings.cpp:26-35, src/fouroversix/matmul/cutlass/backend.py:79-110).
+ *   A u8 [M, K/2], B u8 [N, K/2]; sfA, sfB E8M0 bytes in the FOS_SF_TILED_128X4 layout of
+ *   [M, K/32] / [N, K/32]; M, N, K multiples of 128 (the padded shapes fos_quantize produces).
+ */
+int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                   const float *alpha, int64_t M, int64_t N, int64_t K,
+                   void *D, int out_type, int64_t ldd, fos_stream_t stream);
+
+/*
  * out[rows, cols] = dequantized values of a quantized tensor, cropped to (rows, cols).
  * Stands in for QuantizeBackendBase.dequantize (src/fouroversix/quantize/backend.py:89-160).
  *   codes u8 [rows_p, cols_p/2], sf in sf_layout over [rows_p, cols_p/16], amax f32[1]
  *   divisor = qmax * smax * adjustment of the tensor's scale rule and rounding style
  *   out_type FOS_T_BF16 / FOS_T_F16 / FOS_T_F32, leading dimension ldo
+ * FOS_DTYPE_MXFP4: blocks of 32, E8M0 scales, amax and divisor are ignored (amax may be NULL).
  */
 int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const float *amax,
                    int dtype, int sf_layout, double divisor,

@@ -275,3 +275,75 @@ def gemm_nvfp4(values_a, sf_rows_a, values_b, sf_rows_b, alpha, threads=None):
 
 def bf16_bits_to_f32(bits: np.ndarray) -> np.ndarray:
     return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+# ---- MXFP4: E2M1 codes, one E8M0 scale per 1x32 block --------------------------------------
+# numpy restatement of quantize_to_mxfp4 + fake_quantize_to_e2m1 + the code packing
+# (src/fouroversix/quantize/pytorch/reference.py:30-51, 82-132, 149-181) and of the mx branch
+# of dequantize (src/fouroversix/quantize/backend.py:89-160).  Pinned by tests/golden/mxfp4.npz.
+
+E2M1_VALUES = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6], dtype=np.float32)
+
+
+def pad_bits_mx(xb: np.ndarray) -> np.ndarray:
+    """Zero-pad to rows % 128 == 0, cols % 128 == 0 (4 blocks of 32;
+    src/fouroversix/quantize/pytorch/backend.py:57-79)."""
+    m, n = xb.shape
+    out = np.zeros((-(-m // 128) * 128, -(-n // 128) * 128), dtype=np.uint16)
+    out[:m, :n] = xb
+    return out
+
+
+def quantize_mxfp4(x, *, scale_rule="static_6") -> OracleQuantized:
+    assert scale_rule in ("static_6", "static_4")
+    xb = bf16_bits(x)
+    orig = tuple(int(v) for v in xb.shape)
+    xp = pad_bits_mx(xb)
+    mp, np_ = xp.shape
+    blocks = bf16_bits_to_f32(xp).reshape(-1, 32)
+    qmax = np.float32(6.0 if scale_rule == "static_6" else 4.0)
+    s_hp = (np.abs(blocks).max(axis=1) / qmax).astype(np.float32)
+    u = s_hp.view(np.uint32)
+    e = ((u >> np.uint32(23)) & np.uint32(0xFF)).astype(np.uint8)
+    e = np.where((u & np.uint32(0x7FFFFF)) == 0, e, e + np.uint8(1)).astype(np.uint8)  # round up to a power of two
+    s = (e.astype(np.uint32) << np.uint32(23)).view(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        xs = np.where((e != 0)[:, None], blocks / s[:, None], np.float32(0)).astype(np.float32)
+    a = np.abs(xs)
+    r = np.where(a < 2, np.rint(a + a) * np.float32(0.5), np.where(a < 4, np.rint(a), np.float32(2) * np.rint(a * np.float32(0.5))))
+    fq = (r * np.sign(xs)).astype(np.float32)  # sign(+-0) = 0; a negative value rounding to zero gives -0.0
+    mag = np.searchsorted(E2M1_VALUES, np.abs(fq)).astype(np.uint8)
+    code = (mag | (np.signbit(fq).astype(np.uint8) << 3)).reshape(mp, np_)
+    values = (code[:, 0::2] | (code[:, 1::2] << 4)).astype(np.uint8)
+    sf_rows = e.reshape(mp, np_ // 32)
+    return OracleQuantized(values, to_blocked(sf_rows), sf_rows, np.float32(1.0), "mxfp4", scale_rule, "nearest",
+                           orig, (mp, np_), True)
+
+
+def dequantize_mxfp4(values: np.ndarray, scale_rows: np.ndarray, original_shape=None) -> np.ndarray:
+    """f32 [M, N]: fp16(value) * fp16(2^(e - 127)), the product rounded to fp16 (the reference's
+    intermediate dtype; scales outside fp16's range become 0 or inf there), widened."""
+    code = np.empty((values.shape[0], values.shape[1] * 2), dtype=np.uint8)
+    code[:, 0::2] = values & 0xF
+    code[:, 1::2] = values >> 4
+    v16 = (E2M1_VALUES[code & 7] * np.where(code & 8, np.float32(-1), np.float32(1))).astype(np.float16)
+    with np.errstate(over="ignore"):
+        s16 = np.ldexp(np.float64(1.0), scale_rows.astype(np.int32) - 127).astype(np.float16)
+        out = (v16 * np.repeat(s16, 32, axis=1)).astype(np.float32)
+    if original_shape is not None:
+        out = out[: original_shape[0], : original_shape[1]]
+    return out
+
+
+def gemm_mxfp4(values_a, sf_rows_a, values_b, sf_rows_b):
+    """bf16 bits and f32 of sum_k (a 2^ea)(b 2^eb) on padded operands, accumulated in double
+    (alpha = 1: src/fouroversix/matmul/cutlass/backend.py:79-85)."""
+    def expand(values, sf_rows):
+        code = np.empty((values.shape[0], values.shape[1] * 2), dtype=np.uint8)
+        code[:, 0::2] = values & 0xF
+        code[:, 1::2] = values >> 4
+        v = E2M1_VALUES[code & 7].astype(np.float64) * np.where(code & 8, -1.0, 1.0)
+        return v * np.repeat(np.ldexp(1.0, sf_rows.astype(np.int32) - 127), 32, axis=1)
+
+    o32 = (expand(values_a, sf_rows_a) @ expand(values_b, sf_rows_b).T).astype(np.float32)
+    return f32_to_bf16_bits(o32), o32

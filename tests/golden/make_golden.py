@@ -134,18 +134,62 @@ def write_transform_vectors() -> None:
     print("wrote transform", len(out))
 
 
+def write_mxfp4_vectors(quantize, dequantize, quantized_matmul, QuantizationConfig) -> None:  # noqa: N803
+    """MXFP4 (E2M1 codes, E8M0 scale per 1x32 block; quantize/pytorch/reference.py:149-181)
+    through the reference's PyTorch backend: quantize, dequantize and matmul."""
+    out: dict[str, np.ndarray] = {}
+    for name, kind, shape, seed in [
+        ("randn_256x256", "randn", (256, 256), 41),
+        ("outlier_128x384", "outlier", (128, 384), 42),
+        ("tiny_blocks_128x128", "tiny_blocks", (128, 128), 43),
+        ("ragged_100x80", "randn", (100, 80), 44),
+        ("weight_16x128", "weight", (16, 128), 45),
+    ]:
+        x = make_input(kind, shape, seed)
+        if kind == "randn":
+            x[1, :32] = 0  # an all-zero block
+            x[2, 5] = -0.0
+        out[f"{name}.x"] = bits(x)
+        for rule in ("static_6", "static_4"):
+            q = quantize(x.clone(), QuantizationConfig(backend="pytorch", dtype="mxfp4", scale_rule=rule))
+            key = f"{name}.{rule}"
+            out[key + ".values"] = u8(q.values)
+            out[key + ".sf"] = u8(q.scale_factors)
+            out[key + ".amax"] = np.array([float(q.amax)], dtype=np.float32)
+            out[key + ".padded"] = np.array(q.padded_shape)
+            out[key + ".deq_bf16"] = bits(dequantize(q))
+            out[key + ".deq_f32"] = dequantize(q, torch.float32).numpy().copy()
+    for tag, (m, n, k), rule, seed in [("256x128x256", (256, 128, 256), "static_6", 46),
+                                       ("100x72x160", (100, 72, 160), "static_4", 47)]:
+        g = torch.Generator("cpu").manual_seed(seed)
+        a = torch.randn(m, k, generator=g).bfloat16()
+        b = torch.randn(n, k, generator=g).bfloat16()
+        cfg = QuantizationConfig(backend="pytorch", dtype="mxfp4", scale_rule=rule)
+        o = quantized_matmul(quantize(a, cfg), quantize(b, cfg), backend="pytorch")
+        out[f"mm.{tag}.a"] = bits(a)
+        out[f"mm.{tag}.b"] = bits(b)
+        out[f"mm.{tag}.out"] = bits(o)
+        out[f"mm.{tag}.rule"] = np.array(rule)
+    np.savez_compressed(os.path.join(HERE, "mxfp4.npz"), **out)
+    print("wrote mxfp4", len(out))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
     ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
+    ap.add_argument("--only-mxfp4", action="store_true", help="write only mxfp4.npz")
     args = ap.parse_args()
 
     fos = import_reference()
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
-    write_transform_vectors()
-    if args.only_transform:
+    if not args.only_mxfp4:
+        write_transform_vectors()
+    if not args.only_transform:
+        write_mxfp4_vectors(quantize, dequantize, quantized_matmul, QuantizationConfig)
+    if args.only_transform or args.only_mxfp4:
         return
 
     # ---- quantize + dequantize ------------------------------------------------------

@@ -1,0 +1,114 @@
+"""MXFP4 (E2M1 codes, E8M0 scale per 1x32 block) on the GPU: quantize, dequantize and the
+GEMM on the scaled FP4 matrix instruction, against the reference's vectors and the oracle's
+numpy restatement.  Quantize / dequantize are bit-exact; the GEMM is held to the budget the
+reference gives its own backends (tests/test_matmul.py:15,81-88)."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import fouroversix_amd as fos
+from gpu_utils import bits16, make_input, u8
+
+pytestmark = pytest.mark.gpu
+
+MISMATCH_BUDGET = 1e-3
+MAX_REL = 1e-2
+
+
+def mx_config(rule="static_6", **kw):
+    return fos.QuantizationConfig(dtype="mxfp4", scale_rule=rule, **kw)
+
+
+def from_bits(a):
+    return torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+
+
+def test_mxfp4_matches_reference_vectors(golden_dir):
+    d = np.load(os.path.join(golden_dir, "mxfp4.npz"))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        base = key[: -len(".values")]
+        name, rule = base.split(".")
+        x = from_bits(d[f"{name}.x"]).cuda()
+        q = fos.quantize(x, mx_config(rule))
+        assert tuple(q.padded_shape) == tuple(d[base + ".padded"]), base
+        assert q.scale_factors.dtype == torch.float8_e8m0fnu and q.scale_factors_are_in_blackwell_layout
+        assert np.array_equal(u8(q.values), d[base + ".values"]), base
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), d[base + ".sf"].reshape(-1)), base
+        assert float(q.amax) == 1.0
+        assert np.array_equal(bits16(fos.dequantize(q)), d[base + ".deq_bf16"]), base
+        assert np.array_equal(fos.dequantize(q, torch.float32).cpu().numpy(), d[base + ".deq_f32"]), base
+        n += 1
+    assert n == 10
+    for tag in ("256x128x256", "100x72x160"):
+        rule = str(d[f"mm.{tag}.rule"])
+        a, b = from_bits(d[f"mm.{tag}.a"]).cuda(), from_bits(d[f"mm.{tag}.b"]).cuda()
+        out = fos.quantized_matmul(a, b, input_config=mx_config(rule), other_config=mx_config(rule))
+        ref = d[f"mm.{tag}.out"]
+        assert out.shape == ref.shape
+        assert float((bits16(out) != ref).mean()) <= MISMATCH_BUDGET, tag
+
+
+@pytest.mark.parametrize("rule", ["static_6", "static_4"])
+@pytest.mark.parametrize(("kind", "shape", "scale"), [
+    ("randn", (1024, 2048), 1.0), ("outlier", (300, 200), 1.0), ("tiny_blocks", (130, 528), 1.0),
+    ("zeros", (128, 128), 1.0), ("randn", (64, 96), 2.0 ** -120), ("randn", (256, 640), 2.0 ** 100),
+])
+def test_mxfp4_quantize_dequantize_match_oracle(oracle, kind, shape, scale, rule):
+    """Shapes that are not multiples of (128, 128) or of the 128 x 512 workgroup tile,
+    unaligned row pitch, sub-normal and huge magnitudes (fp16 intermediate under/overflow in
+    dequantize follows the reference)."""
+    x = (make_input(kind, shape, 5).float() * scale).bfloat16()
+    x[0, :3] = -x[0, :3].abs()
+    x[1, 1] = -0.0
+    ref = oracle.quantize_mxfp4(x, scale_rule=rule)
+    for xin in (x.cuda(), torch.nn.functional.pad(x, (0, 3)).cuda()[:, : shape[1]]):  # second: ld % 8 != 0
+        q = fos.quantize(xin, mx_config(rule))
+        assert tuple(q.padded_shape) == tuple(ref.padded_shape)
+        assert np.array_equal(u8(q.values), ref.values)
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), ref.scale_factors)
+    rdeq = oracle.dequantize_mxfp4(ref.values, ref.scale_rows, ref.original_shape)
+    got = fos.dequantize(q, torch.float32).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), rdeq.view(np.uint32))
+    assert np.array_equal(bits16(fos.dequantize(q)), oracle.f32_to_bf16_bits(rdeq))
+    assert np.array_equal(fos.dequantize(q, torch.float16).cpu().numpy().view(np.uint16), rdeq.astype(np.float16).view(np.uint16))
+
+
+def test_mxfp4_unsupported_configurations():
+    x = make_input("randn", (128, 128), 1).cuda()
+    for bad in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True),
+                dict(scale_rule="static_6", round_style="stochastic")):
+        with pytest.raises(ValueError, match="No backend found"):
+            fos.quantize(x, fos.QuantizationConfig(dtype="mxfp4", **bad))
+
+
+@pytest.mark.parametrize(("m", "n", "k"), [(128, 128, 128), (256, 384, 640), (512, 256, 1152), (100, 72, 80),
+                                           (4096, 4096, 1024), (8192, 8192, 8192)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float16"])
+def test_mxfp4_gemm(oracle, m, n, k, out_dtype):
+    """Both tile shapes, odd numbers of 128-wide K steps, ragged shapes through the frontend;
+    192 sampled rows of each operand are multiplied by the oracle in fp64."""
+    if out_dtype == "float16" and m > 1024:
+        pytest.skip("fp16 output covered by the smaller shapes")
+    a, b = make_input("randn", (m, k), 5), make_input("randn", (n, k), 6)
+    qa, qb = fos.quantize(a.cuda(), mx_config()), fos.quantize(b.cuda(), mx_config("static_4"))
+    out = fos.quantized_matmul(qa, qb, out_dtype=out_dtype)
+    assert out.shape == (m, n) and out.dtype == getattr(torch, out_dtype)
+    g = torch.Generator("cpu").manual_seed(7)
+    rows = torch.randperm(m, generator=g)[: min(m, 192)].sort().values
+    cols = torch.randperm(n, generator=g)[: min(n, 192)].sort().values
+    va, vb = u8(qa.values), u8(qb.values)
+    kp = va.shape[1] * 2
+    sa = oracle.from_blocked(u8(qa.scale_factors).reshape(-1), va.shape[0], kp // 32)
+    sb = oracle.from_blocked(u8(qb.scale_factors).reshape(-1), vb.shape[0], kp // 32)
+    _, ref32 = oracle.gemm_mxfp4(va[rows.numpy()], sa[rows.numpy()], vb[cols.numpy()], sb[cols.numpy()])
+    got = out[rows.cuda()][:, cols.cuda()].float().cpu().numpy()
+    expect = torch.from_numpy(ref32).to(getattr(torch, out_dtype)).float().numpy()
+    frac = float((got != expect).mean())
+    rel = float(np.abs(got - expect).max() / max(np.abs(expect).max(), 1e-30))
+    assert frac <= MISMATCH_BUDGET and rel <= MAX_REL, f"{frac:.2e} of outputs differ, max rel {rel:.2e}"

@@ -229,3 +229,36 @@ def test_stochastic_rounding_known_answers(oracle):
     q = oracle.quantize(x, scale_rule="static_6", round_style="stochastic", seed=7)
     deq = oracle.dequantize(q.values, q.scale_rows, q.amax, scale_rule="static_6", round_style="stochastic")
     assert abs(float((deq - xf).mean())) < 2e-3
+
+
+def test_mxfp4_matches_reference_vectors(oracle, golden_dir):
+    """MXFP4 quantize / dequantize / matmul restatement against vectors written by the
+    reference's PyTorch backend (quantize/pytorch/reference.py:149-181, quantize/backend.py:89-160):
+    codes, E8M0 scales in the 128x4-tile layout, amax == 1, padded shapes (cols to 128),
+    dequantized values bit for bit; matmul within the reference's own budget."""
+    d = np.load(os.path.join(golden_dir, "mxfp4.npz"))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        base = key[: -len(".values")]
+        name, rule = base.split(".")
+        q = oracle.quantize_mxfp4(d[f"{name}.x"], scale_rule=rule)
+        assert tuple(q.padded_shape) == tuple(d[base + ".padded"]), base
+        assert np.array_equal(q.values, d[base + ".values"]), base
+        assert np.array_equal(q.scale_factors, d[base + ".sf"].reshape(-1)), base
+        assert q.amax == d[base + ".amax"][0] == 1.0
+        deq = oracle.dequantize_mxfp4(q.values, q.scale_rows, q.original_shape)
+        assert np.array_equal(deq, d[base + ".deq_f32"]), base
+        assert np.array_equal(oracle.f32_to_bf16_bits(deq), d[base + ".deq_bf16"]), base
+        n += 1
+    assert n == 10
+    for tag in ("256x128x256", "100x72x160"):
+        rule = str(d[f"mm.{tag}.rule"])
+        qa = oracle.quantize_mxfp4(d[f"mm.{tag}.a"], scale_rule=rule)
+        qb = oracle.quantize_mxfp4(d[f"mm.{tag}.b"], scale_rule=rule)
+        o16, _ = oracle.gemm_mxfp4(qa.values, qa.scale_rows, qb.values, qb.scale_rows)
+        m, nn = qa.original_shape[0], qb.original_shape[0]
+        ref = d[f"mm.{tag}.out"]
+        got = o16[:m, :nn]
+        assert float((got != ref).mean()) <= 1e-3
