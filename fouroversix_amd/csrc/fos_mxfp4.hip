@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstdlib>
+
 #include "fos_quantize_fast.h"
 #include "fouroversix_hip.h"
 
@@ -340,22 +342,22 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
         uint32_t a[WM], b[WN];  // scale bytes of the step's four K blocks, per row tile
     };
     auto fetch = [&](int64_t ks, Staged &s) {
+        // per-pass and per-step displacements ride in the scalar offset: one address register
         const int kq = (int)(ks * (kMxBK / 2));
 #pragma unroll
         for (int i = 0; i < PA; ++i)
-            s.a[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)(q_off + i * kRowsPerPass * kbytes), kq, 0));
+            s.a[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, kq + (int)(i * kRowsPerPass * kbytes), 0));
 #pragma unroll
         for (int i = 0; i < PB; ++i)
-            s.b[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(q_off + i * kRowsPerPass * kbytes), kq, 0));
+            s.b[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)q_off, kq + (int)(i * kRowsPerPass * kbytes), 0));
     };
-    // lanes of the upper half shift their word by one byte, so that byte 0 / byte 2 of every
-    // lane's register are the scales of the K blocks it feeds in slice 0 / slice 1
+    // raw scale words of step ks (bytes = the four K blocks of the chunk)
     auto fetch_scales = [&](int64_t ks, Scales &s) {
         const int ksf = (int)(ks * 512);
 #pragma unroll
-        for (int i = 0; i < WM; ++i) s.a[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)(sa_off + i * 4), ksf, 0) >> (8 * h);
+        for (int i = 0; i < WM; ++i) s.a[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)sa_off, ksf + i * 4, 0);
 #pragma unroll
-        for (int j = 0; j < WN; ++j) s.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)(sb_off + j * 4), ksf, 0) >> (8 * h);
+        for (int j = 0; j < WN; ++j) s.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)sb_off, ksf + j * 4, 0);
     };
     // half q of the staged registers -> LDS stage `buf`
     auto stage_part = [&](const Staged &s, int buf, int q) {
@@ -396,9 +398,17 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
     // after it.  Branch-free; the last step is its own instantiation.
     auto kstep = [&](auto have_next_c, int64_t ks, int buf, Staged &cur_regs, Staged &nxt, const Scales &s_cur, Scales &s_nxt) {
         constexpr bool have_next = decltype(have_next_c)::value;
+        // lanes of the upper half use the next byte: after the shift, byte 0 / byte 2 of every
+        // lane's register are the scales of the K blocks it feeds in slice 0 / slice 1.  Done
+        // here, a step after the load was issued, so that nothing waits on a fresh load.
+        Scales sh;
+#pragma unroll
+        for (int i = 0; i < WM; ++i) sh.a[i] = s_cur.a[i] >> (8 * h);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) sh.b[j] = s_cur.b[j] >> (8 * h);
         if (have_next) {
-            fetch(ks + 2 < ksteps ? ks + 2 : ksteps - 1, cur_regs);
             fetch_scales(ks + 1, s_nxt);
+            fetch(ks + 2 < ksteps ? ks + 2 : ksteps - 1, cur_regs);
         }
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
@@ -417,10 +427,10 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
                 for (int j = 0; j < WN; ++j) {
                     if (kk == 1)
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            frag_of(fb[1][j]), frag_of(fa[1][i]), acc[i][j], 4, 4, 2, (int)s_cur.b[j], 2, (int)s_cur.a[i]);
+                            frag_of(fb[1][j]), frag_of(fa[1][i]), acc[i][j], 4, 4, 2, (int)sh.b[j], 2, (int)sh.a[i]);
                     else
                         acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            frag_of(fb[0][j]), frag_of(fa[0][i]), acc[i][j], 4, 4, 0, (int)s_cur.b[j], 0, (int)s_cur.a[i]);
+                            frag_of(fb[0][j]), frag_of(fa[0][i]), acc[i][j], 4, 4, 0, (int)sh.b[j], 0, (int)sh.a[i]);
                 }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -500,7 +510,8 @@ extern "C" int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
-    const bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256;
+    bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256;
+    if (const char *e = getenv("FOS_MX_TILE")) big = big && atoi(e) != 128;  // tuning / tests
     if (big) return launch_gemm_mxfp4<2, 4, 4, 2>(p, out_type, s);
     return launch_gemm_mxfp4<2, 2, 2, 2>(p, out_type, s);
 }

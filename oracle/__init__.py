@@ -327,7 +327,7 @@ def dequantize_mxfp4(values: np.ndarray, scale_rows: np.ndarray, original_shape=
     code[:, 0::2] = values & 0xF
     code[:, 1::2] = values >> 4
     v16 = (E2M1_VALUES[code & 7] * np.where(code & 8, np.float32(-1), np.float32(1))).astype(np.float16)
-    with np.errstate(over="ignore"):
+    with np.errstate(over="ignore", invalid="ignore"):  # 0 * inf = NaN, as in the reference's fp16 product
         s16 = np.ldexp(np.float64(1.0), scale_rows.astype(np.int32) - 127).astype(np.float16)
         out = (v16 * np.repeat(s16, 32, axis=1)).astype(np.float32)
     if original_shape is not None:
