@@ -103,15 +103,17 @@ __global__ __launch_bounds__(kThreads) void quantize_mxfp4_kernel(const MxQuantP
         }
     };
 
-    Block32 blk[2];
+    // three row steps in flight per lane (192 bytes)
+    Block32 blk[3];
     load(0, blk[0]);
+    load(1, blk[1]);
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-        if (g + 1 < 8) load(g + 1, blk[(g + 1) & 1]);
+        if (g + 2 < 8) load(g + 2, blk[(g + 2) % 3]);
         if (col_ok) {
             uint4 codes;
             uint32_t e;
-            quantize_block_mxfp4(blk[g & 1], p.qmax, codes, e);
+            quantize_block_mxfp4(blk[g % 3], p.qmax, codes, e);
             const int rr = g * 16 + rr0;
             *reinterpret_cast<uint4 *>(p.codes + (row0 + g * 16) * (p.cols_p >> 1) + cb * 16) = codes;
             if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
