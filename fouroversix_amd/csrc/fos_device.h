@@ -72,9 +72,10 @@ FOS_DEVICE Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t
     return Philox4{{c0, c1, c2, c3}};
 }
 
-// Dither u in [-0.5, 0.5) with 24-bit resolution from one Philox word.
-FOS_DEVICE float dither_from_word(uint32_t w) {
-    return (float)(w >> 8) * 0x1p-24f - 0.5f;
+// Dither of element i (0..3) of a Philox word: (byte + 0.5) / 256 - 0.5, 256 equally likely
+// values symmetric about zero.
+FOS_DEVICE float dither_from_byte(uint32_t w, int i) {
+    return __builtin_fmaf((float)((w >> (8 * i)) & 0xffu), 0x1p-8f, -0.498046875f);
 }
 
 }  // namespace fos

@@ -95,7 +95,18 @@ FOS_DEVICE void reduce_partials(const QuantParams &p, uint32_t *smem, uint32_t &
 
 struct QuantConsts {
     float amax, enc, dec, qdiv, errdiv;
+    float rerr = 0.0f;      // RN(1 / errdiv)
+    bool fast_div = false;  // errdiv is a constant with an exact 3-operation division and every quotient is normal or zero
 };
+
+// v / k.errdiv with IEEE rounding (the sign of a zero quotient may differ; callers subtract).
+FOS_DEVICE float div_errdiv(float v, const QuantConsts &k) {
+    if (k.fast_div) {
+        const float q0 = v * k.rerr;
+        return __builtin_fmaf(__builtin_fmaf(-k.errdiv, q0, v), k.rerr, q0);
+    }
+    return v / k.errdiv;
+}
 
 // compute_nv_scale_factors (reference.py:184-241) for one block maximum.
 FOS_DEVICE void block_scale(const QuantConsts &k, float bmax, bool expand, uint32_t &s, float &sf, float &inv) {
@@ -196,15 +207,13 @@ FOS_DEVICE float error_term(float deq, float x) {
     return RULE == FOS_RULE_MSE ? d * d : fabsf(d);
 }
 
-// Dither for the 16 elements of 1x16 block `blk`, candidate `cand`.
+// Dither for the 16 elements of 1x16 block `blk`, candidate `cand`: one Philox4x32-10
+// call keyed (seed; blk, cand, offset), one byte per element.
 FOS_DEVICE void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float *u) {
+    const Philox4 p = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset,
+                                    (uint32_t)seed, (uint32_t)(seed >> 32));
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        Philox4 p = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)(4 * cand + j),
-                                  (uint32_t)offset, (uint32_t)seed, (uint32_t)(seed >> 32));
-#pragma unroll
-        for (int i = 0; i < 4; ++i) u[4 * j + i] = dither_from_word(p.v[i]);
-    }
+    for (int i = 0; i < 16; ++i) u[i] = dither_from_byte(p.v[i >> 2], i & 3);
 }
 
 // One 1x16 block (one row of a 16x16 tile when TWO_D): 8 input words -> 2 code words
@@ -263,8 +272,8 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
             uint32_t nibA = e2m1_mag_code(r) | (neg ? 8u : 0u);
             float q = int4_round<SR>(xs * 1.16666666f, SR ? uB[i] : 0.0f);
             uint32_t nibB = (uint32_t)((int)q) & 0xfu;
-            float deqA = ((fq * sfA) * k.amax) / k.errdiv;
-            float deqB = (((q * sfA) * k.amax) * 0.8571428571f) / k.errdiv;
+            float deqA = div_errdiv((fq * sfA) * k.amax, k);
+            float deqB = div_errdiv(((q * sfA) * k.amax) * 0.8571428571f, k);
             eA[i] = error_term<RULE>(deqA, x[i]);
             eB[i] = error_term<RULE>(deqB, x[i]);
             if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
@@ -293,8 +302,8 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
         bool negA = xsA < 0.0f, negB = xsB < 0.0f;
         uint32_t nibA = e2m1_mag_code(rA) | (negA ? 8u : 0u);
         uint32_t nibB = e2m1_mag_code(rB) | (negB ? 8u : 0u);
-        float deqA = (((negA ? -rA : rA) * sfA) * k.amax) / k.errdiv;
-        float deqB = (((negB ? -rB : rB) * sfB) * k.amax) / k.errdiv;
+        float deqA = div_errdiv(((negA ? -rA : rA) * sfA) * k.amax, k);
+        float deqB = div_errdiv(((negB ? -rB : rB) * sfB) * k.amax, k);
         eA[i] = error_term<RULE>(deqA, x[i]);
         eB[i] = error_term<RULE>(deqB, x[i]);
         if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }

@@ -39,6 +39,8 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
     const float rq = 1.0f / k.qdiv;
+    k.rerr = 1.0f / k.errdiv;
+    k.fast_div = in_range && (k.errdiv == 1536.0f || k.errdiv == 2688.0f);
     if (FAST) {
         if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
         __syncthreads();

@@ -216,19 +216,19 @@ void fos_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint
 }
 
 /* Dither for the 16 elements of 1x16 block `blk` (= row * blocks_per_row + block column
- * of the padded tensor), candidate `cand`: call j (0..3) uses counter
- * (blk_lo, blk_hi, 4*cand + j, offset_lo) and key (seed_lo, seed_hi) and serves elements
- * 4j..4j+3; u = (word >> 8) * 2^-24 - 0.5. */
+ * of the padded tensor), candidate `cand`: ONE Philox4x32-10 call with counter
+ * (blk_lo, blk_hi, cand, offset_lo) and key (seed_lo, seed_hi); element i takes byte
+ * i % 4 of word i / 4: u = (byte + 0.5) / 256 - 0.5, i.e. 256 equally likely values that
+ * are symmetric about zero (8 random bits per element, as hardware stochastic-rounding
+ * converts consume; the reference draws from torch's generator, so its stream cannot be
+ * matched bit for bit anyway). */
 static void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float u[16]) {
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
-    for (int j = 0; j < 4; ++j) {
-        uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)(4 * cand + j),
-                           (uint32_t)offset};
-        uint32_t w[4];
-        fos_oracle_philox4x32_10(ctr, key, w);
-        for (int i = 0; i < 4; ++i)
-            u[4 * j + i] = (float)(w[i] >> 8) * 5.9604644775390625e-08f - 0.5f;
-    }
+    uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset};
+    uint32_t w[4];
+    fos_oracle_philox4x32_10(ctr, key, w);
+    for (int i = 0; i < 16; ++i)
+        u[i] = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xffu) * 0.00390625f - 0.498046875f;
 }
 
 /* ---- quantize ---------------------------------------------------------------------- */
