@@ -109,6 +109,54 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
     }
 
 
+def extras(dev, steps: int) -> dict:
+    """Timings of the rows built around the headline path (whole calls through the public
+    API, microseconds): small-M GEMMs, fused pseudo-quantize, dequantize, the transpose /
+    random-Hadamard options, stochastic rounding and MXFP4."""
+    import torch
+
+    import fouroversix_amd as fos
+
+    def us(fn):
+        fn()  # warm-up
+        return round(event_ms(fn, steps) * 1e3, 1)
+
+    out = {}
+    xs = [make_activation(8192, 8192, 200 + i).to(dev) for i in range(2)]
+    n = [0]
+
+    def nxt():
+        n[0] += 1
+        return xs[n[0] % 2]
+
+    q = fos.quantize(xs[0], fos.QuantizationConfig(scale_rule="mse"))
+    out["dequantize_8192x8192_us"] = us(lambda: fos.dequantize(q))
+    del q
+    for name, kw in (("pseudo_quantize_mse", dict(scale_rule="mse", pseudo_quantize=True)),
+                     ("quantize_mse_2d", dict(scale_rule="mse", block_scale_2d=True)),
+                     ("quantize_mse_rht", dict(scale_rule="mse", rht=True)),
+                     ("quantize_mse_transpose_rht", dict(scale_rule="mse", rht=True, transpose=True)),
+                     ("quantize_mse_stochastic", dict(scale_rule="mse", round_style="stochastic", kwargs={"seed": 1})),
+                     ("quantize_if4_mse", dict(dtype="if4", scale_rule="mse")),
+                     ("quantize_mxfp4_static_6", dict(dtype="mxfp4", scale_rule="static_6"))):
+        cfg = fos.QuantizationConfig(**kw)
+        out[f"{name}_8192x8192_us"] = us(lambda: fos.quantize(nxt(), cfg))
+    del xs
+    mse = fos.QuantizationConfig(scale_rule="mse")
+    for m, nn, k in ((16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336), (128, 4096, 4096), (2048, 14336, 4096)):
+        qa = fos.quantize(make_activation(m, k, 7).to(dev), mse)
+        qb = fos.quantize(make_activation(nn, k, 8).to(dev), mse)
+        out[f"gemm_nvfp4_{m}x{nn}x{k}_us"] = us(lambda: fos.quantized_matmul(qa, qb))
+    mx = fos.QuantizationConfig(dtype="mxfp4", scale_rule="static_6")
+    qa = fos.quantize(make_activation(8192, 8192, 5).to(dev), mx)
+    qb = fos.quantize(make_activation(8192, 8192, 6).to(dev), mx)
+    fos.quantized_matmul(qa, qb)
+    t = event_ms(lambda: fos.quantized_matmul(qa, qb), steps)
+    out["gemm_mxfp4_8192x8192x8192"] = {"ms": round(t, 4), "TFLOP/s": round(2.0 * 8192 ** 3 / (t * 1e-3) / 1e12, 1),
+                                        "frac_of_fp4_peak": round(2.0 * 8192 ** 3 / (t * 1e-3) / 1e12 / 10100.0, 4)}
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,6 +167,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-oracle baseline leg")
     ap.add_argument("--no-gemm", action="store_true")
     ap.add_argument("--no-stack", action="store_true", help="skip the 32-layer quantized-linear stack")
+    ap.add_argument("--no-extras", action="store_true", help="skip the timings of the surrounding operations")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -250,6 +299,12 @@ def main() -> int:
     if not args.no_stack and not args.no_gemm:
         stack = linear_stack(dev, steps=3, warmup=1)
 
+    extra = None
+    if not args.no_extras:
+        del xs[1:]
+        torch.cuda.empty_cache()
+        extra = extras(dev, steps=max(5, K // 5))
+
     # ---- CPU baseline: the C oracle on the host cores, bounded sample -----------------
     cpu = None
     if not args.no_cpu:
@@ -298,6 +353,7 @@ def main() -> int:
         "cpu_baseline": cpu,
         "gemm": gemm,
         "linear_stack": stack,
+        "extras": extra,
     }
     print(json.dumps(line))
     return 0

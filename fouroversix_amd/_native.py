@@ -32,6 +32,7 @@ EXPORTS = (
     "fos_transform",
     "fos_gemm_nvfp4",
     "fos_gemm_mxfp4",
+    "fos_gemm_alpha",
     "fos_padded_cols_for",
     "fos_gemm_workspace_bytes",
     "fos_dequantize",
@@ -78,6 +79,8 @@ def lib() -> ctypes.CDLL:
     L.fos_transform.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
+    L.fos_gemm_alpha.argtypes = [vp, vp, dbl, vp, vp]
+    L.fos_gemm_alpha.restype = i32
     L.fos_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp]
     L.fos_gemm_mxfp4.restype = i32
     L.fos_padded_cols_for.argtypes = [i32, i64]

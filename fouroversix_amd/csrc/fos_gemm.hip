@@ -624,6 +624,22 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
 
 using namespace fos;
 
+namespace fos {
+// tensor / python-scalar on a GPU is, in torch, a multiplication by the reciprocal, which is
+// formed once on the host in double precision and rounded to fp32 (measured against
+// torch on the device); the reference's alpha is formed that way
+__global__ void gemm_alpha_kernel(const float *amax_a, const float *amax_b, float inv_den, float *alpha) {
+    *alpha = (*amax_a * *amax_b) * inv_den;
+}
+}  // namespace fos
+
+extern "C" int fos_gemm_alpha(const float *amax_a, const float *amax_b, double denominator, float *alpha,
+                              fos_stream_t stream) {
+    if (!amax_a || !amax_b || !alpha) return FOS_E_NULL_POINTER;
+    hipLaunchKernelGGL(gemm_alpha_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, amax_a, amax_b, (float)(1.0 / denominator), alpha);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
 extern "C" size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || (M < 128 && K % 256 != 0) || N % 128 != 0 || K % 64 != 0)
         return 0;

@@ -40,8 +40,15 @@ def is_supported(input: QuantizedTensor, other: QuantizedTensor, *, out_dtype: D
 
 
 def gemm_alpha(input: QuantizedTensor, other: QuantizedTensor) -> torch.Tensor:
+    """``(amaxA * amaxB) / (qA sA qB sB adjA adjB)`` as a device f32[1] (reference
+    matmul/cutlass/backend.py:86-98); one small kernel when both maxima are f32 GPU tensors."""
     den = dequantize_divisor(input) * dequantize_divisor(other)
-    return ((input.amax * other.amax) / den).to(torch.float32).reshape(1)
+    a, b = input.amax, other.amax
+    if a.dtype == torch.float32 and b.dtype == torch.float32 and a.is_cuda and b.device == a.device:
+        alpha = torch.empty(1, dtype=torch.float32, device=a.device)
+        ops.gemm_alpha_into(a, b, den, alpha)
+        return alpha
+    return ((a * b) / den).to(torch.float32).reshape(1)
 
 
 def quantized_matmul(

@@ -248,6 +248,15 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
     return out
 
 
+def gemm_alpha_into(amax_a, amax_b, denominator, alpha):
+    """alpha[0] = (amax_a * amax_b) * f32(1 / denominator) on the device, torch's GPU arithmetic for
+    ``(amax_a * amax_b) / denominator``."""
+    with _on_device(alpha.device):
+        rc = nat.lib().fos_gemm_alpha(amax_a.data_ptr(), amax_b.data_ptr(), float(denominator), alpha.data_ptr(),
+                                      nat.current_stream(alpha.device))
+    nat.check(rc, "fouroversix::gemm_alpha")
+
+
 def _gemm_mxfp4_impl(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):
     """MXFP4 x MXFP4 GEMM on the scaled FP4 matrix instruction; checks as the NVFP4 op
     (reference csrc/include/element_traits.hpp:122-170 with blocks of 32, E8M0 scales)."""

@@ -155,6 +155,16 @@ int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const
                    void *D, int out_type, int64_t ldd,
                    void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
+/*
+ * alpha[0] = (amax_a[0] * amax_b[0]) * f32(1 / denominator), in fp32 on the device: the
+ * GEMM's output scale as src/fouroversix/matmul/cutlass/backend.py:86-98 forms it on a GPU
+ * (torch divides a tensor by a host scalar through the reciprocal, taken in double and
+ * rounded to fp32; denominator = the product of both operands' qmax * smax * rounding
+ * adjustment), in one launch.
+ */
+int fos_gemm_alpha(const float *amax_a, const float *amax_b, double denominator, float *alpha,
+                   fos_stream_t stream);
+
 /* Bytes of workspace with which fos_gemm_nvfp4 runs this shape fastest (0 = none needed).
  * The reference's op runs CUTLASS without a workspace
  * (src/fouroversix/csrc/fp4_gemm.cu:148-151), so this has no counterpart there. */

@@ -254,11 +254,13 @@ def quantized_matmul(qa: OracleQuantized, qb: OracleQuantized, threads=None):
 
 
 def gemm_alpha(qa: OracleQuantized, qb: OracleQuantized) -> np.float32:
-    """alpha of the native GEMM form (reference matmul/cutlass/backend.py:86-98)."""
+    """alpha of the native GEMM form (reference matmul/cutlass/backend.py:86-98), with the
+    arithmetic torch uses for ``tensor / python_scalar`` on a GPU (where that backend
+    runs): the product times the reciprocal, taken in double and rounded to fp32."""
     qa_max, sa_max = qmax_smax(qa.dtype, qa.scale_rule)
     qb_max, sb_max = qmax_smax(qb.dtype, qb.scale_rule)
     den = qa_max * sa_max * qb_max * sb_max * adjustment(qa.round_style) * adjustment(qb.round_style)
-    return np.float32(np.float32(qa.amax * qb.amax) / np.float32(den))
+    return np.float32(np.float32(np.float32(qa.amax) * np.float32(qb.amax)) * np.float32(1.0 / den))
 
 
 def gemm_nvfp4(values_a, sf_rows_a, values_b, sf_rows_b, alpha, threads=None):

@@ -176,3 +176,19 @@ def test_linear_layer_forward(oracle):
     lin2.load_state_dict({"weight": w, "bias": bias})
     keep = fos.FourOverSixLinear(lin2.cuda(), fos.ModuleQuantizationConfig(weight_scale_2d=True, keep_master_weights=True))
     assert torch.equal(keep(x.cuda()), y)
+
+
+def test_gemm_alpha_kernel_matches_the_reference_expression():
+    """alpha = (amaxA * amaxB) / (qA sA qB sB adjA adjB) with fp32 operations
+    (reference matmul/cutlass/backend.py:86-98): the one-launch kernel against torch."""
+    cfgs = [fos.QuantizationConfig(scale_rule=r, round_style=s) for r, s in
+            (("mse", "nearest"), ("static_6", "nearest"), ("static_4", "stochastic_unbiased"), ("mae", "stochastic"))]
+    for i, ca in enumerate(cfgs):
+        cb = cfgs[(i + 1) % len(cfgs)]
+        qa = fos.quantize((make_input("randn", (128, 64), 30 + i) * (3.0 ** i)).cuda(), ca)
+        qb = fos.quantize((make_input("weight", (128, 64), 40 + i)).cuda(), cb)
+        den = fos.quantize.__globals__["dequantize_divisor"](qa) * fos.quantize.__globals__["dequantize_divisor"](qb)
+        expect = ((qa.amax * qb.amax) / den).to(torch.float32).reshape(1)
+        got = fos.matmul.frontend.gemm_alpha(qa, qb)
+        assert got.dtype == torch.float32 and got.shape == (1,)
+        assert torch.equal(got.view(torch.int32), expect.view(torch.int32))
