@@ -38,100 +38,118 @@ struct MxQuantParams {
     int sf_layout;
     int tiles_x;
     int vector_loads;        // x 16-byte aligned, ld % 8 == 0
+    float *amax;             // written with 1: the format has no tensor scale
 };
 
-struct Block32 {
-    uint32_t w[16];
-};
+// One lane owns 8 consecutive elements (one 128-bit load), four neighbouring lanes own a
+// 1x32 block: every load instruction of a wavefront covers 1 KiB of one row (whole cache
+// lines), the block maximum is two quad permutes, and the codes leave as one 32-bit word
+// per lane (256 contiguous bytes per wavefront and row).
+FOS_DEVICE uint32_t quad_max_u32(uint32_t v) {
+    const uint32_t a = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+    v = v > a ? v : a;
+    const uint32_t b = (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+    return v > b ? v : b;
+}
 
-// Codes (4 words) and scale byte of one 1x32 block.
-FOS_DEVICE void quantize_block_mxfp4(const Block32 &b, float qmax, uint4 &codes, uint32_t &e) {
+// 8 elements (4 words of 2 bf16) of a block -> their code word and the block's scale byte.
+FOS_DEVICE void quantize_octet_mxfp4(const uint4 &x, float qmax, uint32_t &codes, uint32_t &e) {
+    const uint32_t w[4] = {x.x, x.y, x.z, x.w};
     uint32_t m = 0;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) m = pk_max_u16(m, b.w[i] & 0x7fff7fffu);
-    const uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    for (int i = 0; i < 4; ++i) m = pk_max_u16(m, w[i] & 0x7fff7fffu);
+    uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    mm = quad_max_u32(mm);
     const float s_hp = u2f(mm << 16) / qmax;
     const uint32_t u = f2u(s_hp);
     e = (u >> 23) & 0xffu;
     if (u & 0x7fffffu) e = (e + 1u) & 0xffu;  // round up to the next power of two
     // 1 / 2^(e - 127); e == 0 marks an all-zero block (values become 0), 255 is inf / NaN
     const float inv = e == 0u || e == 255u ? 0.0f : (e == 254u ? u2f(0x00400000u) : u2f((254u - e) << 23));
-    uint32_t c[4] = {0, 0, 0, 0};
-    static_for<0, 16>([&](auto jc) {
+    uint32_t c = 0;
+    static_for<0, 4>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
         // + 0: the reference multiplies by sign(x) with sign(-0.0) = 0, so a negative zero
         // (also one produced by underflow) must not keep its sign; a negative value that
         // rounds to zero does
-        const float lo = __builtin_fmaf(u2f(b.w[j] << 16), inv, 0.0f);
-        const float hi = __builtin_fmaf(u2f(b.w[j] & 0xffff0000u), inv, 0.0f);
-        c[j >> 2] = pack_fp4<(j & 3)>(c[j >> 2], lo, hi);
+        const float lo = __builtin_fmaf(u2f(w[j] << 16), inv, 0.0f);
+        const float hi = __builtin_fmaf(u2f(w[j] & 0xffff0000u), inv, 0.0f);
+        c = pack_fp4<j>(c, lo, hi);
     });
-    codes = make_uint4(c[0], c[1], c[2], c[3]);
+    codes = c;
 }
 
-// Workgroup tile 128 rows x 512 columns (16 blocks): a wavefront covers 4 rows x 16
-// blocks = 1 KiB contiguous per row; eight steps of 16 rows; the four complete 128x4 scale
-// tiles are staged in LDS and leave as one contiguous 2 KiB run.
-__global__ __launch_bounds__(kThreads) void quantize_mxfp4_kernel(const MxQuantParams p) {
+// Workgroup tile 128 rows x 512 columns (16 blocks per row): a wavefront covers one row of
+// the tile per load instruction (512 elements = 1 KiB), four rows per step; 8 wavefronts,
+// four steps of 32 rows; the four complete 128x4 scale tiles are staged in LDS and leave as
+// one contiguous 2 KiB run.
+constexpr int kMxQuantThreads = 512;
+__global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const MxQuantParams p) {
     __shared__ uint32_t sf_stage[4 * 128];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int lb = lane & 15, rr0 = wave * 4 + (lane >> 4);
+    const int lb = lane >> 2;  // block column inside the tile
     const int64_t sf_cols = p.cols_p >> 5;
     const int64_t tile_y = blockIdx.x / p.tiles_x, tile_x = blockIdx.x - tile_y * p.tiles_x;
     const int64_t cb = tile_x * 16 + lb;
+    const int64_t c0 = tile_x * 512 + lane * 8;  // first column of this lane's 8 elements
     const bool col_ok = cb < sf_cols;
     const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
-    const int64_t row0 = tile_y * 128 + rr0;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *p.amax = 1.0f;  // the reference reports amax = 1 (reference.py:573-578)
 
-    auto load = [&](int g, Block32 &b) {
-        const int64_t r = row0 + g * 16, c0 = cb * 32;
-        if (r < p.rows && c0 + 32 <= p.cols && p.vector_loads) {
-            const uint4 *q = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint4 t = q[v];
-                b.w[4 * v] = t.x; b.w[4 * v + 1] = t.y; b.w[4 * v + 2] = t.z; b.w[4 * v + 3] = t.w;
-            }
+    auto load = [&](int64_t r, uint4 &v) {
+        if (r < p.rows && c0 + 8 <= p.cols && p.vector_loads) {
+            v = *reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
         } else {
+            uint32_t w[4];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < 4; ++i) {
                 uint32_t lo = 0, hi = 0;
                 if (r < p.rows && c0 + 2 * i < p.cols) lo = p.x[r * p.ld + c0 + 2 * i];
                 if (r < p.rows && c0 + 2 * i + 1 < p.cols) hi = p.x[r * p.ld + c0 + 2 * i + 1];
-                b.w[i] = lo | (hi << 16);
+                w[i] = lo | (hi << 16);
             }
+            v = make_uint4(w[0], w[1], w[2], w[3]);
         }
     };
 
-    // three row steps in flight per lane (192 bytes)
-    Block32 blk[3];
-    load(0, blk[0]);
-    load(1, blk[1]);
+    // rows of step g: tile_y * 128 + g * 32 + wave * 4 + j; three steps (12 loads) in flight
+    constexpr int kSteps = 4;
+    uint4 x[3][4];
+    const int64_t row_w = tile_y * 128 + wave * 4;
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-        if (g + 2 < 8) load(g + 2, blk[(g + 2) % 3]);
-        if (col_ok) {
-            uint4 codes;
-            uint32_t e;
-            quantize_block_mxfp4(blk[g % 3], p.qmax, codes, e);
-            const int rr = g * 16 + rr0;
-            *reinterpret_cast<uint4 *>(p.codes + (row0 + g * 16) * (p.cols_p >> 1) + cb * 16) = codes;
-            if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
-            else p.sf[(row0 + g * 16) * sf_cols + cb] = (uint8_t)e;
+    for (int j = 0; j < 4; ++j) load(row_w + j, x[0][j]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load(row_w + 32 + j, x[1][j]);
+#pragma unroll
+    for (int g = 0; g < kSteps; ++g) {
+        if (g + 2 < kSteps) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load(row_w + (g + 2) * 32 + j, x[(g + 2) % 3][j]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t codes, e;
+            quantize_octet_mxfp4(x[g % 3][j], p.qmax, codes, e);  // all lanes: the quad permutes need their neighbours
+            if (!col_ok) continue;
+            const int rr = g * 32 + wave * 4 + j;
+            const int64_t r = tile_y * 128 + rr;
+            *reinterpret_cast<uint32_t *>(p.codes + r * (p.cols_p >> 1) + (c0 >> 1)) = codes;
+            if ((lane & 3) == 0) {
+                if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
+                else p.sf[r * sf_cols + cb] = (uint8_t)e;
+            }
         }
     }
     if (tiled) {
         __syncthreads();
-        const int t = threadIdx.x >> 6;  // scale tile of this wavefront: 512 bytes, 8 per lane
+        const int t = threadIdx.x >> 6;  // wavefronts 0-3: one scale tile each, 512 bytes, 8 per lane
         const int64_t group = tile_x * 4 + t;
-        if (group < (sf_cols >> 2)) {
+        if (t < 4 && group < (sf_cols >> 2)) {
             uint2 *out = reinterpret_cast<uint2 *>(p.sf + (tile_y * (sf_cols >> 2) + group) * 512);
             out[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
         }
     }
 }
-
-__global__ void set_one_kernel(float *amax) { *amax = 1.0f; }
 
 int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
                           uint8_t *sf, float *amax, hipStream_t s) {
@@ -147,9 +165,8 @@ int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld,
     p.vector_loads = (((uintptr_t)x & 15) == 0) && (ld % 8 == 0);
     const int64_t grid = (p.rows_p / 128) * p.tiles_x;
     if (grid > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
-    hipLaunchKernelGGL(quantize_mxfp4_kernel, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
-    // the format has no tensor scale; the reference reports amax = 1 (reference.py:573-578)
-    hipLaunchKernelGGL(set_one_kernel, dim3(1), dim3(1), 0, s, amax);
+    p.amax = amax;
+    hipLaunchKernelGGL(quantize_mxfp4_kernel, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
