@@ -1,7 +1,10 @@
 """``FourOverSixLinear``: ``nn.Linear`` whose forward quantizes the activations on the fly
 and multiplies them with a (pre-)quantized weight on the FP4 GEMM
-(reference ``src/fouroversix/model/modules/linear.py:43-94, 291-453``; forward pass only,
-the reference's quantized backward is training machinery outside this library).
+(reference ``src/fouroversix/model/modules/linear.py:43-94, 291-453``), and whose backward
+(``keep_master_weights=True``) computes both gradients on the FP4 GEMM as well
+(``linear.py:96-288``, without the Quartet-II variant): dgrad from the stochastically
+rounded gradient and the weight quantized along its other dimension, wgrad from the
+transposed, random-Hadamard-rotated gradient and activations.
 
 The quantized weight lives in four buffers with the reference's names and shapes --
 ``quantized_weight_values`` u8 [out, in/2], ``quantized_weight_scale_factors`` E4M3 flat,
@@ -17,7 +20,8 @@ import torch
 import torch.nn as nn
 
 from fouroversix_amd.matmul import quantized_matmul
-from fouroversix_amd.quantize import QuantizedTensor, quantize
+from fouroversix_amd.quantize import QuantizedTensor, dequantize, quantize
+from fouroversix_amd.utils import DataType
 
 from .config import ModuleQuantizationConfig
 from .quantize import QuantizedModule
@@ -50,6 +54,64 @@ def fp4_linear(
     if bias is not None:
         out = out + bias
     return out
+
+
+class FourOverSixLinearFunction(torch.autograd.Function):
+    """Differentiable FP4 linear layer (reference ``linear.py:40-288``)."""
+
+    @staticmethod
+    def forward(ctx, config: ModuleQuantizationConfig, input: torch.Tensor, weight, bias=None) -> torch.Tensor:
+        if isinstance(weight, nn.Parameter):
+            ctx.config = config
+            ctx.save_for_backward(input, weight, bias)
+        return fp4_linear(config, input, weight, bias)
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        input, weight, bias = ctx.saved_tensors
+        cfg: ModuleQuantizationConfig = ctx.config
+        if cfg.quartet_ii_dtype is not None:
+            msg = "the Quartet-II backward is not implemented"
+            raise NotImplementedError(msg)
+        out_dtype = cfg.output_dtype.torch_dtype
+        g = grad_output.reshape(-1, grad_output.shape[-1])  # [tokens, out]
+        x = input.reshape(-1, input.shape[-1])              # [tokens, in]
+        w = weight.data
+
+        # dgrad = g @ W: W is quantized along its other dimension (blocks along `out`)
+        grad_input = None
+        if ctx.needs_input_grad[1]:
+            g_cfg = cfg.get_gradient_config()
+            w_cfg = cfg.get_weight_config(transpose=True)
+            if cfg.disable_dgrad_quantization == "quantize_grad_only":
+                gq = dequantize(quantize(g, g_cfg), torch.float32)
+                grad_input = torch.matmul(gq, w.float()).to(out_dtype)
+            elif cfg.disable_dgrad_quantization:
+                grad_input = torch.matmul(g, w)
+            elif cfg.pseudo_quantize:
+                grad_input = torch.matmul(quantize(g, g_cfg), quantize(w, w_cfg).T)
+            else:
+                grad_input = quantized_matmul(g, w, backend=cfg.matmul_backend, input_config=g_cfg, other_config=w_cfg,
+                                              out_dtype=cfg.output_dtype)
+            grad_input = grad_input.reshape(*grad_output.shape[:-1], weight.shape[1])
+
+        # wgrad = g^T @ x: both operands transposed and rotated by the random Hadamard
+        # transform along the token dimension (the rotation cancels in the product)
+        grad_weight = None
+        if ctx.needs_input_grad[2]:
+            extra = {"dtype": DataType.nvint4} if cfg.wgrad_nvint4 else {}
+            g_cfg = cfg.get_gradient_config(rht=True, transpose=True, **extra)
+            x_cfg = cfg.get_activation_config(rht=True, transpose=True, **extra)
+            if cfg.disable_wgrad_quantization:
+                grad_weight = torch.matmul(g.T, x)
+            elif cfg.pseudo_quantize:
+                grad_weight = torch.matmul(quantize(g, g_cfg), quantize(x, x_cfg).T)
+            else:
+                grad_weight = quantized_matmul(g, x, backend=cfg.matmul_backend, input_config=g_cfg, other_config=x_cfg,
+                                               out_dtype=cfg.output_dtype)
+
+        grad_bias = g.sum(0) if bias is not None and ctx.needs_input_grad[3] else None
+        return None, grad_input, grad_weight, grad_bias
 
 
 @QuantizedModule.register(nn.Linear)
@@ -142,4 +204,4 @@ class FourOverSixLinear(nn.Linear):
         return self._quantized_weight
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return fp4_linear(self.config, input, self.quantized_weight(), self.bias)
+        return FourOverSixLinearFunction.apply(self.config, input, self.quantized_weight(), self.bias)

@@ -192,3 +192,51 @@ def test_gemm_alpha_kernel_matches_the_reference_expression():
         got = fos.matmul.frontend.gemm_alpha(qa, qb)
         assert got.dtype == torch.float32 and got.shape == (1,)
         assert torch.equal(got.view(torch.int32), expect.view(torch.int32))
+
+
+def test_linear_backward_on_the_fp4_gemm():
+    """keep_master_weights=True: forward and both gradients run on the FP4 GEMM
+    (reference model/modules/linear.py:96-288).  The gradients equal the explicit
+    composition of the public calls under the same torch seed (the stochastic-rounding
+    seeds come from torch's generator) and are close to the fp32 gradients."""
+    torch.manual_seed(0)
+    tokens, k, n = 256, 512, 384
+    lin = nn.Linear(k, n, bias=True, dtype=torch.bfloat16).cuda()
+    cfg = fos.ModelQuantizationConfig(keep_master_weights=True)
+    model = nn.Sequential(lin)
+    fos.quantize_model(model, cfg)
+    layer = model[0]
+    assert isinstance(layer, fos.FourOverSixLinear) and isinstance(layer.weight, nn.Parameter)
+    x = torch.randn(1, tokens, k, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    g = torch.randn(1, tokens, n, device="cuda", dtype=torch.bfloat16)
+
+    torch.manual_seed(123)
+    y = layer(x)
+    y.backward(g)
+    gx, gw, gb = x.grad.clone(), layer.weight.grad.clone(), layer.bias.grad.clone()
+    assert gx.shape == x.shape and gw.shape == layer.weight.shape and gb.shape == (n,)
+
+    # explicit composition, same seed stream: dgrad draws first, then the two wgrad operands
+    torch.manual_seed(123)
+    mc = layer.config
+    g2, x2, w = g.reshape(-1, n), x.detach().reshape(-1, k), layer.weight.data
+    e_gx = fos.quantized_matmul(g2, w, input_config=mc.get_gradient_config(), other_config=mc.get_weight_config(transpose=True))
+    e_gw = fos.quantized_matmul(g2, x2, input_config=mc.get_gradient_config(rht=True, transpose=True),
+                                other_config=mc.get_activation_config(rht=True, transpose=True))
+    assert torch.equal(gx.reshape(-1, k), e_gx) and torch.equal(gw, e_gw)
+    assert torch.equal(gb, g2.sum(0))
+
+    # against full precision
+    rx = g2.float() @ w.float()
+    rw = g2.float().T @ x2.float()
+    ry = x2.float() @ w.float().T + layer.bias.float()
+    rel = lambda a, b: float((a.detach().float() - b).norm() / b.norm())  # noqa: E731
+    assert rel(y.reshape(-1, n), ry) < 0.2 and rel(gx.reshape(-1, k), rx) < 0.25 and rel(gw, rw) < 0.25
+
+    # unquantized gradient paths
+    for kw in (dict(disable_dgrad_quantization=True, disable_wgrad_quantization=True), dict(pseudo_quantize=True)):
+        layer.config = fos.ModelQuantizationConfig(keep_master_weights=True, **kw)
+        x.grad = None
+        layer.weight.grad = None
+        layer(x).backward(g)
+        assert rel(x.grad.reshape(-1, k), rx) < 0.25 and rel(layer.weight.grad, rw) < 0.25
