@@ -327,7 +327,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
     constexpr int kRowsPerPass = kThreadsG / 4;  // 4 lanes cover the 64 bytes of a row
     constexpr int PA = BM / kRowsPerPass, PB = BN / kRowsPerPass;
-    static_assert(PA == 2 && PB == 2 && WM * 32 <= 128 && WN * 32 <= 128, "tile shape: staged in two halves");
+    static_assert(PA % 2 == 0 && PB % 2 == 0 && WM * 32 <= 128 && WN * 32 <= 128, "tile shape: staged in two halves");
     extern __shared__ __attribute__((aligned(16))) uint8_t mx_lds[];
     uint8_t *lds_a[2] = {mx_lds, mx_lds + (BM + BN) * kMxPitch};
     uint8_t *lds_b[2] = {mx_lds + BM * kMxPitch, mx_lds + (BM + BN) * kMxPitch + BM * kMxPitch};
@@ -380,8 +380,12 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
     };
     // half q of the staged registers -> LDS stage `buf`
     auto stage_part = [&](const Staged &s, int buf, int q) {
-        *reinterpret_cast<uint4 *>(lds_a[buf] + lds_off + q * kRowsPerPass * kMxPitch) = s.a[q];
-        *reinterpret_cast<uint4 *>(lds_b[buf] + lds_off + q * kRowsPerPass * kMxPitch) = s.b[q];
+#pragma unroll
+        for (int i = q * (PA / 2); i < (q + 1) * (PA / 2); ++i)
+            *reinterpret_cast<uint4 *>(lds_a[buf] + lds_off + i * kRowsPerPass * kMxPitch) = s.a[i];
+#pragma unroll
+        for (int i = q * (PB / 2); i < (q + 1) * (PB / 2); ++i)
+            *reinterpret_cast<uint4 *>(lds_b[buf] + lds_off + i * kRowsPerPass * kMxPitch) = s.b[i];
     };
 
     mx_v16f acc[WM][WN];
