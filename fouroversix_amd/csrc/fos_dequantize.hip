@@ -21,19 +21,19 @@ struct DequantParams {
     int vector_stores;  // out and ldo allow 16-byte stores of whole blocks
 };
 
-// One thread per 1x16 block (consecutive threads = consecutive blocks of a row: 512
-// contiguous bytes of codes in, 2 KiB of bf16 out per wavefront).  `p.fast_div`: the divisor
-// is one of the constants for which the 3-operation division is exact; it is used when amax
-// is far enough from the ends of the float range for every quotient to be normal or zero.
+// One thread per 8 consecutive elements, i.e. half a 1x16 block (consecutive threads =
+// consecutive octets of a row: a wavefront reads 256 contiguous bytes of codes and writes
+// 1 KiB per store instruction).  `p.fast_div`: the divisor is one of the constants for which
+// the 3-operation division is exact; it is used when amax is far enough from the ends of
+// the float range for every quotient to be normal or zero.
 template <int DT, int OUT>
 __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) {
     const int64_t sf_cols = p.cols_p >> 4;
-    const int64_t blk = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t bpr = (p.cols + 15) >> 4;
-    const int64_t n_blocks = p.rows * bpr;
-    if (blk >= n_blocks) return;
-    const int64_t r = blk / bpr, cb = blk - r * bpr;
-    const uint2 q = *reinterpret_cast<const uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8);
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t opr = (p.cols + 7) >> 3;  // octets per row
+    if (idx >= p.rows * opr) return;
+    const int64_t r = idx / opr, oc = idx - r * opr, cb = oc >> 1;
+    const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
     const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
                              ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
                              : r * sf_cols + cb;
@@ -42,20 +42,20 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
     const float sf = e4m3_decode(sb & 0x7fu);
 
     // value * scale, as the fp16 product of the reference (exact for E2M1 values)
-    float f[16];
+    float f[8];
     if (DT == FOS_DTYPE_IF4 && (sb & 0x80u)) {
         const _Float16 s16 = (_Float16)sf;
         const float six_sevenths = (float)(6.0 / 7.0);
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const uint32_t code = ((i < 8 ? q.x : q.y) >> (4 * (i & 7))) & 0xfu;
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t code = (q >> (4 * i)) & 0xfu;
             const int iv = ((int)(code << 28)) >> 28;
             f[i] = (float)((_Float16)((float)iv * six_sevenths) * s16);
         }
     } else {
-        static_for<0, 8>([&](auto jc) {
+        static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
-            const float2_t v = unpack_fp4<(j & 3)>(j < 4 ? q.x : q.y);
+            const float2_t v = unpack_fp4<j>(q);
             f[2 * j] = v.x * sf;
             f[2 * j + 1] = v.y * sf;
         });
@@ -63,32 +63,32 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
     if (p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f) {
         const float rc = 1.0f / p.divisor;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
+        for (int i = 0; i < 8; ++i) {
             const float t = f[i] * amax;
             f[i] = u2f((f2u(div_const(t, p.divisor, rc)) & 0x7fffffffu) | (f2u(t) & 0x80000000u));
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) f[i] = (f[i] * amax) / p.divisor;
+        for (int i = 0; i < 8; ++i) f[i] = (f[i] * amax) / p.divisor;
     }
 
-    const int64_t c0 = cb * 16;
-    const bool whole = p.vector_stores && c0 + 16 <= p.cols;
+    const int64_t c0 = oc * 8;
+    const bool whole = p.vector_stores && c0 + 8 <= p.cols;
     if (OUT == FOS_T_F32) {
         float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
         if (whole) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v) reinterpret_cast<float4 *>(o)[v] = make_float4(f[4 * v], f[4 * v + 1], f[4 * v + 2], f[4 * v + 3]);
+            reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
+            reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
+            for (int i = 0; i < 8; ++i)
                 if (c0 + i < p.cols) o[i] = f[i];
         }
         return;
     }
-    uint32_t w[8];
+    uint32_t w[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 4; ++j) {
         const float2_t v = {f[2 * j], f[2 * j + 1]};
         if (OUT == FOS_T_F16) {
             typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
@@ -100,11 +100,10 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
     }
     uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
     if (whole) {
-        reinterpret_cast<uint4 *>(o)[0] = make_uint4(w[0], w[1], w[2], w[3]);
-        reinterpret_cast<uint4 *>(o)[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        *reinterpret_cast<uint4 *>(o) = make_uint4(w[0], w[1], w[2], w[3]);
     } else {
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
+        for (int i = 0; i < 8; ++i)
             if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
     }
 }
@@ -145,7 +144,7 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;
     if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
     if (out_type != FOS_T_BF16 && out_type != FOS_T_F16 && out_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
-    if (((uintptr_t)codes & 7) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
+    if (((uintptr_t)codes & 3) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
     DequantParams p;
     p.codes = codes; p.sf = sf; p.amax = amax; p.out = out;
     p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
@@ -154,9 +153,9 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.fast_div = p.divisor == 1536.0f || p.divisor == 1792.0f || p.divisor == 2688.0f;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
-    const int64_t n_blocks = rows * ((cols + 15) / 16);
-    if ((n_blocks + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
-    dim3 grid((unsigned)((n_blocks + 255) / 256));
+    const int64_t n_octets = rows * ((cols + 7) / 8);
+    if ((n_octets + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    dim3 grid((unsigned)((n_octets + 255) / 256));
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FOS_DTYPE_IF4) launch_dequant<FOS_DTYPE_IF4>(p, out_type, grid, s);
     else launch_dequant<FOS_DTYPE_NVFP4>(p, out_type, grid, s);

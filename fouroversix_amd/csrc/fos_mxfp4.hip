@@ -184,47 +184,48 @@ struct MxDequantParams {
 
 typedef _Float16 mx_half2_t __attribute__((ext_vector_type(2)));
 
-// One thread per 1x32 block.  value (fp16) * fp16(2^(e - 127)), product in fp16: scales
-// outside fp16's range turn into 0 / inf there, as in the reference.
+// One thread per 8 consecutive elements (a quarter of a 1x32 block; a wavefront reads 256
+// contiguous bytes of codes and writes 1 KiB per store instruction).  value (fp16) *
+// fp16(2^(e - 127)), product in fp16: scales outside fp16's range turn into 0 / inf there,
+// as in the reference.
 template <int OUT>
 __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantParams p) {
     const int64_t sf_cols = p.cols_p >> 5;
-    const int64_t bpr = (p.cols + 31) >> 5;
-    const int64_t blk = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (blk >= p.rows * bpr) return;
-    const int64_t r = blk / bpr, cb = blk - r * bpr;
-    const uint4 q = *reinterpret_cast<const uint4 *>(p.codes + r * (p.cols_p >> 1) + cb * 16);
+    const int64_t opr = (p.cols + 7) >> 3;  // octets per row
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= p.rows * opr) return;
+    const int64_t r = idx / opr, oc = idx - r * opr, cb = oc >> 2;
+    const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
     const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
                              ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
                              : r * sf_cols + cb;
     const uint32_t e = p.sf[sofs];
     const _Float16 s16 = (_Float16)(e == 0u ? u2f(0x00400000u) : u2f(e << 23));
     const mx_half2_t s2 = {s16, s16};
-    const uint32_t words[4] = {q.x, q.y, q.z, q.w};
-    float f[32];
-    static_for<0, 16>([&](auto jc) {
+    float f[8];
+    static_for<0, 4>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
-        const mx_half2_t v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(words[j >> 2], 1.0f, j & 3) * s2;
+        const mx_half2_t v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 1.0f, j) * s2;
         f[2 * j] = (float)v.x;
         f[2 * j + 1] = (float)v.y;
     });
-    const int64_t c0 = cb * 32;
-    const bool whole = p.vector_stores && c0 + 32 <= p.cols;
+    const int64_t c0 = oc * 8;
+    const bool whole = p.vector_stores && c0 + 8 <= p.cols;
     if (OUT == FOS_T_F32) {
         float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
         if (whole) {
-#pragma unroll
-            for (int v = 0; v < 8; ++v) reinterpret_cast<float4 *>(o)[v] = make_float4(f[4 * v], f[4 * v + 1], f[4 * v + 2], f[4 * v + 3]);
+            reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
+            reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
         } else {
 #pragma unroll
-            for (int i = 0; i < 32; ++i)
+            for (int i = 0; i < 8; ++i)
                 if (c0 + i < p.cols) o[i] = f[i];
         }
         return;
     }
-    uint32_t w[16];
+    uint32_t w[4];
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
+    for (int j = 0; j < 4; ++j) {
         const float2_t v = {f[2 * j], f[2 * j + 1]};
         if (OUT == FOS_T_F16) {
             w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
@@ -235,11 +236,10 @@ __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantPa
     }
     uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
     if (whole) {
-#pragma unroll
-        for (int v = 0; v < 4; ++v) reinterpret_cast<uint4 *>(o)[v] = make_uint4(w[4 * v], w[4 * v + 1], w[4 * v + 2], w[4 * v + 3]);
+        *reinterpret_cast<uint4 *>(o) = make_uint4(w[0], w[1], w[2], w[3]);
     } else {
 #pragma unroll
-        for (int i = 0; i < 32; ++i)
+        for (int i = 0; i < 8; ++i)
             if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
     }
 }
@@ -247,16 +247,16 @@ __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantPa
 int launch_dequantize_mxfp4(const uint8_t *codes, const uint8_t *sf, int sf_layout, int64_t rows, int64_t cols,
                             int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, hipStream_t s) {
     if (cols_p % 32 != 0 || (sf_layout == FOS_SF_TILED_128X4 && cols_p % 128 != 0)) return FOS_E_BAD_SHAPE;
-    if ((uintptr_t)codes & 15) return FOS_E_BAD_ALIGNMENT;
+    if ((uintptr_t)codes & 3) return FOS_E_BAD_ALIGNMENT;
     MxDequantParams p;
     p.codes = codes; p.sf = sf; p.out = out;
     p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
     p.sf_layout = sf_layout;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
-    const int64_t n_blocks = rows * ((cols + 31) / 32);
-    if ((n_blocks + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
-    dim3 grid((unsigned)((n_blocks + 255) / 256));
+    const int64_t n_octets = rows * ((cols + 7) / 8);
+    if ((n_octets + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    dim3 grid((unsigned)((n_octets + 255) / 256));
     if (out_type == FOS_T_F32) hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_F32>, grid, dim3(256), 0, s, p);
     else if (out_type == FOS_T_F16) hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_F16>, grid, dim3(256), 0, s, p);
     else hipLaunchKernelGGL(dequantize_mxfp4_kernel<FOS_T_BF16>, grid, dim3(256), 0, s, p);
