@@ -124,10 +124,13 @@ template <bool SR>
 FOS_DEVICE float e2m1_round(float a, float u) {
     float r;
     if (SR) {
-        float r1 = __builtin_rintf((a + a) + u) * 0.5f;
-        float r2 = __builtin_rintf(a + u);
-        float r3 = fminf(2.0f * __builtin_rintf(a * 0.5f + u), 6.0f);
-        r = a < 2.0f ? r1 : (a < 4.0f ? r2 : r3);
+        // one rounding on the regime's grid: step 2^k, k = -1 (a < 2), 0 (a < 4), 1 (else),
+        // read off the exponent field; the scalings by 2^k are exact, so this is the
+        // reference's rint(2a + u) / 2, rint(a + u), 2 rint(a / 2 + u)
+        const int e = (int)((f2u(a) >> 23) & 0xffu);
+        const int k = (e < 127 ? 127 : (e > 129 ? 129 : e)) - 128;
+        r = __builtin_ldexpf(__builtin_rintf(__builtin_ldexpf(a, -k) + u), k);
+        r = fminf(r, 6.0f);
         r = (r == 0.0f) ? 0.0f : r;
     } else {
         float r1 = __builtin_rintf(a + a) * 0.5f;
@@ -207,6 +210,18 @@ FOS_DEVICE float error_term(float deq, float x) {
     return RULE == FOS_RULE_MSE ? d * d : fabsf(d);
 }
 
+// 16 values on the E2M1 grid (|v| <= 6) -> two words of packed codes (element i in nibble i).
+FOS_DEVICE void pack16_fp4(const float *v, uint32_t &c0, uint32_t &c1) {
+    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v[0], v[1], 1.0f, 0);
+    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[2], v[3], 1.0f, 1);
+    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[4], v[5], 1.0f, 2);
+    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[6], v[7], 1.0f, 3);
+    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v[8], v[9], 1.0f, 0);
+    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[10], v[11], 1.0f, 1);
+    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[12], v[13], 1.0f, 2);
+    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[14], v[15], 1.0f, 3);
+}
+
 // Dither for the 16 elements of 1x16 block `blk`, candidate `cand`: one Philox4x32-10
 // call keyed (seed; blk, cand, offset), one byte per element.
 FOS_DEVICE void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float *u) {
@@ -242,13 +257,25 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
 
     if (STATIC) {
         uint32_t c0 = 0, c1 = 0;
+        if (SR) {
+            // dithered values lie on the grid and are clamped to 6, so the hardware convert
+            // packs them exactly; x * inv + 0 drops the sign of a zero product, as `xs < 0` does
+            float fq[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            float xs = (sA != 0) ? x[i] * invA : 0.0f;
-            float r = e2m1_round<SR>(fabsf(xs), SR ? uA[i] : 0.0f);
-            uint32_t nib = e2m1_mag_code(r) | ((xs < 0.0f) ? 8u : 0u);
-            if (i < 8) c0 |= nib << (4 * i);
-            else c1 |= nib << (4 * (i - 8));
+            for (int i = 0; i < 16; ++i) {
+                const float xs = (sA != 0) ? __builtin_fmaf(x[i], invA, 0.0f) : 0.0f;
+                fq[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xs), uA[i]), xs);
+            }
+            pack16_fp4(fq, c0, c1);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float xs = (sA != 0) ? x[i] * invA : 0.0f;
+                float r = e2m1_round<false>(fabsf(xs), 0.0f);
+                uint32_t nib = e2m1_mag_code(r) | ((xs < 0.0f) ? 8u : 0u);
+                if (i < 8) c0 |= nib << (4 * i);
+                else c1 |= nib << (4 * (i - 8));
+            }
         }
         codes[0] = c0;
         codes[1] = c1;
@@ -293,21 +320,36 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
     uint32_t sB;
     float sfB, invB;
     block_scale(k, bmax, true, sB, sfB, invB);
+    if (SR) {
+        float fqA[16], fqB[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        float xsA = (sA != 0) ? x[i] * invA : 0.0f;
-        float xsB = (sB != 0) ? x[i] * invB : 0.0f;
-        float rA = e2m1_round<SR>(fabsf(xsA), SR ? uA[i] : 0.0f);
-        float rB = e2m1_round<SR>(fabsf(xsB), SR ? uB[i] : 0.0f);
-        bool negA = xsA < 0.0f, negB = xsB < 0.0f;
-        uint32_t nibA = e2m1_mag_code(rA) | (negA ? 8u : 0u);
-        uint32_t nibB = e2m1_mag_code(rB) | (negB ? 8u : 0u);
-        float deqA = div_errdiv(((negA ? -rA : rA) * sfA) * k.amax, k);
-        float deqB = div_errdiv(((negB ? -rB : rB) * sfB) * k.amax, k);
-        eA[i] = error_term<RULE>(deqA, x[i]);
-        eB[i] = error_term<RULE>(deqB, x[i]);
-        if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
-        else { a1 |= nibA << (4 * (i - 8)); b1 |= nibB << (4 * (i - 8)); }
+        for (int i = 0; i < 16; ++i) {
+            const float xsA = (sA != 0) ? __builtin_fmaf(x[i], invA, 0.0f) : 0.0f;
+            const float xsB = (sB != 0) ? __builtin_fmaf(x[i], invB, 0.0f) : 0.0f;
+            fqA[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xsA), uA[i]), xsA);
+            fqB[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xsB), uB[i]), xsB);
+            eA[i] = error_term<RULE>(div_errdiv((fqA[i] * sfA) * k.amax, k), x[i]);
+            eB[i] = error_term<RULE>(div_errdiv((fqB[i] * sfB) * k.amax, k), x[i]);
+        }
+        pack16_fp4(fqA, a0, a1);
+        pack16_fp4(fqB, b0, b1);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            float xsA = (sA != 0) ? x[i] * invA : 0.0f;
+            float xsB = (sB != 0) ? x[i] * invB : 0.0f;
+            float rA = e2m1_round<false>(fabsf(xsA), 0.0f);
+            float rB = e2m1_round<false>(fabsf(xsB), 0.0f);
+            bool negA = xsA < 0.0f, negB = xsB < 0.0f;
+            uint32_t nibA = e2m1_mag_code(rA) | (negA ? 8u : 0u);
+            uint32_t nibB = e2m1_mag_code(rB) | (negB ? 8u : 0u);
+            float deqA = div_errdiv(((negA ? -rA : rA) * sfA) * k.amax, k);
+            float deqB = div_errdiv(((negB ? -rB : rB) * sfB) * k.amax, k);
+            eA[i] = error_term<RULE>(deqA, x[i]);
+            eB[i] = error_term<RULE>(deqB, x[i]);
+            if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
+            else { a1 |= nibA << (4 * (i - 8)); b1 |= nibB << (4 * (i - 8)); }
+        }
     }
     float errA = reduce_error<RULE, TWO_D>(eA);
     float errB = reduce_error<RULE, TWO_D>(eB);
