@@ -197,21 +197,29 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
             if (kk + 1 < BK / 16) read_frags(buf, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
-            if (have_next) {
-                stage_quarter(nxt, buf ^ 1, kk);
-                if (kk + 1 == BK / 16) {
-                    __syncthreads();
-                    read_frags(buf ^ 1, 0, fa[0], fb[0]);
-                    // keep this slice's MFMAs below the barrier (the scheduler would
-                    // otherwise hoist them and leave the matrix pipe idle behind it)
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+            if (have_next) stage_quarter(nxt, buf ^ 1, kk);
+            const bool at_barrier = have_next && kk + 1 == BK / 16;
+            auto mfmas = [&](int i_begin, int i_end) {
+#pragma unroll
+                for (int i = i_begin; i < i_end; ++i)
+#pragma unroll
+                    for (int j = 0; j < WN; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
+            };
+            if (at_barrier) {
+                // half of the last slice's MFMAs go above the barrier, where they overlap the
+                // last quarter's dequantisation, and half below it, where they cover the LDS
+                // latency of the next step's first fragments (the scheduler must not move
+                // them across: either side would leave the matrix pipe idle)
+                mfmas(0, WM / 2);
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                read_frags(buf ^ 1, 0, fa[0], fb[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                mfmas(WM / 2, WM);
+            } else {
+                mfmas(0, WM);
             }
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-#pragma unroll
-                for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i], acc[i][j], 0, 0, 0);
             // slices are scheduled one at a time: a wider window only raises register pressure
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -219,17 +227,16 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 
     using yes = std::integral_constant<bool, true>;
     using no = std::integral_constant<bool, false>;
+    // Steps go in pairs (the two LDS buffers and register sets alternate by name).  The
+    // last pair stages the clamped prefetch -- the final step's data once more -- into the
+    // buffer nobody reads again, which is cheaper than a separate copy of the loop body
+    // for the end of the K range; an odd step count leaves one step without staging.
     int64_t ks = 0;
-    for (; ks + 2 < ksteps; ks += 2) {
+    for (; ks + 2 <= ksteps; ks += 2) {
         kstep(yes{}, ks, 0, st[0], st[1]);
         kstep(yes{}, ks + 1, 1, st[1], st[0]);
     }
-    if (ks + 2 == ksteps) {
-        kstep(yes{}, ks, 0, st[0], st[1]);
-        kstep(no{}, ks + 1, 1, st[1], st[0]);
-    } else {
-        kstep(no{}, ks, 0, st[0], st[1]);
-    }
+    if (ks < ksteps) kstep(no{}, ks, 0, st[0], st[1]);
 
     // epilogue: acc[i][j][4*g + e] is D[m][n] with m = wm*WM*32 + i*32 + (lane & 31),
     // n = wn*WN*32 + j*32 + 8*g + 4*(lane >> 5) + e

@@ -80,7 +80,8 @@ int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, 
  * quantize/pytorch/reference.py:555-679): the input is zero-padded to
  * (fos_padded_rows, fos_padded_cols) and every padded output element is written.
  *
- *   x_type      FOS_T_BF16 or FOS_T_F16
+ *   x_type      FOS_T_BF16 (the only input type implemented; anything else returns
+ *               FOS_E_UNSUPPORTED)
  *   dtype       FOS_DTYPE_*; rule FOS_RULE_* (IF4 takes only the adaptive rules)
  *   round_style FOS_ROUND_*; seed/offset key the Philox dither of the stochastic styles
  *   block2d     non-zero: one scale and one decision per 16x16 tile
