@@ -117,28 +117,15 @@ FOS_DEVICE void block_scale(const QuantConsts &k, float bmax, bool expand, uint3
     inv = 1.0f / (k.dec * sf);
 }
 
-// E2M1 grid rounding of a magnitude (reference.py:30-51).  Round-to-nearest has no clamp
-// (a magnitude in [7, 9) gives 8, which the nibble encoding below spills into bit 3
-// exactly as the reference's bit extraction does); the dithered variant clamps to 6.
-template <bool SR>
-FOS_DEVICE float e2m1_round(float a, float u) {
-    float r;
-    if (SR) {
-        // one rounding on the regime's grid: step 2^k, k = -1 (a < 2), 0 (a < 4), 1 (else),
-        // read off the exponent field; the scalings by 2^k are exact, so this is the
-        // reference's rint(2a + u) / 2, rint(a + u), 2 rint(a / 2 + u)
-        const int e = (int)((f2u(a) >> 23) & 0xffu);
-        const int k = (e < 127 ? 127 : (e > 129 ? 129 : e)) - 128;
-        r = __builtin_ldexpf(__builtin_rintf(__builtin_ldexpf(a, -k) + u), k);
-        r = fminf(r, 6.0f);
-        r = (r == 0.0f) ? 0.0f : r;
-    } else {
-        float r1 = __builtin_rintf(a + a) * 0.5f;
-        float r2 = __builtin_rintf(a);
-        float r3 = 2.0f * __builtin_rintf(a * 0.5f);
-        r = a < 2.0f ? r1 : (a < 4.0f ? r2 : r3);
-    }
-    return r;
+// E2M1 grid rounding of a magnitude, round to nearest (reference.py:30-51): no clamp (a
+// magnitude in [7, 9) gives 8, which the nibble encoding below spills into bit 3 exactly
+// as the reference's bit extraction does).  The stochastic styles round with the
+// hardware convert (sr_pack16), which clamps to 6 as the reference's dithered branch does.
+FOS_DEVICE float e2m1_round(float a) {
+    float r1 = __builtin_rintf(a + a) * 0.5f;
+    float r2 = __builtin_rintf(a);
+    float r3 = 2.0f * __builtin_rintf(a * 0.5f);
+    return a < 2.0f ? r1 : (a < 4.0f ? r2 : r3);
 }
 
 // Grid magnitude {0,.5,1,1.5,2,3,4,6,(8)} -> 3-bit code (8 for the overflow value).
@@ -210,25 +197,11 @@ FOS_DEVICE float error_term(float deq, float x) {
     return RULE == FOS_RULE_MSE ? d * d : fabsf(d);
 }
 
-// 16 values on the E2M1 grid (|v| <= 6) -> two words of packed codes (element i in nibble i).
-FOS_DEVICE void pack16_fp4(const float *v, uint32_t &c0, uint32_t &c1) {
-    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v[0], v[1], 1.0f, 0);
-    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[2], v[3], 1.0f, 1);
-    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[4], v[5], 1.0f, 2);
-    c0 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c0, v[6], v[7], 1.0f, 3);
-    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v[8], v[9], 1.0f, 0);
-    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[10], v[11], 1.0f, 1);
-    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[12], v[13], 1.0f, 2);
-    c1 = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(c1, v[14], v[15], 1.0f, 3);
-}
-
-// Dither for the 16 elements of 1x16 block `blk`, candidate `cand`: one Philox4x32-10
-// call keyed (seed; blk, cand, offset), one byte per element.
-FOS_DEVICE void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float *u) {
-    const Philox4 p = philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset,
-                                    (uint32_t)seed, (uint32_t)(seed >> 32));
-#pragma unroll
-    for (int i = 0; i < 16; ++i) u[i] = dither_from_byte(p.v[i >> 2], i & 3);
+// Random words for the 16 elements of 1x16 block `blk`, candidate `cand`: one
+// Philox4x32-10 call keyed (seed; blk, cand, offset).
+FOS_DEVICE Philox4 block_philox(uint64_t seed, uint64_t offset, uint64_t blk, int cand) {
+    return philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset, (uint32_t)seed,
+                         (uint32_t)(seed >> 32));
 }
 
 // One 1x16 block (one row of a 16x16 tile when TWO_D): 8 input words -> 2 code words
@@ -252,26 +225,25 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
     uint32_t sA;
     float sfA, invA;
     block_scale(k, bmax, false, sA, sfA, invA);
-    float uA[16], uB[16];
-    if (SR) dither16(seed, offset, blk, 0, uA);
+    // x * inv + 0 drops the sign of a zero product, as the reference's sign(x) does
+    auto scaled = [&](uint32_t s, float inv, float *xs) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xs[i] = (s != 0) ? __builtin_fmaf(x[i], inv, 0.0f) : 0.0f;
+    };
+    Philox4 pA, pB;
+    if (SR) pA = block_philox(seed, offset, blk, 0);
 
     if (STATIC) {
         uint32_t c0 = 0, c1 = 0;
         if (SR) {
-            // dithered values lie on the grid and are clamped to 6, so the hardware convert
-            // packs them exactly; x * inv + 0 drops the sign of a zero product, as `xs < 0` does
-            float fq[16];
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float xs = (sA != 0) ? __builtin_fmaf(x[i], invA, 0.0f) : 0.0f;
-                fq[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xs), uA[i]), xs);
-            }
-            pack16_fp4(fq, c0, c1);
+            float xs[16];
+            scaled(sA, invA, xs);
+            sr_pack16(xs, pA, c0, c1);
         } else {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float xs = (sA != 0) ? x[i] * invA : 0.0f;
-                float r = e2m1_round<false>(fabsf(xs), 0.0f);
+                float r = e2m1_round(fabsf(xs));
                 uint32_t nib = e2m1_mag_code(r) | ((xs < 0.0f) ? 8u : 0u);
                 if (i < 8) c0 |= nib << (4 * i);
                 else c1 |= nib << (4 * (i - 8));
@@ -283,28 +255,41 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
         return;
     }
 
-    if (SR) dither16(seed, offset, blk, 1, uB);
+    if (SR) pB = block_philox(seed, offset, blk, 1);
     float eA[16], eB[16];
     uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
 
     if (DT == FOS_DTYPE_IF4) {
         // select_intfloat (reference.py:328-425): candidate A = E2M1, candidate B = INT4
         // on the same scale; B wins on a strictly smaller error.
+        float xsS[16], fqS[16];
+        if (SR) {
+            scaled(sA, invA, xsS);
+            sr_pack16(xsS, pA, a0, a1);
+            unpack16_fp4(a0, a1, fqS);
+        }
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             float xs = (sA != 0) ? x[i] * invA : 0.0f;
-            float r = e2m1_round<SR>(fabsf(xs), SR ? uA[i] : 0.0f);
-            bool neg = xs < 0.0f;
-            float fq = neg ? -r : r;
-            uint32_t nibA = e2m1_mag_code(r) | (neg ? 8u : 0u);
-            float q = int4_round<SR>(xs * 1.16666666f, SR ? uB[i] : 0.0f);
+            float fq;
+            if (SR) {
+                fq = fqS[i];
+            } else {
+                float r = e2m1_round(fabsf(xs));
+                bool neg = xs < 0.0f;
+                fq = neg ? -r : r;
+                uint32_t nibA = e2m1_mag_code(r) | (neg ? 8u : 0u);
+                if (i < 8) a0 |= nibA << (4 * i);
+                else a1 |= nibA << (4 * (i - 8));
+            }
+            float q = int4_round<SR>(xs * 1.16666666f, SR ? dither_from_byte(pB.v[i >> 2], i & 3) : 0.0f);
             uint32_t nibB = (uint32_t)((int)q) & 0xfu;
             float deqA = div_errdiv((fq * sfA) * k.amax, k);
             float deqB = div_errdiv(((q * sfA) * k.amax) * 0.8571428571f, k);
             eA[i] = error_term<RULE>(deqA, x[i]);
             eB[i] = error_term<RULE>(deqB, x[i]);
-            if (i < 8) { a0 |= nibA << (4 * i); b0 |= nibB << (4 * i); }
-            else { a1 |= nibA << (4 * (i - 8)); b1 |= nibB << (4 * (i - 8)); }
+            if (i < 8) b0 |= nibB << (4 * i);
+            else b1 |= nibB << (4 * (i - 8));
         }
         float errA = reduce_error<RULE, TWO_D>(eA);
         float errB = reduce_error<RULE, TWO_D>(eB);
@@ -321,25 +306,25 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
     float sfB, invB;
     block_scale(k, bmax, true, sB, sfB, invB);
     if (SR) {
-        float fqA[16], fqB[16];
+        float xsA[16], xsB[16], fqA[16], fqB[16];
+        scaled(sA, invA, xsA);
+        scaled(sB, invB, xsB);
+        sr_pack16(xsA, pA, a0, a1);
+        sr_pack16(xsB, pB, b0, b1);
+        unpack16_fp4(a0, a1, fqA);
+        unpack16_fp4(b0, b1, fqB);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float xsA = (sA != 0) ? __builtin_fmaf(x[i], invA, 0.0f) : 0.0f;
-            const float xsB = (sB != 0) ? __builtin_fmaf(x[i], invB, 0.0f) : 0.0f;
-            fqA[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xsA), uA[i]), xsA);
-            fqB[i] = __builtin_copysignf(e2m1_round<true>(fabsf(xsB), uB[i]), xsB);
             eA[i] = error_term<RULE>(div_errdiv((fqA[i] * sfA) * k.amax, k), x[i]);
             eB[i] = error_term<RULE>(div_errdiv((fqB[i] * sfB) * k.amax, k), x[i]);
         }
-        pack16_fp4(fqA, a0, a1);
-        pack16_fp4(fqB, b0, b1);
     } else {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             float xsA = (sA != 0) ? x[i] * invA : 0.0f;
             float xsB = (sB != 0) ? x[i] * invB : 0.0f;
-            float rA = e2m1_round<false>(fabsf(xsA), 0.0f);
-            float rB = e2m1_round<false>(fabsf(xsB), 0.0f);
+            float rA = e2m1_round(fabsf(xsA));
+            float rB = e2m1_round(fabsf(xsB));
             bool negA = xsA < 0.0f, negB = xsB < 0.0f;
             uint32_t nibA = e2m1_mag_code(rA) | (negA ? 8u : 0u);
             uint32_t nibB = e2m1_mag_code(rB) | (negB ? 8u : 0u);

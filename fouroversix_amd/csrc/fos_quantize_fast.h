@@ -31,30 +31,6 @@
 
 namespace fos {
 
-typedef float float2_t __attribute__((ext_vector_type(2)));
-
-// Compile-time loop: f(std::integral_constant<int, I>) for I = 0 .. N-1 (the convert
-// builtins take their byte selector as an immediate).
-template <int I, int N, class F>
-FOS_DEVICE void static_for(F &&f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
-
-// Two floats -> two E2M1 nibbles (a low, b high) into byte SEL of `old`.
-template <int SEL>
-FOS_DEVICE uint32_t pack_fp4(uint32_t old, float a, float b) {
-    return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, SEL);
-}
-
-// Byte SEL of `word` -> the two E2M1 values (low nibble in .x).
-template <int SEL>
-FOS_DEVICE float2_t unpack_fp4(uint32_t word) {
-    return __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, SEL);
-}
-
 struct FastLutEntry {
     float inv;       // 1 / (dec * s)                       (0 for s == 0)
     float d1;        // RN((s * amax) / errdiv)             factor for fq in {.5, 1, 2, 4}
@@ -248,12 +224,12 @@ __device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantCo
             const int idx = l + 8 * h;
             const float x = block_element(w, idx);
             const float xsA = (sA != 0) ? x * invA : 0.0f;
-            const float rA = e2m1_round<false>(fabsf(xsA), 0.0f);
+            const float rA = e2m1_round(fabsf(xsA));
             const bool negA = xsA < 0.0f;
             ca |= (uint64_t)(e2m1_mag_code(rA) | (negA ? 8u : 0u)) << (4 * idx);
             if (!STATIC) {
                 const float xsB = (sB != 0) ? x * invB : 0.0f;
-                const float rB = e2m1_round<false>(fabsf(xsB), 0.0f);
+                const float rB = e2m1_round(fabsf(xsB));
                 const bool negB = xsB < 0.0f;
                 cb |= (uint64_t)(e2m1_mag_code(rB) | (negB ? 8u : 0u)) << (4 * idx);
                 const float deqA = (((negA ? -rA : rA) * sfA) * k.amax) / k.errdiv;

@@ -56,6 +56,8 @@ def lib() -> ctypes.CDLL:
         L.fos_oracle_e4m3_to_f32.restype = f32
         L.fos_oracle_e2m1_rtn.argtypes = [f32]
         L.fos_oracle_e2m1_rtn.restype = f32
+        L.fos_oracle_e2m1_sr_code.argtypes = [f32, c.c_uint32]
+        L.fos_oracle_e2m1_sr_code.restype = c.c_uint8
         L.fos_oracle_e2m1_decode.argtypes = [c.c_uint8]
         L.fos_oracle_e2m1_decode.restype = f32
         L.fos_oracle_sum16.argtypes = [vp]

@@ -18,7 +18,7 @@
  *   src/fouroversix/matmul/pytorch.py          quantized_matmul :33-52
  *   src/fouroversix/kernels/constants.py       IF4 expansion constants :4-5
  *
- * Parity pins (tests/test_oracle_*.py): E4M3 cast vs torch's own cast over a full sweep;
+ * Parity pins (tests/test_oracle.py): E4M3 cast vs torch's own cast over a full sweep;
  * E2M1 rounding vs the reference's threshold table over every bf16 value; the 16- and
  * 256-element summation orders vs torch.sum; closed forms for zeros / ones / rand01;
  * golden vectors written by the reference itself (tests/golden); the if4_mac golden
@@ -115,16 +115,36 @@ float fos_oracle_e2m1_rtn(float xs) {
     return sign_of(xs) * r;
 }
 
-/* reference.py:39-44: dither u in [-0.5,0.5) added before each rint; the regime is
- * chosen by the undithered magnitude; only the top regime is clamped (to 6).  A zero
- * result is canonicalised to +0 before the sign is applied. */
-static float e2m1_sr(float xs, float u) {
-    float a = fabsf(xs), r;
-    if (a < 2.0f) r = rintf(2.0f * a + u) / 2.0f;
-    else if (a < 4.0f) r = rintf(a + u);
-    else { r = 2.0f * rintf(a / 2.0f + u); if (r > 6.0f) r = 6.0f; }
-    if (r == 0.0f) r = 0.0f;
-    return sign_of(xs) * r;
+/* Stochastic rounding of a scaled value to an E2M1 code (reference.py:39-44 adds
+ * U[-0.5, 0.5) before the rint of the magnitude's regime and clamps to 6).  Restated in
+ * the form the gfx950 convert V_CVT_SCALEF32_SR_PK_FP4_F32 implements, so that kernel and
+ * oracle agree bit for bit: the top 22 bits of `rword` are added to the discarded bits
+ * of the significand, aligned to their top, and the sum is truncated -- rounding up with
+ * probability (discarded fraction) to within 2^-22; saturation at 6; the sign is kept,
+ * also on a zero result.  M = 1.m * 2^23 (0.m * 2^23 for a sub-normal float), d = 22
+ * discarded bits for |x| >= 1 and 22 - exponent below, q = (M + (R << (d - 22))) >> d
+ * counts half-steps of the binade (of 1 below 1.0). */
+uint8_t fos_oracle_e2m1_sr_code(float xs, uint32_t rword) {
+    uint32_t b;
+    memcpy(&b, &xs, 4);
+    uint32_t sign = b >> 31, exp = (b >> 23) & 0xffu, mant = b & 0x7fffffu;
+    uint32_t code;
+    if (exp == 255) {
+        code = 7;
+    } else {
+        uint64_t M = exp ? (mant | 0x800000u) : mant;
+        int e = exp ? (int)exp - 127 : -126;
+        int d = e >= 0 ? 22 : 22 - e;
+        uint64_t R = rword >> 10;
+        uint64_t q = d >= 46 ? 0 : (M + (R << (d - 22))) >> d;
+        if (e >= 0) {
+            uint64_t c = 2 * (uint64_t)(e > 8 ? 8 : e) + q;
+            code = c > 7 ? 7 : (uint32_t)c;
+        } else {
+            code = (uint32_t)q;
+        }
+    }
+    return (uint8_t)(code | (sign << 3));
 }
 
 /* reference.py:54-63 */
@@ -215,20 +235,25 @@ void fos_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint
     memcpy(out, c, 16);
 }
 
-/* Dither for the 16 elements of 1x16 block `blk` (= row * blocks_per_row + block column
- * of the padded tensor), candidate `cand`: ONE Philox4x32-10 call with counter
- * (blk_lo, blk_hi, cand, offset_lo) and key (seed_lo, seed_hi); element i takes byte
- * i % 4 of word i / 4: u = (byte + 0.5) / 256 - 0.5, i.e. 256 equally likely values that
- * are symmetric about zero (8 random bits per element, as hardware stochastic-rounding
- * converts consume; the reference draws from torch's generator, so its stream cannot be
- * matched bit for bit anyway). */
-static void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float u[16]) {
+/* Random words for the 16 elements of 1x16 block `blk` (= row * blocks_per_row + block
+ * column of the padded tensor), candidate `cand`: ONE Philox4x32-10 call with counter
+ * (blk_lo, blk_hi, cand, offset_lo) and key (seed_lo, seed_hi).  Element i belongs to byte
+ * i % 4 of word i / 4.  E2M1 rounding takes the word rotated so that this byte leads
+ * (rw[i]; the convert uses its top 22 bits: the leading 8 are the element's own, the rest
+ * come from its three neighbours at 1/256 of the weight); the INT4 candidate of IF4 takes
+ * u = (byte + 0.5) / 256 - 0.5, 256 equally likely values symmetric about zero.  The
+ * reference draws from torch's generator, so its stream cannot be matched bit for bit. */
+static void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float u[16], uint32_t rw[16]) {
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset};
     uint32_t w[4];
     fos_oracle_philox4x32_10(ctr, key, w);
-    for (int i = 0; i < 16; ++i)
-        u[i] = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xffu) * 0.00390625f - 0.498046875f;
+    for (int i = 0; i < 16; ++i) {
+        uint32_t word = w[i >> 2];
+        int sh = (8 * ((i & 3) + 1)) & 31;
+        u[i] = (float)((word >> (8 * (i & 3))) & 0xffu) * 0.00390625f - 0.498046875f;
+        rw[i] = sh ? ((word >> sh) | (word << (32 - sh))) : word;
+    }
 }
 
 /* ---- quantize ---------------------------------------------------------------------- */
@@ -247,7 +272,7 @@ typedef struct {
 
 /* compute_nv_scale_factors (reference.py:184-241) for one block. */
 static void scale_block(const qctx *q, const float *x, int n, float bmax, int expand,
-                        uint8_t *s_out, float *xs) {
+                        uint8_t *s_out, float *xs, float *inv_out) {
     float s_hp;
     if (q->amax == 0.0f) s_hp = 0.0f;
     else s_hp = (bmax / q->qdiv) * q->enc;
@@ -257,6 +282,7 @@ static void scale_block(const qctx *q, const float *x, int n, float bmax, int ex
     float inv = 1.0f / (q->dec * sf);
     for (int i = 0; i < n; ++i) xs[i] = (s != 0) ? x[i] * inv : 0.0f;
     *s_out = s;
+    *inv_out = inv;
 }
 
 static float block_error(int rule, const float *deq, const float *x, int n) {
@@ -275,9 +301,18 @@ static float block_error(int rule, const float *deq, const float *x, int n) {
 
 /* Fill the dither for every element of an n-element block (n = 16, or 256 for a 16x16
  * tile whose r-th row is 1x16 block blk0 + r * blocks_per_row). */
-static void block_dither(const qctx *q, uint64_t blk0, int n, int cand, float *u) {
+static void block_dither(const qctx *q, uint64_t blk0, int n, int cand, float *u, uint32_t *rw) {
     for (int r = 0; r < n / 16; ++r)
-        dither16(q->seed, q->offset, blk0 + (uint64_t)r * (uint64_t)q->blocks_per_row, cand, u + 16 * r);
+        dither16(q->seed, q->offset, blk0 + (uint64_t)r * (uint64_t)q->blocks_per_row, cand, u + 16 * r, rw + 16 * r);
+}
+
+/* E2M1 candidate of one block with stochastic rounding: x * inv + 0 (one rounding; the
+ * sign of a zero product is dropped, as the reference's sign(x) does), then the convert. */
+static void e2m1_sr_block(const float *x, int n, uint8_t s, float inv, const uint32_t *rw, float *fq) {
+    for (int i = 0; i < n; ++i) {
+        float xs = (s != 0) ? fmaf(x[i], inv, 0.0f) : 0.0f;
+        fq[i] = fos_oracle_e2m1_decode(fos_oracle_e2m1_sr_code(xs, rw[i]));
+    }
 }
 
 /* One block (16 or 256 floats): writes fake-quantized values fq[n], whether they are
@@ -286,25 +321,34 @@ static void quantize_block(const qctx *q, const float *x, int n, uint64_t blk0,
                            float *fq, int *is_int, uint8_t *s_out) {
     float bmax = 0.0f;
     for (int i = 0; i < n; ++i) { float a = fabsf(x[i]); if (a > bmax) bmax = a; }
-    float xs6[256], xs4[256], f6[256], f4[256], d6[256], d4[256], u[256];
+    float xs6[256], xs4[256], f6[256], f4[256], d6[256], d4[256], u[256], inv6, inv4;
+    uint32_t rw[256];
     uint8_t s6, s4;
     int sr = q->round_style != ROUND_NEAREST;
     *is_int = 0;
 
     if (q->rule == RULE_STATIC6 || q->rule == RULE_STATIC4) {
-        scale_block(q, x, n, bmax, 0, &s6, xs6);
-        if (sr) block_dither(q, blk0, n, 0, u);
-        for (int i = 0; i < n; ++i) fq[i] = sr ? e2m1_sr(xs6[i], u[i]) : fos_oracle_e2m1_rtn(xs6[i]);
+        scale_block(q, x, n, bmax, 0, &s6, xs6, &inv6);
+        if (sr) {
+            block_dither(q, blk0, n, 0, u, rw);
+            e2m1_sr_block(x, n, s6, inv6, rw, fq);
+        } else {
+            for (int i = 0; i < n; ++i) fq[i] = fos_oracle_e2m1_rtn(xs6[i]);
+        }
         *s_out = s6;
         return;
     }
 
     if (q->dtype == FOS_IF4) { /* select_intfloat, reference.py:328-425 */
-        scale_block(q, x, n, bmax, 0, &s6, xs6);
+        scale_block(q, x, n, bmax, 0, &s6, xs6, &inv6);
         float sf = fos_oracle_e4m3_to_f32(s6);
-        if (sr) block_dither(q, blk0, n, 0, u);
-        for (int i = 0; i < n; ++i) f6[i] = sr ? e2m1_sr(xs6[i], u[i]) : fos_oracle_e2m1_rtn(xs6[i]);
-        if (sr) block_dither(q, blk0, n, 1, u);
+        if (sr) {
+            block_dither(q, blk0, n, 0, u, rw);
+            e2m1_sr_block(x, n, s6, inv6, rw, f6);
+            block_dither(q, blk0, n, 1, u, rw);
+        } else {
+            for (int i = 0; i < n; ++i) f6[i] = fos_oracle_e2m1_rtn(xs6[i]);
+        }
         for (int i = 0; i < n; ++i) {
             float y = xs6[i] * 1.16666666f;
             f4[i] = sr ? int4_sr(y, u[i]) : int4_rtn(y);
@@ -323,12 +367,17 @@ static void quantize_block(const qctx *q, const float *x, int n, uint64_t blk0,
     }
 
     /* 4/6 adaptive, reference.py:519-552 and 262-325 */
-    scale_block(q, x, n, bmax, 0, &s6, xs6);
-    scale_block(q, x, n, bmax, 1, &s4, xs4);
-    if (sr) block_dither(q, blk0, n, 0, u);
-    for (int i = 0; i < n; ++i) f6[i] = sr ? e2m1_sr(xs6[i], u[i]) : fos_oracle_e2m1_rtn(xs6[i]);
-    if (sr) block_dither(q, blk0, n, 1, u);
-    for (int i = 0; i < n; ++i) f4[i] = sr ? e2m1_sr(xs4[i], u[i]) : fos_oracle_e2m1_rtn(xs4[i]);
+    scale_block(q, x, n, bmax, 0, &s6, xs6, &inv6);
+    scale_block(q, x, n, bmax, 1, &s4, xs4, &inv4);
+    if (sr) {
+        block_dither(q, blk0, n, 0, u, rw);
+        e2m1_sr_block(x, n, s6, inv6, rw, f6);
+        block_dither(q, blk0, n, 1, u, rw);
+        e2m1_sr_block(x, n, s4, inv4, rw, f4);
+    } else {
+        for (int i = 0; i < n; ++i) f6[i] = fos_oracle_e2m1_rtn(xs6[i]);
+        for (int i = 0; i < n; ++i) f4[i] = fos_oracle_e2m1_rtn(xs4[i]);
+    }
     float sf6 = fos_oracle_e4m3_to_f32(s6), sf4 = fos_oracle_e4m3_to_f32(s4);
     for (int i = 0; i < n; ++i) {
         d6[i] = ((f6[i] * sf6) * q->amax) / q->errdiv;
