@@ -150,9 +150,19 @@ template <int DT, int RULE>
 void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, hipStream_t s) {
     if (round_style == FOS_ROUND_NEAREST) {
         // NVFP4 round-to-nearest lives in fos_quantize_fast.hip
-        if constexpr (DT == FOS_DTYPE_NVFP4) launch_quantize_nvfp4_rtn(p, RULE, two_d, aligned, s);
+        if constexpr (DT == FOS_DTYPE_NVFP4) launch_quantize_nvfp4_fast(p, RULE, two_d, aligned, false, s);
         else dispatch_2d<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, aligned, s);
     } else {
+        // ... and so does stochastic rounding of aligned inputs (the unbiased style differs
+        // in the host-computed constants only; the MSE rule decides through its certified
+        // shortcut there and the other adaptive rules stay with the generic kernel)
+        if constexpr (DT == FOS_DTYPE_NVFP4) {
+            constexpr bool kShortcut = RULE == FOS_RULE_MSE || RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
+            if (aligned && (round_style == FOS_ROUND_STOCHASTIC || kShortcut)) {
+                launch_quantize_nvfp4_fast(p, RULE, two_d, aligned, true, s);
+                return;
+            }
+        }
         dispatch_2d<DT, RULE, FOS_ROUND_STOCHASTIC>(p, two_d, aligned, s);
     }
 }

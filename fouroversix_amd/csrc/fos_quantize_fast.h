@@ -249,10 +249,21 @@ __device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantCo
     return BlockOut{(uint32_t)c, (uint32_t)(c >> 32), pickB ? sB : sA};
 }
 
-// One 1x16 block, NVFP4 round-to-nearest, any rule; falls back by itself.
+// Operation-by-operation form for the stochastic style (quantize_block, out of line).
 template <int RULE, bool TWO_D>
-FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
-                                             bool in_range, const FastLutEntry *lut) {
+__device__ __attribute__((noinline)) BlockOut generic_block_sr(Block16 blk, QuantConsts k, uint64_t seed, uint64_t offset,
+                                                              uint64_t blkid) {
+    uint32_t codes[2], sbyte;
+    quantize_block<FOS_DTYPE_NVFP4, RULE, FOS_ROUND_STOCHASTIC, TWO_D>(blk.w, k, seed, offset, blkid, codes, sbyte);
+    return BlockOut{codes[0], codes[1], sbyte};
+}
+
+// One 1x16 block, NVFP4, any rule, round to nearest or (SR) a stochastic style; falls
+// back by itself.  `blkid` = row * (cols_p / 16) + block column keys the dither.
+template <int RULE, bool TWO_D, bool SR>
+FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
+                                              bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
+                                              uint64_t blkid) {
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
     if (in_range) {
         float x[16];
@@ -270,7 +281,12 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
         for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
         if (TWO_D) bmax = row16_max(bmax);
 
-        const float s_hp6 = div_const(bmax, k.qdiv, rq) * enc;
+        // the 3-operation division is exact for the divisors 6 and 4 (every bf16 numerator);
+        // the unbiased stochastic style rescales them, and f32(6 * 16 / 17) is not
+        float bq;
+        if (SR && k.qdiv != 6.0f && k.qdiv != 4.0f) bq = bmax / k.qdiv;
+        else bq = div_const(bmax, k.qdiv, rq);
+        const float s_hp6 = bq * enc;
         const float s_hp4 = s_hp6 * 1.5f;
         const uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp6, s_hp4, 0, false);
         const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
@@ -279,8 +295,66 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
         // rounded down by more than 7/6 (only candidate "6" can get there).  A zero scale
         // byte of a non-zero block has no scaled domain at all.  Everything else -- normal
         // and sub-normal scales alike -- is exact on the fast path.
+        // The stochastic style clamps to 6 in the reference as well, so only the zero scale
+        // byte is left out there.
         const FastLutEntry A = lut[s6];
-        if (s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f)) {
+        if (SR ? s6 != 0u : (s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f))) {
+            if constexpr (SR) {
+                // scaled values, hardware stochastic rounding (one Philox call per candidate);
+                // the certified shortcut holds unchanged: its bound does not use how far a
+                // rounded value may lie from the scaled one
+                float xa[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) xa[i] = x[i] * A.inv;
+                const Philox4 pA = block_philox(seed, offset, blkid, 0);
+                uint32_t a0, a1;
+                sr_pack16(xa, pA, a0, a1);
+                if (STATIC) return BlockOut{a0, a1, s6};
+                const FastLutEntry B = lut[s4];
+                float xb[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) xb[i] = x[i] * B.inv;
+                const Philox4 pB = block_philox(seed, offset, blkid, 1);
+                uint32_t b0, b1;
+                sr_pack16(xb, pB, b0, b1);
+                bool pickB = false, certain = false;
+                if (RULE == FOS_RULE_MSE) {
+                    float SA = 0.0f, SB = 0.0f;
+                    static_for<0, 8>([&](auto jc) {
+                        constexpr int j = decltype(jc)::value;
+                        const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+                        const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
+                        const float ra0 = fa.x - xa[2 * j], ra1 = fa.y - xa[2 * j + 1];
+                        const float rb0 = fb.x - xb[2 * j], rb1 = fb.y - xb[2 * j + 1];
+                        SA = __builtin_fmaf(ra0, ra0, SA);
+                        SA = __builtin_fmaf(ra1, ra1, SA);
+                        SB = __builtin_fmaf(rb0, rb0, SB);
+                        SB = __builtin_fmaf(rb1, rb1, SB);
+                    });
+                    if (TWO_D) {
+                        SA = row16_sum_lane0(SA);
+                        SB = row16_sum_lane0(SB);
+                    }
+                    constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
+                    constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
+                    const float hA = A.d1 * A.d1, hB = B.d1 * B.d1;
+                    const float EA = hA * SA, EB = hB * SB;
+                    const float tA = hA * __builtin_fmaf(k1, SA, k0);
+                    const float tB = hB * __builtin_fmaf(k1, SB, k0);
+                    const bool surely_b = EB + tB < EA - tA;
+                    const bool surely_a = EB - tB > EA + tA;
+                    certain = surely_a || surely_b;
+                    pickB = surely_b;
+                }
+                if (!certain) {
+                    bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
+                    if (TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
+                    if (tie) pickB = false;
+                    else if (k.errdiv == 1536.0f) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                    else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // the unbiased style's divisor
+                }
+                return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
+            }
             if (STATIC) {
                 uint32_t c0 = 0, c1 = 0;
                 static_for<0, 4>([&](auto jc) {
@@ -345,7 +419,8 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_rtn(const Block16 &blk, const QuantCons
         }
         if (bmax == 0.0f) return BlockOut{0, 0, 0};  // an all-zero block: zero codes, zero scale
     }
-    return generic_block<RULE, TWO_D>(blk, k);
+    if constexpr (SR) return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);
+    else return generic_block<RULE, TWO_D>(blk, k);
 }
 
 // The 16 dequantised values of a quantised NVFP4 block as bf16 pairs, with the operations

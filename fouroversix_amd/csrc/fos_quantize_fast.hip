@@ -1,14 +1,14 @@
-// Pass 2 for NVFP4 with round-to-nearest, around the fast block formulation of
-// fos_quantize_fast.h.  Two lane mappings:
+// Pass 2 for NVFP4 with round-to-nearest or plain stochastic rounding, around the fast
+// block formulation of fos_quantize_fast.h.  Two lane mappings:
 //
-//  * 1x16 blocks (quantize_nvfp4_rtn_rows_kernel): a wavefront covers 4 rows x 16 blocks,
+//  * 1x16 blocks (quantize_nvfp4_rows_kernel): a wavefront covers 4 rows x 16 blocks,
 //    i.e. 512 contiguous bytes per row.  Measured on MI355X, a wavefront that touches 16
 //    rows x 128 bytes streams at ~4.1 TB/s while 4 rows x 512 bytes reaches ~6 TB/s, so the
 //    row-contiguous mapping is what the HBM-bound path uses.  A 256-thread workgroup
 //    covers 128 rows x 256 columns in eight steps of 16 rows (the next step's loads are
 //    issued before the current step is processed), stages the 4 complete 128x4 scale
 //    tiles in LDS and writes them as one contiguous 2 KiB run.
-//  * 16x16 tiles (quantize_nvfp4_rtn_kernel): the 16 rows of a tile must lie along one DPP
+//  * 16x16 tiles (quantize_nvfp4_tile_kernel): the 16 rows of a tile must lie along one DPP
 //    row for the tile reductions, so a wavefront covers 16 rows x 4 blocks; persistent
 //    workgroups walk over 128 x 64 tiles with the next tile prefetched.
 #include <cstdlib>
@@ -39,8 +39,8 @@ FOS_DEVICE void load_tile(const QuantParams &p, uint32_t tile, int lane, int wav
     }
 }
 
-template <int RULE, bool TWO_D, bool PSEUDO>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_kernel(const QuantParams p) {
+template <int RULE, bool TWO_D, bool PSEUDO, bool SR>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_tile_kernel(const QuantParams p) {
     __shared__ uint32_t red[4];
     __shared__ uint32_t sf_tile[2][128];
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
@@ -73,7 +73,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         for (int h = 0; h < 2; ++h) {
             const int rr = h * 64 + wave * 16 + (lane & 15);
             const int64_t r = tile_y * 128 + rr;
-            const BlockOut o = quantize_block_nvfp4_rtn<RULE, TWO_D>(t.b[h], k, enc_fast, rq, maybe_negzero, in_range, lut);
+            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, SR>(t.b[h], k, enc_fast, rq, maybe_negzero, in_range, lut,
+                                                                          p.seed, p.offset, (uint64_t)(r * sf_cols + cb));
             if (PSEUDO) {
                 uint32_t w[8];
                 if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
@@ -117,8 +118,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 // within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns; workgroups stride
 // over the tiles so that the per-workgroup setup (tensor maximum, scale table) is paid
 // once for several tiles.  FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
-template <int RULE, bool FULL, bool PSEUDO>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rtn_rows_kernel(
+template <int RULE, bool FULL, bool PSEUDO, bool SR>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
     __shared__ uint32_t sf_stage[2][4 * 128];  // 4 scale tiles of 512 bytes, double-buffered
@@ -178,7 +179,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             if (g + 2 < 8) load(g + 2, blk[g + 2]);
             if (col_ok) {
                 const int rr = g * 16 + rr0;
-                const BlockOut o = quantize_block_nvfp4_rtn<RULE, false>(blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut);
+                const BlockOut o = quantize_block_nvfp4_fast<RULE, false, SR>(
+                    blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut, p.seed, p.offset,
+                    (uint64_t)((row0 + g * 16) * sf_cols + cb));
                 if (PSEUDO) {
                     uint32_t w[8];
                     if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
@@ -209,10 +212,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     }
 }
 
-template <int RULE, bool PSEUDO>
+template <int RULE, bool PSEUDO, bool SR>
 static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     if (!aligned) {
-        if (PSEUDO) return;  // rejected by the entry point
+        if (PSEUDO || SR) return;  // rejected by the entry point / routed to the generic kernel
         if (two_d) launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
         else launch_quantize<true, FOS_DTYPE_NVFP4, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
         return;
@@ -227,9 +230,9 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         if (grid > n) grid = n;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
         if (full)
-            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+            hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else
-            hipLaunchKernelGGL((quantize_nvfp4_rtn_rows_kernel<RULE, false, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+            hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         return;
     }
     p.tiles_x = (int)(p.cols_p / 64);
@@ -239,26 +242,30 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     int64_t grid = 256 * 6;
     if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
     if (grid > n_tiles) grid = n_tiles;
-    hipLaunchKernelGGL((quantize_nvfp4_rtn_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL((quantize_nvfp4_tile_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
-template <bool PSEUDO>
+template <bool PSEUDO, bool SR>
 static void by_rule(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {
     switch (rule) {
         case FOS_RULE_STATIC_6:
         case FOS_RULE_STATIC_4:
             // the two static rules differ only in the host-computed constants
-            by_dim<FOS_RULE_STATIC_6, PSEUDO>(p, two_d, aligned, s);
+            by_dim<FOS_RULE_STATIC_6, PSEUDO, SR>(p, two_d, aligned, s);
             break;
-        case FOS_RULE_MAE: by_dim<FOS_RULE_MAE, PSEUDO>(p, two_d, aligned, s); break;
-        case FOS_RULE_MSE: by_dim<FOS_RULE_MSE, PSEUDO>(p, two_d, aligned, s); break;
-        default: by_dim<FOS_RULE_ABS_MAX, PSEUDO>(p, two_d, aligned, s); break;
+        case FOS_RULE_MAE: by_dim<FOS_RULE_MAE, PSEUDO, SR>(p, two_d, aligned, s); break;
+        case FOS_RULE_MSE: by_dim<FOS_RULE_MSE, PSEUDO, SR>(p, two_d, aligned, s); break;
+        default: by_dim<FOS_RULE_ABS_MAX, PSEUDO, SR>(p, two_d, aligned, s); break;
     }
 }
 
-void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s) {
-    if (p.pseudo_out) by_rule<true>(p, rule, two_d, aligned, s);
-    else by_rule<false>(p, rule, two_d, aligned, s);
+// `sr`: a stochastic style on an aligned input.  The fast exact evaluation is tied to the
+// selection divisor 1536; with the unbiased style's rescaled divisor an inconclusive
+// shortcut falls back to the operation-by-operation form.
+void launch_quantize_nvfp4_fast(QuantParams &p, int rule, bool two_d, bool aligned, bool sr, hipStream_t s) {
+    if (sr) by_rule<false, true>(p, rule, two_d, aligned, s);
+    else if (p.pseudo_out) by_rule<true, false>(p, rule, two_d, aligned, s);
+    else by_rule<false, false>(p, rule, two_d, aligned, s);
 }
 
 }  // namespace fos

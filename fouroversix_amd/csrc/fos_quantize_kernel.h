@@ -94,7 +94,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
             Block16 blk;
 #pragma unroll
             for (int i = 0; i < 8; ++i) blk.w[i] = w[it][i];
-            const BlockOut o = quantize_block_nvfp4_rtn<RULE, TWO_D>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut);
+            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, false>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut, 0, 0, 0);
             codes[0] = o.c0;
             codes[1] = o.c1;
             sbyte = o.s;
@@ -154,8 +154,9 @@ void launch_quantize(QuantParams &p, bool aligned, hipStream_t s) {
     }
 }
 
-// Defined in fos_quantize_fast.hip: NVFP4, round to nearest, any rule.
-void launch_quantize_nvfp4_rtn(QuantParams &p, int rule, bool two_d, bool aligned, hipStream_t s);
+// Defined in fos_quantize_fast.hip: NVFP4, any rule, round to nearest or (sr, aligned inputs
+// only) a stochastic style.
+void launch_quantize_nvfp4_fast(QuantParams &p, int rule, bool two_d, bool aligned, bool sr, hipStream_t s);
 
 // MXFP4 (fos_mxfp4.hip)
 int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,

@@ -155,7 +155,8 @@ def test_reference_op_schema(oracle):
 
 @pytest.mark.parametrize(("dtype", "rule", "two_d"), [
     ("nvfp4", "static_6", False), ("nvfp4", "mse", False), ("nvfp4", "mse", True), ("if4", "mse", False),
-    ("nvfp4", "abs_max", False),
+    ("nvfp4", "abs_max", False), ("nvfp4", "mae", False), ("nvfp4", "static_4", True), ("nvfp4", "mae", True),
+    ("if4", "abs_max", True),
 ])
 @pytest.mark.parametrize("style", ["stochastic", "stochastic_unbiased"])
 def test_stochastic_rounding_bit_exact_with_oracle_key(oracle, dtype, rule, two_d, style):
@@ -167,6 +168,43 @@ def test_stochastic_rounding_bit_exact_with_oracle_key(oracle, dtype, rule, two_
     assert_same_quantization(q, ref, str(kw))
     q2 = hip_quantize(x, kwargs={"seed": 100, "offset": 3}, **kw)
     assert (u8(q2.values) != u8(q.values)).mean() > 0.05
+
+
+@pytest.mark.parametrize("style", ["stochastic", "stochastic_unbiased"])
+def test_stochastic_rounding_edge_cases_bit_exact(oracle, style):
+    """The stochastic styles on the inputs that steer the kernels off their main path:
+    ragged shapes (zero padding, partial tiles), tensors outside [2^-100, 2^100] and blocks
+    with sub-normal scales (operation-by-operation form), negative zeros, an input that is
+    only 2-byte aligned (generic kernel), outlier channels (exact ties between the candidates)."""
+    def check(x, what, **cfg):
+        kw = dict(round_style=style, **cfg)
+        q = hip_quantize(x, kwargs={"seed": 5, "offset": 1}, **kw)
+        assert_same_quantization(q, oracle.quantize(x.cpu().contiguous(), seed=5, offset=1, **kw), f"{what} {kw}")
+
+    for shape in ((100, 80), (1, 16), (257, 1000), (130, 272)):
+        x = make_input("randn", shape, 21)
+        check(x, f"ragged {shape}", scale_rule="mse")
+        check(x, f"ragged {shape}", scale_rule="static_6", block_scale_2d=True)
+        check(x, f"ragged {shape}", scale_rule="mse", block_scale_2d=True)
+    for scale in (2.0**-110, 2.0**105):
+        x = (make_input("randn", (256, 128), 12).float() * scale).bfloat16()
+        for two_d in (False, True):
+            check(x, f"scale {scale}", scale_rule="mse", block_scale_2d=two_d)
+            check(x, f"scale {scale}", scale_rule="static_6", block_scale_2d=two_d)
+    x = make_input("tiny_blocks", (256, 512), 22)
+    check(x, "tiny blocks", scale_rule="mse")
+    check(x, "tiny blocks", scale_rule="static_4")
+    x = make_input("randn", (256, 256), 13)
+    x[::3, ::5] = -0.0
+    x[1::7, 3::11] = -1e-4
+    check(x, "negative zeros", scale_rule="mse")
+    check(x, "negative zeros", scale_rule="static_6")
+    flat = make_input("randn", (1, 256 * 130 + 1), 5).cuda().reshape(-1)
+    odd = flat[1:].reshape(256, 130)[:, :128]   # 2-byte aligned only, ld 130
+    check(odd, "unaligned", scale_rule="mse")
+    x = make_input("outlier", (256, 1024), 23)
+    check(x, "outlier", scale_rule="mse")
+    check(x, "outlier", scale_rule="mse", block_scale_2d=True)
 
 
 def test_stochastic_rounding_known_answers():
