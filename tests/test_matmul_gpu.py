@@ -178,6 +178,37 @@ def test_linear_layer_forward(oracle):
     assert torch.equal(keep(x.cuda()), y)
 
 
+def test_linear_forward_replays_in_a_hip_graph():
+    """A decode-sized forward (quantize -> alpha -> weight-streaming GEMM, twice) captured in
+    a HIP graph: every replay, interleaved with eager work and synchronisations, equals
+    the eager result on fresh input contents."""
+    torch.manual_seed(1)
+    model = nn.Sequential(nn.Linear(1024, 2048, bias=False), nn.SiLU(), nn.Linear(2048, 1024, bias=True)).cuda().bfloat16()
+    fos.quantize_model(model, fos.ModelQuantizationConfig(weight_scale_2d=True))
+    for mod in model.modules():
+        if isinstance(mod, fos.FourOverSixLinear):
+            mod.quantize_weight_()
+    static_x = torch.randn(16, 1024, device="cuda").bfloat16()
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                model(static_x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_y = model(static_x)
+        for i in range(4):
+            xi = torch.randn(16, 1024, device="cuda").bfloat16() * (i + 1)
+            static_x.copy_(xi)
+            graph.replay()
+            torch.cuda.synchronize()
+            eager = model(xi)
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, eager), f"replay {i}"
+
+
 def test_gemm_alpha_kernel_matches_the_reference_expression():
     """alpha = (amaxA * amaxB) / (qA sA qB sB adjA adjB) with fp32 operations
     (reference matmul/cutlass/backend.py:86-98): the one-launch kernel against torch."""
