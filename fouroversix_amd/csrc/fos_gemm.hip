@@ -616,7 +616,10 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     }
     // split so that about kTargetWorkgroups workgroups run, each with a useful share of K
     const int64_t min_steps = g.kind == kPlanSkinny ? 8 : 4;
-    int64_t want = tiles >= kTargetWorkgroups / 2 ? 1 : (kTargetWorkgroups + tiles - 1) / tiles;
+    // (the weight-streaming kernel also splits in two when its workgroups would cover exactly
+    // half of the compute units: measured 18.8 -> 15.1 us at M = 16, N = 4096, K = 14336)
+    const int64_t enough = g.kind == kPlanSkinny ? kTargetWorkgroups / 2 + 1 : kTargetWorkgroups / 2;
+    int64_t want = tiles >= enough ? 1 : (kTargetWorkgroups + tiles - 1) / tiles;
     if (want > steps / min_steps) want = steps / min_steps;
     want = env_int("FOS_GEMM_SPLITK", (int)want);  // tuning / tests
     if (want > steps) want = steps;
