@@ -261,7 +261,7 @@ def test_linear_backward_on_the_fp4_gemm():
     rx = g2.float() @ w.float()
     rw = g2.float().T @ x2.float()
     ry = x2.float() @ w.float().T + layer.bias.float()
-    rel = lambda a, b: float((a.detach().float() - b).norm() / b.norm())  # noqa: E731
+    rel = lambda a, b: float((a.detach().float() - b.detach()).norm() / b.detach().norm())  # noqa: E731
     assert rel(y.reshape(-1, n), ry) < 0.2 and rel(gx.reshape(-1, k), rx) < 0.25 and rel(gw, rw) < 0.25
 
     # unquantized gradient paths
