@@ -97,6 +97,11 @@ struct QuantConsts {
     float amax, enc, dec, qdiv, errdiv;
     float rerr = 0.0f;      // RN(1 / errdiv)
     bool fast_div = false;  // errdiv is a constant with an exact 3-operation division and every quotient is normal or zero
+    // The fast exact evaluation of a candidate's error (one fma per element from a per-scale
+    // table) needs scale * amax to be exact in fp32 -- a tensor maximum with at most 8
+    // significant bits, which every maximum of bf16 data has but a caller-supplied one need
+    // not -- and the divisor 1536; without both, undecided blocks take the generic form.
+    bool exact_ok = false;
 };
 
 // v / k.errdiv with IEEE rounding (the sign of a zero quotient may differ; callers subtract).

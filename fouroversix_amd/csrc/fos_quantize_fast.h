@@ -350,8 +350,8 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
                     if (TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                     if (tie) pickB = false;
-                    else if (k.errdiv == 1536.0f) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
-                    else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // the unbiased style's divisor
+                    else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                    else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // e.g. the unbiased style's divisor
                 }
                 return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
             }
@@ -413,7 +413,9 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     // every row of the tile must agree
                     tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                 }
-                pickB = tie ? false : exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                if (tie) pickB = false;
+                else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                else return generic_block<RULE, TWO_D>(blk, k);
             }
             return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
         }

@@ -54,6 +54,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     k.dec = 1.0f / (p.c / k.amax);
     k.qdiv = p.qdiv;
     k.errdiv = p.errdiv;
+    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
@@ -134,6 +135,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     k.dec = 1.0f / (p.c / k.amax);
     k.qdiv = p.qdiv;
     k.errdiv = p.errdiv;
+    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;

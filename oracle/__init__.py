@@ -68,6 +68,8 @@ def lib() -> ctypes.CDLL:
         L.fos_oracle_philox4x32_10.restype = None
         L.fos_oracle_quantize.argtypes = [vp, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, i32]
         L.fos_oracle_quantize.restype = i32
+        L.fos_oracle_quantize_with_amax.argtypes = [vp, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, vp, i32]
+        L.fos_oracle_quantize_with_amax.restype = i32
         L.fos_oracle_blocked_offset.argtypes = [i64, i64, i64]
         L.fos_oracle_blocked_offset.restype = i64
         L.fos_oracle_to_blocked.argtypes = [vp, i64, i64, vp]
@@ -176,7 +178,7 @@ def transform(xb: np.ndarray, *, transpose=False, rht=False) -> np.ndarray:
 
 def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
              block_scale_2d=False, seed=0, offset=0, threads=None,
-             transpose=False, rht=False) -> OracleQuantized:
+             transpose=False, rht=False, amax=None) -> OracleQuantized:
     xb = bf16_bits(x)
     assert xb.ndim == 2
     if transpose or rht:
@@ -186,11 +188,12 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
     mp, np_ = xp.shape
     codes = np.zeros((mp, np_ // 2), dtype=np.uint8)
     sf = np.zeros((mp, np_ // 16), dtype=np.uint8)
+    amax_in = None if amax is None else np.array([amax], dtype=np.float32)
     amax = np.zeros(1, dtype=np.float32)
-    rc = lib().fos_oracle_quantize(
+    rc = lib().fos_oracle_quantize_with_amax(
         _ptr(xp), mp, np_, DTYPE_IDS[dtype], RULE_IDS[scale_rule], ROUND_IDS[round_style],
         int(block_scale_2d), seed, offset, _ptr(codes), _ptr(sf), _ptr(amax),
-        threads or default_threads(),
+        None if amax_in is None else _ptr(amax_in), threads or default_threads(),
     )
     if rc != 0:
         raise ValueError(f"oracle: unsupported combination {dtype}/{scale_rule}")

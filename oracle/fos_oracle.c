@@ -404,18 +404,25 @@ static double adj_of(int round_style) {
  *   amax  : f32 max|x|
  * Returns 0, or -1 on an unsupported combination.
  */
-int fos_oracle_quantize(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,
-                        int round_style, int block2d, uint64_t seed, uint64_t offset,
-                        uint8_t *codes, uint8_t *sf, float *amax_out, int nthreads) {
+/* `amax_in` (may be NULL) is the reference function's x_amax argument (reference.py:557,
+ * 573-578): the tensor scale to use instead of max|x|. */
+int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,
+                                  int round_style, int block2d, uint64_t seed, uint64_t offset,
+                                  uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                                  int nthreads) {
     if (N % 16 != 0 || (block2d && M % 16 != 0)) return -1;
     if (dtype != FOS_NVFP4 && dtype != FOS_IF4) return -1;
     if (dtype == FOS_IF4 && (rule == RULE_STATIC6 || rule == RULE_STATIC4)) return -1;
     if (rule < 0 || rule > 4) return -1;
 
     float amax = 0.0f;
-    for (int64_t i = 0; i < M * N; ++i) {
-        float a = fabsf(bf16_to_f32(x[i]));
-        if (a > amax) amax = a;
+    if (amax_in) {
+        amax = *amax_in;
+    } else {
+        for (int64_t i = 0; i < M * N; ++i) {
+            float a = fabsf(bf16_to_f32(x[i]));
+            if (a > amax) amax = a;
+        }
     }
     *amax_out = amax;
 
@@ -477,6 +484,13 @@ int fos_oracle_quantize(const uint16_t *x, int64_t M, int64_t N, int dtype, int 
         }
     }
     return 0;
+}
+
+int fos_oracle_quantize(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,
+                        int round_style, int block2d, uint64_t seed, uint64_t offset,
+                        uint8_t *codes, uint8_t *sf, float *amax_out, int nthreads) {
+    return fos_oracle_quantize_with_amax(x, M, N, dtype, rule, round_style, block2d, seed, offset, codes, sf,
+                                         amax_out, NULL, nthreads);
 }
 
 /* ---- scale layout ------------------------------------------------------------------ */

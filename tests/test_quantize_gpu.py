@@ -136,6 +136,18 @@ def test_caller_supplied_amax(oracle):
     amax = torch.tensor(float(ref.amax), device="cuda")
     q = fos.quantize(x.cuda(), fos.QuantizationConfig(kwargs={"amax": amax}))
     assert_same_quantization(q, ref, "amax given")
+    # a maximum that is not a bf16 value (24 significant bits, larger than max|x|), on inputs
+    # whose blocks tie or nearly tie: the undecided blocks must take the generic evaluation
+    for kind, shape in (("randn", (1024, 1024)), ("rand01", (256, 256)), ("outlier", (256, 1024))):
+        x = make_input(kind, shape, 7)
+        given = float(np.float32(float(x.abs().max()) * 1.2345678))
+        for cfg in (dict(scale_rule="mse"), dict(scale_rule="mse", block_scale_2d=True), dict(scale_rule="static_6"),
+                    dict(scale_rule="mse", round_style="stochastic", kwargs={"seed": 3})):
+            ocfg = {k: v for k, v in cfg.items() if k != "kwargs"}
+            ref = oracle.quantize(x, amax=given, seed=cfg.get("kwargs", {}).get("seed", 0), **ocfg)
+            kw = dict(cfg.get("kwargs", {}), amax=torch.tensor(given, device="cuda"))
+            q = fos.quantize(x.cuda(), fos.QuantizationConfig(**{**ocfg, "kwargs": kw}))
+            assert_same_quantization(q, ref, f"{kind} {cfg}")
 
 
 def test_reference_op_schema(oracle):
