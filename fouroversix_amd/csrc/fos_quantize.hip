@@ -150,8 +150,15 @@ template <int DT, int RULE>
 void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, hipStream_t s) {
     if (round_style == FOS_ROUND_NEAREST) {
         // NVFP4 round-to-nearest lives in fos_quantize_fast.hip
-        if constexpr (DT == FOS_DTYPE_NVFP4) launch_quantize_nvfp4_fast(p, RULE, two_d, aligned, false, s);
-        else dispatch_2d<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, aligned, s);
+        if constexpr (DT == FOS_DTYPE_NVFP4) {
+            launch_quantize_nvfp4_fast(p, RULE, two_d, aligned, false, s);
+        } else if constexpr (RULE == FOS_RULE_MSE) {
+            // IF4 with the MSE rule: fast block formulation inside the generic kernel's mapping
+            if (two_d) launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
+            else launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
+        } else {
+            dispatch_2d<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, aligned, s);
+        }
     } else {
         // ... and so does stochastic rounding of aligned inputs (the unbiased style differs
         // in the host-computed constants only; the MSE rule decides through its certified

@@ -45,7 +45,7 @@ FOS_DEVICE FastLutEntry make_lut_entry(uint32_t s, const QuantConsts &k) {
     e.inv = s == 0 ? 0.0f : 1.0f / (k.dec * sf);
     const float g = sf * k.amax;
     e.d1 = g / k.errdiv;
-    e.delta = f2u(g * 0x1p-10f) - f2u(e.d1);  // errdiv is 1536 = 1.5 * 2^10 on this path
+    e.delta = f2u((1.5f * g) / k.errdiv) - f2u(e.d1);  // 1.5 g is exact; with errdiv = 1536 this is g / 1024
     e.pad = 0;
     return e;
 }
@@ -423,6 +423,88 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
     }
     if constexpr (SR) return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);
     else return generic_block<RULE, TWO_D>(blk, k);
+}
+
+// ---------------------------------------------------------------------------------------
+// IF4 (one scale; E2M1 candidate against INT4 candidate), 4/6-style MSE selection
+// ---------------------------------------------------------------------------------------
+//
+// Both candidates share the scale, so in the block's scaled domain (h = s * amax / 2688)
+// their errors are h^2 S_fp and h^2 S_int with S_fp = sum (fq - x/h)^2 and
+// S_int = sum (0.857... q - x/h)^2, and the decision err_int < err_fp compares the two
+// sums.  The rounding bound of the 4/6 shortcut carries over (the INT4 value goes
+// through one more rounding, 12u instead of 6u on a scaled magnitude <= 6, inside the
+// same threefold margin); undecided blocks take the operation-by-operation form.
+template <int RULE, bool TWO_D>
+__device__ __attribute__((noinline)) BlockOut generic_block_if4(Block16 blk, QuantConsts k) {
+    uint32_t codes[2], sbyte;
+    quantize_block<FOS_DTYPE_IF4, RULE, FOS_ROUND_NEAREST, TWO_D>(blk.w, k, 0, 0, 0, codes, sbyte);
+    return BlockOut{codes[0], codes[1], sbyte};
+}
+
+template <bool TWO_D>
+FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
+                                           bool in_range, const FastLutEntry *lut) {
+    if (in_range) {
+        float x[16];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            x[2 * i] = u2f(blk.w[i] << 16);
+            x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
+        }
+        if (canon) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) x[i] = x[i] + 0.0f;
+        }
+        float bmax = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
+        if (TWO_D) bmax = row16_max(bmax);
+        const float s_hp = div_const(bmax, k.qdiv, rq) * enc;
+        const uint32_t s = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp, 0.0f, 0, false) & 0xffu;
+        const FastLutEntry A = lut[s];
+        // same exclusions as the NVFP4 path: the unclamped E2M1 value 8 and the zero scale byte
+        if (s >= 8u || (s != 0u && bmax * A.inv < 7.0f)) {
+            uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+            float SA = 0.0f, SB = 0.0f;
+            static_for<0, 8>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const float x0 = x[2 * j] * A.inv, x1 = x[2 * j + 1] * A.inv;
+                if (j < 4) a0 = pack_fp4<(j & 3)>(a0, x0, x1);
+                else a1 = pack_fp4<(j & 3)>(a1, x0, x1);
+                const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+                const float r0 = fa.x - x0, r1 = fa.y - x1;
+                SA = __builtin_fmaf(r0, r0, SA);
+                SA = __builtin_fmaf(r1, r1, SA);
+                // INT4: rint(clamp(x * 7/6, -7, 7)); adding 1.5 * 2^23 rounds to nearest even and
+                // leaves the two's-complement integer in the low mantissa bits
+                const float t0 = __builtin_amdgcn_fmed3f(x0 * 1.16666666f, -7.0f, 7.0f) + 12582912.0f;
+                const float t1 = __builtin_amdgcn_fmed3f(x1 * 1.16666666f, -7.0f, 7.0f) + 12582912.0f;
+                const float q0 = t0 - 12582912.0f, q1 = t1 - 12582912.0f;
+                const float d0 = __builtin_fmaf(q0, 0.8571428571f, -x0), d1 = __builtin_fmaf(q1, 0.8571428571f, -x1);
+                SB = __builtin_fmaf(d0, d0, SB);
+                SB = __builtin_fmaf(d1, d1, SB);
+                const uint32_t byte = (f2u(t0) & 0xfu) | ((f2u(t1) & 0xfu) << 4);
+                if (j < 4) b0 |= byte << (8 * (j & 3));
+                else b1 |= byte << (8 * (j & 3));
+            });
+            if (TWO_D) {
+                SA = row16_sum_lane0(SA);
+                SB = row16_sum_lane0(SB);
+            }
+            constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
+            constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
+            const float tA = __builtin_fmaf(k1, SA, k0), tB = __builtin_fmaf(k1, SB, k0);
+            const bool surely_int = SB + tB < SA - tA;
+            const bool surely_fp = SB - tB > SA + tA;
+            if (surely_int) return BlockOut{b0, b1, s | 0x80u};
+            if (surely_fp) return BlockOut{a0, a1, s};
+            // undecided (uniform over the 16 lanes of a tile when TWO_D: both sums are tile sums)
+        } else if (bmax == 0.0f) {
+            return BlockOut{0, 0, 0};
+        }
+    }
+    return generic_block_if4<FOS_RULE_MSE, TWO_D>(blk, k);
 }
 
 // The 16 dequantised values of a quantised NVFP4 block as bf16 pairs, with the operations

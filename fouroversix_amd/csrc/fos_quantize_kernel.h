@@ -14,8 +14,8 @@
 
 namespace fos {
 
-// FAST: NVFP4 round-to-nearest through quantize_block_fast, with the operation-by-
-// operation form as the per-block fallback.  ALIGNED: x 16-byte aligned, ld % 8 == 0,
+// FAST: NVFP4 round-to-nearest (or IF4 round-to-nearest with the MSE rule) through the fast
+// block formulations, with the operation-by-operation form as the per-block fallback.  ALIGNED: x 16-byte aligned, ld % 8 == 0,
 // cols % 16 == 0 -> 128-bit loads.
 template <bool FAST, int DT, int RULE, int ROUND, bool TWO_D, int T, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p) {
@@ -95,7 +95,9 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
             Block16 blk;
 #pragma unroll
             for (int i = 0; i < 8; ++i) blk.w[i] = w[it][i];
-            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, false>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut, 0, 0, 0);
+            BlockOut o;
+            if constexpr (DT == FOS_DTYPE_IF4) o = quantize_block_if4_mse<TWO_D>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut);
+            else o = quantize_block_nvfp4_fast<RULE, TWO_D, false>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut, 0, 0, 0);
             codes[0] = o.c0;
             codes[1] = o.c1;
             sbyte = o.s;
@@ -133,7 +135,7 @@ void launch_quantize(QuantParams &p, bool aligned, hipStream_t s) {
     // workgroups to fill the chip; narrow tiles for small or unaligned tensors.
     const int64_t tiles_y = p.rows_p / 128;
     const int64_t groups = p.cols_p / 64;
-    if constexpr (FAST) {
+    if constexpr (FAST && DT == FOS_DTYPE_NVFP4) {
         // aligned NVFP4 round-to-nearest inputs go to the persistent kernel instead
         p.tiles_x = (int)groups;
         hipLaunchKernelGGL((quantize_kernel<FAST, DT, RULE, ROUND, TWO_D, 1, false>),

@@ -87,7 +87,8 @@ def test_full_size_workloads_bit_exact(oracle, shape, kind, cfg):
 @pytest.mark.parametrize("shape", [(100, 80), (16, 64), (1, 16), (130, 8), (257, 1000), (128, 72)])
 def test_ragged_shapes_are_zero_padded(oracle, shape):
     x = make_input("randn", shape, 3)
-    for cfg in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True), dict(dtype="if4", scale_rule="mae")):
+    for cfg in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True), dict(dtype="if4", scale_rule="mae"),
+                dict(dtype="if4", scale_rule="mse"), dict(dtype="if4", scale_rule="mse", block_scale_2d=True)):
         assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), f"{shape} {cfg}")
 
 
@@ -101,6 +102,24 @@ def test_extreme_ranges_take_the_operation_by_operation_path(oracle, scale, two_
         q = hip_quantize(x, scale_rule=rule, block_scale_2d=two_d)
         ref = oracle.quantize(x, scale_rule=rule, block_scale_2d=two_d)
         assert_same_quantization(q, ref, f"scale {scale} {rule}")
+    q = hip_quantize(x, dtype="if4", scale_rule="mse", block_scale_2d=two_d)
+    assert_same_quantization(q, oracle.quantize(x, dtype="if4", scale_rule="mse", block_scale_2d=two_d), f"scale {scale} if4")
+
+
+@pytest.mark.parametrize("two_d", [False, True], ids=["1d", "2d"])
+def test_if4_mse_fast_path_inputs(oracle, two_d):
+    """IF4 with the MSE rule decides most blocks from sums in the scaled domain; inputs that
+    make the two candidates tie or nearly tie (constant blocks, 0/1 data, outlier channels,
+    blocks with tiny scales) must fall through to the exact evaluation and still match."""
+    for kind, shape, seed in (("ones", (128, 256), 0), ("rand01", (256, 256), 1), ("outlier", (256, 1024), 2),
+                              ("tiny_blocks", (256, 512), 3), ("weight", (512, 512), 4), ("randn", (1024, 1024), 5)):
+        x = make_input(kind, shape, seed)
+        q = hip_quantize(x, dtype="if4", scale_rule="mse", block_scale_2d=two_d)
+        assert_same_quantization(q, oracle.quantize(x, dtype="if4", scale_rule="mse", block_scale_2d=two_d), kind)
+    x = make_input("randn", (256, 256), 6)
+    given = float(np.float32(float(x.abs().max()) * 1.2345678))
+    q = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype="if4", block_scale_2d=two_d, kwargs={"amax": torch.tensor(given, device="cuda")}))
+    assert_same_quantization(q, oracle.quantize(x, dtype="if4", block_scale_2d=two_d, amax=given), "24-bit maximum")
 
 
 def test_negative_zero_inputs(oracle):
