@@ -91,14 +91,32 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
             x = fos.quantized_matmul(gate, layer["down"], input_config=acfg)
         return x
 
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / steps
+    def step_shared():
+        # variant: projections that read the same tensor share one quantization of it
+        x = x0
+        for layer in weights:
+            qx = fos.quantize(x, acfg)
+            q = fos.quantized_matmul(qx, layer["q"])
+            fos.quantized_matmul(qx, layer["k"])
+            fos.quantized_matmul(qx, layer["v"])
+            qh = fos.quantize(fos.quantized_matmul(q, layer["o"], input_config=acfg), acfg)
+            gate = fos.quantized_matmul(qh, layer["gate"])
+            fos.quantized_matmul(qh, layer["up"])
+            x = fos.quantized_matmul(gate, layer["down"], input_config=acfg)
+        return x
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    sec = timed(step)
+    sec_shared = timed(step_shared)
     flops = 2.0 * tokens * sum(n * k for _, n, k in shapes) * layers
     return {
         "workload": f"{layers} layers x (q,k,v,o,gate,up,down) quantize+GEMM, {tokens} tokens, hidden {hidden}, "
@@ -106,6 +124,7 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
         "ms_per_step": round(sec * 1e3, 3),
         "tokens_per_s": round(tokens / sec, 1),
         "TFLOP/s": round(flops / sec / 1e12, 1),
+        "shared_activation_quantize": {"ms_per_step": round(sec_shared * 1e3, 3), "tokens_per_s": round(tokens / sec_shared, 1)},
     }
 
 

@@ -202,12 +202,17 @@ FOS_DEVICE float error_term(float deq, float x) {
     return RULE == FOS_RULE_MSE ? d * d : fabsf(d);
 }
 
-// Random words for the 16 elements of 1x16 block `blk`, candidate `cand`: one
-// Philox4x32-10 call keyed (seed; blk, cand, offset).
-FOS_DEVICE Philox4 block_philox(uint64_t seed, uint64_t offset, uint64_t blk, int cand) {
-    return philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset, (uint32_t)seed,
-                         (uint32_t)(seed >> 32));
+// Random words for 1x16 block `blk`: ONE Philox4x32-10 call keyed (seed; blk, 0, offset)
+// serves both candidates of the block.  The first candidate's element i reads word i / 4;
+// the second candidate's element i reads what the first one's element i ^ 8 does (words
+// exchanged pairwise), so within a candidate no two elements share a dither and the two
+// dithers of one element are as independent as those of different elements.  (The
+// reference's own native kernel rounds every element of the tensor and both candidates
+// with one 32-bit word, src/fouroversix/csrc/include/utils.h:521,611,649-650.)
+FOS_DEVICE Philox4 block_philox(uint64_t seed, uint64_t offset, uint64_t blk) {
+    return philox4x32_10((uint32_t)blk, (uint32_t)(blk >> 32), 0u, (uint32_t)offset, (uint32_t)seed, (uint32_t)(seed >> 32));
 }
+FOS_DEVICE Philox4 second_candidate_words(const Philox4 &p) { return Philox4{{p.v[2], p.v[3], p.v[0], p.v[1]}}; }
 
 // One 1x16 block (one row of a 16x16 tile when TWO_D): 8 input words -> 2 code words
 // and the scale byte.  `blk` = row * (cols_p / 16) + block column keys the dither.
@@ -236,7 +241,7 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
         for (int i = 0; i < 16; ++i) xs[i] = (s != 0) ? __builtin_fmaf(x[i], inv, 0.0f) : 0.0f;
     };
     Philox4 pA, pB;
-    if (SR) pA = block_philox(seed, offset, blk, 0);
+    if (SR) pA = block_philox(seed, offset, blk);
 
     if (STATIC) {
         uint32_t c0 = 0, c1 = 0;
@@ -260,7 +265,7 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
         return;
     }
 
-    if (SR) pB = block_philox(seed, offset, blk, 1);
+    if (SR) pB = second_candidate_words(pA);
     float eA[16], eB[16];
     uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
 

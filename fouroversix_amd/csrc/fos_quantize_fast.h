@@ -300,13 +300,13 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
         const FastLutEntry A = lut[s6];
         if (SR ? s6 != 0u : (s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f))) {
             if constexpr (SR) {
-                // scaled values, hardware stochastic rounding (one Philox call per candidate);
+                // scaled values, hardware stochastic rounding (one Philox call per block);
                 // the certified shortcut holds unchanged: its bound does not use how far a
                 // rounded value may lie from the scaled one
                 float xa[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) xa[i] = x[i] * A.inv;
-                const Philox4 pA = block_philox(seed, offset, blkid, 0);
+                const Philox4 pA = block_philox(seed, offset, blkid);
                 uint32_t a0, a1;
                 sr_pack16(xa, pA, a0, a1);
                 if (STATIC) return BlockOut{a0, a1, s6};
@@ -314,7 +314,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 float xb[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) xb[i] = x[i] * B.inv;
-                const Philox4 pB = block_philox(seed, offset, blkid, 1);
+                const Philox4 pB = second_candidate_words(pA);
                 uint32_t b0, b1;
                 sr_pack16(xb, pB, b0, b1);
                 bool pickB = false, certain = false;

@@ -236,9 +236,13 @@ void fos_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint
 }
 
 /* Random words for the 16 elements of 1x16 block `blk` (= row * blocks_per_row + block
- * column of the padded tensor), candidate `cand`: ONE Philox4x32-10 call with counter
- * (blk_lo, blk_hi, cand, offset_lo) and key (seed_lo, seed_hi).  Element i belongs to byte
- * i % 4 of word i / 4.  E2M1 rounding takes the word rotated so that this byte leads and
+ * column of the padded tensor): ONE Philox4x32-10 call with counter (blk_lo, blk_hi, 0,
+ * offset_lo) and key (seed_lo, seed_hi) serves both candidates of the block; the second
+ * candidate's element i takes what the first one's element i ^ 8 takes (`cand`), so no two
+ * elements of a candidate share a dither.  (The reference's own native kernel rounds a
+ * whole tensor and both candidates with one 32-bit word,
+ * src/fouroversix/csrc/include/utils.h:521,611,649-650.)  Element i of the first candidate
+ * belongs to byte i % 4 of word i / 4.  E2M1 rounding takes the word rotated so that this byte leads and
  * from it the 22 bits that the convert's slot reads -- 31..10 for even i, 30..9 for odd i
  * (rw[i]; the leading 7 or 8 bits are the element's own, the rest come from its three
  * neighbours at 1/256 of the weight); the INT4 candidate of IF4 takes
@@ -246,11 +250,11 @@ void fos_oracle_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint
  * reference draws from torch's generator, so its stream cannot be matched bit for bit. */
 static void dither16(uint64_t seed, uint64_t offset, uint64_t blk, int cand, float u[16], uint32_t rw[16]) {
     uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
-    uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)cand, (uint32_t)offset};
+    uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), 0u, (uint32_t)offset};
     uint32_t w[4];
     fos_oracle_philox4x32_10(ctr, key, w);
     for (int i = 0; i < 16; ++i) {
-        uint32_t word = w[i >> 2];
+        uint32_t word = w[((i >> 2) + (cand ? 2 : 0)) & 3];
         int sh = (8 * ((i & 3) + 1)) & 31;
         u[i] = (float)((word >> (8 * (i & 3))) & 0xffu) * 0.00390625f - 0.498046875f;
         uint32_t rot = sh ? ((word >> sh) | (word << (32 - sh))) : word;
