@@ -191,6 +191,9 @@ extern "C" int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, i
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
+// Inputs up to this many elements (128 KiB) are quantized in one launch.
+constexpr int64_t kFusedAmaxElements = 65536;
+
 // Shared body of fos_quantize and fos_pseudo_quantize (pseudo_out != null: bf16 round trip
 // instead of codes / scales).
 static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
@@ -248,6 +251,11 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         p.partials = (const uint32_t *)amax;
         p.n_partials = 0;
         p.amax_out = nullptr;
+    } else if (aligned && ld == cols && rows * cols <= kFusedAmaxElements) {
+        // decode-sized input: one launch, every workgroup of pass 2 finds the maximum itself
+        p.partials = partials;
+        p.n_partials = -1;
+        p.amax_out = amax;
     } else {
         p.partials = partials;
         p.n_partials = launch_amax(x, rows, cols, ld, aligned, partials, s);

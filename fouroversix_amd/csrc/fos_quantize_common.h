@@ -23,7 +23,8 @@ struct QuantParams {
     uint8_t *codes;              // [rows_p, cols_p / 2]
     uint8_t *sf;                 // rows_p * cols_p / 16 bytes
     const uint32_t *partials;    // pass-1 results, pairs {max|x| as f32 bits, 1 if a -0.0 was seen}
-    int n_partials;              // number of pairs; 0 = `partials` points at a caller-supplied f32 amax
+    int n_partials;              // number of pairs; 0 = `partials` points at a caller-supplied f32 amax;
+                                 // -1 = no pass 1 ran: pass 2 scans the (small, contiguous, aligned) input itself
     float *amax_out;             // written by workgroup 0 when not null
     uint64_t seed, offset;
     int sf_layout;
@@ -77,6 +78,35 @@ FOS_DEVICE void reduce_partials(const QuantParams &p, uint32_t *smem, uint32_t &
     if (p.n_partials == 0) {
         amax_bits = p.partials[0];
         maybe_negzero = true;
+        return;
+    }
+    if (p.n_partials < 0) {
+        // small contiguous input: no pass 1 was launched and every workgroup scans the
+        // whole tensor itself (rows * cols / 8 aligned 128-bit vectors, 128 KiB out of L2 at
+        // most), which costs less than a launch and its dependency
+        const uint4 *v4 = reinterpret_cast<const uint4 *>(p.x);
+        const int n_vec = (int)((p.rows * p.cols) >> 3);
+        uint32_t m = 0, z = 0;
+        constexpr int U = 16;  // loads in flight per thread: the scan is latency-bound
+        for (int base = 0; base < n_vec; base += U * kThreads) {
+            uint4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = base + u * kThreads + (int)threadIdx.x;
+                v[u] = i < n_vec ? v4[i] : make_uint4(0u, 0u, 0u, 0u);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                m = pk_max_u16(m, v[u].x & 0x7fff7fffu);
+                m = pk_max_u16(m, v[u].y & 0x7fff7fffu);
+                m = pk_max_u16(m, v[u].z & 0x7fff7fffu);
+                m = pk_max_u16(m, v[u].w & 0x7fff7fffu);
+                z = pk_min_i16(pk_min_i16(z, v[u].x), pk_min_i16(v[u].y, pk_min_i16(v[u].z, v[u].w)));
+            }
+        }
+        const uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+        amax_bits = block_max_u32(mm, smem) << 16;  // bf16 magnitude bits -> fp32 bits
+        maybe_negzero = block_max_u32(((z & 0xffffu) == 0x8000u || (z >> 16) == 0x8000u) ? 1u : 0u, smem) != 0;
         return;
     }
     uint32_t m = 0, z = 0;

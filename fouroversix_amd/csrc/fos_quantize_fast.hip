@@ -181,9 +181,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             if (g + 2 < 8) load(g + 2, blk[g + 2]);
             if (col_ok) {
                 const int rr = g * 16 + rr0;
-                const BlockOut o = quantize_block_nvfp4_fast<RULE, false, SR>(
-                    blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut, p.seed, p.offset,
-                    (uint64_t)((row0 + g * 16) * sf_cols + cb));
+                // a 16-row step that lies wholly in the row padding (decode-sized inputs: seven of
+                // the eight steps) only writes its zero codes and scales
+                const bool padding_step = !FULL && (int64_t)tile_y * 128 + g * 16 >= p.rows;
+                BlockOut o{0u, 0u, 0u};
+                if (!padding_step)
+                    o = quantize_block_nvfp4_fast<RULE, false, SR>(blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut, p.seed,
+                                                                   p.offset, (uint64_t)((row0 + g * 16) * sf_cols + cb));
                 if (PSEUDO) {
                     uint32_t w[8];
                     if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
