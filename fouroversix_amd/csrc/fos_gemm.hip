@@ -35,7 +35,9 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 struct GemmParams {
     const uint8_t *A, *B;      // [M, K/2], [N, K/2]
     const uint8_t *sfA, *sfB;  // 128x4-tiled E4M3 bytes
-    const float *alpha;
+    const float *alpha;        // output scale on the device, or null: (amax_a * amax_b) * inv_den
+    const float *amax_a, *amax_b;
+    float inv_den;
     void *D;
     int64_t M, N, K, ldd;
     int tiles_m, tiles_n;
@@ -44,6 +46,12 @@ struct GemmParams {
     float *partials;
     int splits, ksteps_per_split;
 };
+
+// Output scale: read from the device, or formed from the two tensor maxima with the
+// arithmetic of gemm_alpha_kernel (product, then times the fp32 reciprocal of the divisor).
+FOS_DEVICE float load_alpha(const GemmParams &p) {
+    return p.alpha ? *p.alpha : (*p.amax_a * *p.amax_b) * p.inv_den;
+}
 
 // The two E4M3 bytes in the low 16 bits of `w` -> fp16 pair {s0, s1} (one hardware
 // convert; exact, sub-normals included -- checked against the OCP decode of all 256 bytes).
@@ -256,7 +264,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
         }
         return;
     }
-    const float alpha = *p.alpha;
+    const float alpha = load_alpha(p);
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
@@ -476,7 +484,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
         }
         return;
     }
-    const float alpha = *p.alpha;
+    const float alpha = load_alpha(p);
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
@@ -517,7 +525,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
         const float4 v = P[y * stride];
         s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
     }
-    const float alpha = *p.alpha;
+    const float alpha = load_alpha(p);
     const float v[4] = {alpha * s.x, alpha * s.y, alpha * s.z, alpha * s.w};
     uint16_t o[4];
 #pragma unroll
@@ -657,11 +665,13 @@ extern "C" size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     return g.splits > 1 ? (size_t)g.splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
-extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
-                              const float *alpha, int64_t M, int64_t N, int64_t K,
-                              void *D, int out_type, int64_t ldd,
-                              void *workspace, size_t workspace_bytes, fos_stream_t stream) {
-    if (!A || !B || !sfA || !sfB || !alpha || !D) return FOS_E_NULL_POINTER;
+static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                           const float *alpha, const float *amax_a, const float *amax_b, double denominator,
+                           int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd,
+                           void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!A || !B || !sfA || !sfB || !D) return FOS_E_NULL_POINTER;
+    if (!alpha && (!amax_a || !amax_b)) return FOS_E_NULL_POINTER;
+    if (!alpha && (((uintptr_t)amax_a & 3) || ((uintptr_t)amax_b & 3))) return FOS_E_BAD_ALIGNMENT;
     if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || N % 128 != 0 || K % 64 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
     if (M < 128 && K % 256 != 0) return FOS_E_BAD_SHAPE;  // partial bands only through the weight-streaming kernel
     if (out_type != FOS_T_BF16 && out_type != FOS_T_F16) return FOS_E_UNSUPPORTED;
@@ -671,6 +681,7 @@ extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 24)) return FOS_E_BAD_SHAPE;
     GemmParams p;
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
+    p.amax_a = amax_a; p.amax_b = amax_b; p.inv_den = alpha ? 0.0f : (float)(1.0 / denominator);
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
     GemmPlan g = plan_gemm(M, N, K);
@@ -692,4 +703,23 @@ extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
             return launch_skinny<4, 1>(p, out_type, s);
         default: return launch_gemm<2, 2, 2, 2>(p, out_type, s);
     }
+}
+
+extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                              const float *alpha, int64_t M, int64_t N, int64_t K,
+                              void *D, int out_type, int64_t ldd,
+                              void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!alpha) return FOS_E_NULL_POINTER;
+    return gemm_nvfp4_impl(A, B, sfA, sfB, alpha, nullptr, nullptr, 1.0, M, N, K, D, out_type, ldd, workspace,
+                           workspace_bytes, stream);
+}
+
+extern "C" int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                                   const float *amax_a, const float *amax_b, double denominator,
+                                   int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd,
+                                   void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!amax_a || !amax_b) return FOS_E_NULL_POINTER;
+    if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, workspace,
+                           workspace_bytes, stream);
 }

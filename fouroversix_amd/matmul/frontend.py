@@ -91,18 +91,34 @@ def quantized_matmul(
         )
         return out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
 
-    alpha = gemm_alpha(input, other)
-    gemm = (
-        ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
-        if out_dtype == DataType.bfloat16
-        else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
-    )
     a_values = input.values
     m_orig = input.original_shape[0]
     if m_orig < 128 and a_values.shape[0] == 128 and a_values.shape[1] % 128 == 0:
         # small batch: hand over only the real rows, so the kernel skips the padding
         a_values = a_values[:m_orig]
-    out = gemm(a_values, other.values, input.scale_factors, other.scale_factors, alpha)
+    a_amax, b_amax = input.amax, other.amax
+    if (
+        type(a_values) is torch.Tensor
+        and not torch.compiler.is_compiling()
+        and a_amax.dtype == torch.float32
+        and b_amax.dtype == torch.float32
+        and a_amax.is_cuda
+        and b_amax.device == a_amax.device == a_values.device
+    ):
+        # the kernel forms alpha from the two maxima itself (same arithmetic, one launch less)
+        den = dequantize_divisor(input) * dequantize_divisor(other)
+        out = ops.gemm_nvfp4_from_amax(
+            a_values, other.values, input.scale_factors, other.scale_factors, a_amax, b_amax, den,
+            torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16,
+        )
+    else:
+        alpha = gemm_alpha(input, other)
+        gemm = (
+            ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
+            if out_dtype == DataType.bfloat16
+            else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
+        )
+        out = gemm(a_values, other.values, input.scale_factors, other.scale_factors, alpha)
     out_shape = (input.original_shape[0], other.original_shape[0])
     if tuple(out.shape) != out_shape:
         out = out[: out_shape[0], : out_shape[1]]

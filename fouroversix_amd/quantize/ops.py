@@ -205,8 +205,11 @@ def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selec
     return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, amax)
 
 
-def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
-    for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), ("alpha", alpha)):
+def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None):
+    """``amax`` = (amax_a, amax_b, denominator) forms the output scale inside the kernel
+    (``alpha`` is then ignored and may be None)."""
+    scale_tensors = (("alpha", alpha),) if amax is None else (("amax_a", amax[0]), ("amax_b", amax[1]))
+    for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), *scale_tensors):
         nat.require_gpu_tensor(t, name)
         if not t.is_contiguous():
             raise RuntimeError(f"gemm: {name} must be contiguous")
@@ -239,11 +242,13 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype):
         # split-K partial tiles of small-M shapes; from torch's caching allocator, which
         # keeps the block tied to the current stream
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-        rc = L.fos_gemm_nvfp4(
-            a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(),
-            m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n,
-            ws.data_ptr() if ws is not None else None, ws_bytes, nat.current_stream(a.device),
-        )
+        tail = (m, n, ka, out.data_ptr(), nat.TORCH_TO_T[out_dtype], n,
+                ws.data_ptr() if ws is not None else None, ws_bytes, nat.current_stream(a.device))
+        if amax is None:
+            rc = L.fos_gemm_nvfp4(a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(), *tail)
+        else:
+            rc = L.fos_gemm_nvfp4_amax(a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(),
+                                       amax[0].data_ptr(), amax[1].data_ptr(), float(amax[2]), *tail)
     nat.check(rc, "fouroversix::gemm_nvfp4nvfp4_accum_fp32")
     return out
 
@@ -409,6 +414,12 @@ def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
     if _direct(a):
         return _gemm_impl(a, b, a_sf, b_sf, alpha, torch.float16)
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
+
+
+def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype):
+    """The NVFP4 GEMM with the output scale ``(amax_a * amax_b) * f32(1 / denominator)`` formed
+    in the kernel (``fos_gemm_nvfp4_amax``): one launch less than alpha + GEMM, same result."""
+    return _gemm_impl(a, b, a_sf, b_sf, None, out_dtype, amax=(amax_a, amax_b, denominator))
 
 
 def gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):

@@ -157,6 +157,17 @@ int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const
                    void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * fos_gemm_nvfp4 with the output scale formed inside the kernel from the operands' tensor
+ * maxima: alpha = (amax_a[0] * amax_b[0]) * f32(1 / denominator), the value fos_gemm_alpha
+ * writes (src/fouroversix/matmul/cutlass/backend.py:86-98), without that launch.
+ * amax_a / amax_b are device f32[1], e.g. the `amax` outputs of fos_quantize.
+ */
+int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                        const float *amax_a, const float *amax_b, double denominator,
+                        int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd,
+                        void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * alpha[0] = (amax_a[0] * amax_b[0]) * f32(1 / denominator), in fp32 on the device: the
  * GEMM's output scale as src/fouroversix/matmul/cutlass/backend.py:86-98 forms it on a GPU
  * (torch divides a tensor by a host scalar through the reciprocal, taken in double and

