@@ -63,14 +63,10 @@ def quantized_matmul(
 ) -> torch.Tensor:
     """FP4 matrix product ``input @ other.T`` -> ``[M, N]`` tensor of ``out_dtype``."""
     del kwargs
-    if input_config is None:
-        input_config = QuantizationConfig()
     if isinstance(input, torch.Tensor):
-        input = quantize(input, input_config)
-    if other_config is None:
-        other_config = QuantizationConfig()
+        input = quantize(input, QuantizationConfig() if input_config is None else input_config)
     if isinstance(other, torch.Tensor):
-        other = quantize(other, other_config)
+        other = quantize(other, QuantizationConfig() if other_config is None else other_config)
     if isinstance(out_dtype, str):
         out_dtype = DataType(out_dtype)
 

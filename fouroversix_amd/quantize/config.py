@@ -3,7 +3,7 @@
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field, fields
+from dataclasses import dataclass, field
 from typing import Any
 
 from fouroversix_amd.utils import DataType, QuantizeBackend, RoundStyle, ScaleRule
@@ -42,8 +42,7 @@ class QuantizationConfig:
     transpose: bool = False
 
     def __post_init__(self) -> None:
-        for f in fields(self):
-            enum_cls = _ENUM_FIELDS.get(f.name)
-            value = getattr(self, f.name)
-            if enum_cls is not None and isinstance(value, str) and not isinstance(value, enum_cls):
-                setattr(self, f.name, enum_cls(value))
+        for name, enum_cls in _ENUM_FIELDS.items():
+            value = getattr(self, name)
+            if isinstance(value, str) and not isinstance(value, enum_cls):
+                setattr(self, name, enum_cls(value))
