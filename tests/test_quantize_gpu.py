@@ -169,6 +169,25 @@ def test_caller_supplied_amax(oracle):
             assert_same_quantization(q, ref, f"{kind} {cfg}")
 
 
+def test_concurrent_streams_do_not_share_the_workspace(oracle):
+    """Two streams quantize different tensors at the same time (the two-launch path, which
+    hands partial maxima from pass 1 to pass 2 through a per-stream workspace)."""
+    xs = [make_input("randn", (1024, 2048), 50 + i) * (1.0 + 3.0 * i) for i in range(2)]
+    refs = [oracle.quantize(x, scale_rule="mse") for x in xs]
+    dev = [x.cuda() for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    outs = [[], []]
+    for _ in range(8):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                outs[i].append(fos.quantize(dev[i]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for q in outs[i]:
+            assert_same_quantization(q, refs[i], f"stream {i}")
+
+
 def test_reference_op_schema(oracle):
     """torch.ops.fouroversix.quantize with the reference's positional schema."""
     x = make_input("randn", (256, 128), 7)
