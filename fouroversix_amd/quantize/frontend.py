@@ -45,6 +45,31 @@ def can_quantize(x: torch.Tensor, config: QuantizationConfig) -> bool:
     return unsupported_reason(x, config) is None
 
 
+def _quantize_meta(x: torch.Tensor, config: QuantizationConfig) -> QuantizedTensor | torch.Tensor:
+    """Shapes only, for tensors on the meta device (model construction before weights are
+    loaded): zero-filled meta tensors of the padded sizes, as the reference's PyTorch backend
+    returns (``src/fouroversix/quantize/pytorch/backend.py:57-97``)."""
+    if config.pseudo_quantize:
+        return torch.empty_like(x)
+    shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
+    block = config.dtype.block_size
+    rows_p, cols_p = -(-shape[0] // 128) * 128, -(-shape[1] // (4 * block)) * (4 * block)
+    sf_dtype = config.dtype.scale_type.torch_dtype
+    if sf_dtype == torch.float8_e8m0fnu:
+        sf_dtype = torch.uint8
+    linear = config.dtype in _LINEAR_SCALE_FORMATS
+    return QuantizedTensor(
+        torch.zeros(rows_p, cols_p // config.dtype.quantized_value_type.packing_factor, dtype=torch.uint8, device=x.device),
+        torch.zeros(rows_p * cols_p // block, dtype=sf_dtype, device=x.device),
+        torch.zeros(1, dtype=torch.float32, device=x.device),
+        config.dtype,
+        tuple(shape),
+        config.scale_rule,
+        config.round_style,
+        scale_factors_are_in_blackwell_layout=not linear,
+    )
+
+
 def quantize(
     x: torch.Tensor,
     config: QuantizationConfig | None = None,
@@ -58,6 +83,9 @@ def quantize(
     """
     if config is None:
         config = QuantizationConfig()
+
+    if x.device.type == "meta" and x.dim() == 2:
+        return _quantize_meta(x, config)
 
     reason = unsupported_reason(x, config)
     if reason is not None:

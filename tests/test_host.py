@@ -131,3 +131,21 @@ def test_registry_rules():
         QuantizedModule.register(MyLinear)
     assert QuantizedModule.is_quantized_module_type(fos.FourOverSixLinear)
     assert QuantizedModule.get_cls(nn.Linear) is fos.FourOverSixLinear
+
+
+def test_quantize_of_meta_tensors_returns_padded_shapes():
+    """Meta-device inputs (model construction before the weights exist) yield zero-filled meta
+    tensors of the padded sizes, as the reference's PyTorch backend does
+    (src/fouroversix/quantize/pytorch/backend.py:57-97): no kernel, no GPU."""
+    x = torch.empty(100, 80, dtype=torch.bfloat16, device="meta")
+    q = fos.quantize(x)
+    assert q.values.device.type == "meta" and tuple(q.values.shape) == (128, 64) and q.values.dtype == torch.uint8
+    assert q.scale_factors.numel() == 128 * 128 // 16 and q.scale_factors.dtype == torch.float8_e4m3fn
+    assert tuple(q.amax.shape) in ((1,), ()) and q.original_shape == (100, 80) and tuple(q.padded_shape) == (128, 128)
+    assert q.scale_factors_are_in_blackwell_layout
+    q = fos.quantize(x, fos.QuantizationConfig(dtype="mxfp4", scale_rule="static_6", transpose=True))
+    assert q.original_shape == (80, 100) and q.scale_factors.numel() == 128 * 128 // 32
+    q = fos.quantize(x, fos.QuantizationConfig(dtype="if4"))
+    assert not q.scale_factors_are_in_blackwell_layout
+    y = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True))
+    assert y.device.type == "meta" and y.shape == x.shape and y.dtype == x.dtype
