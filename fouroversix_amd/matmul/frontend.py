@@ -16,8 +16,8 @@ import torch
 
 from fouroversix_amd.quantize import QuantizationConfig, QuantizedTensor, quantize
 from fouroversix_amd.quantize import ops
-from fouroversix_amd.quantize.frontend import dequantize_divisor
-from fouroversix_amd.utils import DataType, MatmulBackend
+from fouroversix_amd.quantize.frontend import dequantize, dequantize_divisor
+from fouroversix_amd.utils import NATIVE_FORMAT_IDS, DataType, MatmulBackend
 
 
 def is_supported(input: QuantizedTensor, other: QuantizedTensor, *, out_dtype: DataType) -> bool:
@@ -36,6 +36,17 @@ def is_supported(input: QuantizedTensor, other: QuantizedTensor, *, out_dtype: D
         and out_dtype in (DataType.bfloat16, DataType.float16)
         and input.scale_factors_are_in_blackwell_layout
         and other.scale_factors_are_in_blackwell_layout
+    )
+
+
+def _dequantize_form_applies(input: QuantizedTensor, other: QuantizedTensor, out_dtype: DataType) -> bool:
+    """Both operands are formats the dequantize kernel reads, on one GPU."""
+    return (
+        input.dtype.value in NATIVE_FORMAT_IDS
+        and other.dtype.value in NATIVE_FORMAT_IDS
+        and input.values.is_cuda
+        and other.values.device == input.values.device
+        and out_dtype in (DataType.bfloat16, DataType.float16, DataType.float32)
     )
 
 
@@ -71,6 +82,15 @@ def quantized_matmul(
         out_dtype = DataType(out_dtype)
 
     if not is_supported(input, other, out_dtype=out_dtype):
+        if _dequantize_form_applies(input, other, out_dtype):
+            # formats without a native GEMM (IF4; mixed formats): the reference's PyTorch backend,
+            # ``matmul(dequantize(a, f32), dequantize(b, f32).T)`` rounded to the output type
+            # (src/fouroversix/matmul/pytorch.py:33-52) -- the dequantize kernel plus a library GEMM
+            out = torch.matmul(
+                dequantize(input, dtype=torch.float32), dequantize(other, dtype=torch.float32).T
+            ).to(out_dtype.torch_dtype)
+            out_shape = (input.original_shape[0], other.original_shape[0])
+            return out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
         if backend is None:
             msg = "No backend found that supports the given parameters"
         else:

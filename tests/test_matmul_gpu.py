@@ -178,6 +178,26 @@ def test_linear_layer_forward(oracle):
     assert torch.equal(keep(x.cuda()), y)
 
 
+def test_formats_without_a_native_gemm_take_the_dequantize_form(oracle):
+    """IF4 operands (and an fp32 result) go through dequantize + matmul, the reference's
+    PyTorch matmul backend (src/fouroversix/matmul/pytorch.py:33-52); compared with the
+    oracle's statement of that backend under the reference's mismatch budget."""
+    a, b = make_input("randn", (200, 512), 61), make_input("weight", (300, 512), 62)
+    cfg = dict(dtype="if4", scale_rule="mse")
+    out = fos.quantized_matmul(a.cuda(), b.cuda(), input_config=fos.QuantizationConfig(**cfg),
+                               other_config=fos.QuantizationConfig(block_scale_2d=True, **cfg))
+    assert out.shape == (200, 300) and out.dtype == torch.bfloat16
+    ra, rb = oracle.quantize(a, **cfg), oracle.quantize(b, block_scale_2d=True, **cfg)
+    o16, o32 = oracle.quantized_matmul(ra, rb)
+    expect = torch.from_numpy(o16.view(np.int16).copy()).view(torch.bfloat16)
+    assert float((out.cpu() != expect).float().mean()) <= 2 * MISMATCH_BUDGET
+    qa, qb = fos.quantize(a.cuda()), fos.quantize(b.cuda())
+    out32 = fos.quantized_matmul(qa, qb, out_dtype="float32")
+    ref32 = oracle.quantized_matmul(oracle.quantize(a), oracle.quantize(b))[1]
+    assert out32.dtype == torch.float32
+    assert float((out32.cpu() - torch.from_numpy(ref32)).abs().max()) <= 1e-3 * float(np.abs(ref32).max())
+
+
 def test_linear_forward_replays_in_a_hip_graph():
     """A decode-sized forward (quantize -> alpha -> weight-streaming GEMM, twice) captured in
     a HIP graph: every replay, interleaved with eager work and synchronisations, equals
