@@ -90,7 +90,7 @@ def lib() -> ctypes.CDLL:
     L.fos_padded_cols_for.restype = i64
     L.fos_gemm_workspace_bytes.argtypes = [i64, i64, i64]
     L.fos_gemm_workspace_bytes.restype = ctypes.c_size_t
-    L.fos_dequantize.argtypes = [vp, vp, vp, i32, i32, dbl, i64, i64, i64, i64, vp, i32, i64, vp]
+    L.fos_dequantize.argtypes = [vp, vp, vp, i32, i32, dbl, i64, i64, i64, i64, vp, i32, i64, i32, vp]
     L.fos_dequantize.restype = i32
     _lib = L
     return L

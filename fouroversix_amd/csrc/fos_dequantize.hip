@@ -19,6 +19,7 @@ struct DequantParams {
     int sf_layout;
     int fast_div;       // divisor is 1536, 1792 or 2688 (exact 3-operation division)
     int vector_stores;  // out and ldo allow 16-byte stores of whole blocks
+    int f32_product;    // value * scale formed in fp32 instead of fp16 (differs for IF4's integer blocks)
 };
 
 // One thread per 8 consecutive elements, i.e. half a 1x16 block (consecutive threads =
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
         for (int i = 0; i < 8; ++i) {
             const uint32_t code = (q >> (4 * i)) & 0xfu;
             const int iv = ((int)(code << 28)) >> 28;
-            f[i] = (float)((_Float16)((float)iv * six_sevenths) * s16);
+            f[i] = p.f32_product ? ((float)iv * six_sevenths) * sf : (float)((_Float16)((float)iv * six_sevenths) * s16);
         }
     } else {
         static_for<0, 4>([&](auto jc) {
@@ -113,7 +114,8 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
 namespace fos {
 // MXFP4 (fos_mxfp4.hip)
 int launch_dequantize_mxfp4(const uint8_t *codes, const uint8_t *sf, int sf_layout, int64_t rows, int64_t cols,
-                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, hipStream_t s);
+                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, int f32_product,
+                            hipStream_t s);
 }  // namespace fos
 
 using namespace fos;
@@ -130,14 +132,17 @@ void launch_dequant(const DequantParams &p, int out_type, dim3 grid, hipStream_t
 extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const float *amax,
                               int dtype, int sf_layout, double divisor,
                               int64_t rows, int64_t cols, int64_t rows_p, int64_t cols_p,
-                              void *out, int out_type, int64_t ldo, fos_stream_t stream) {
+                              void *out, int out_type, int64_t ldo, int intermediate_type, fos_stream_t stream) {
     if (!codes || !sf || !out || (!amax && dtype != FOS_DTYPE_MXFP4)) return FOS_E_NULL_POINTER;
+    if (intermediate_type != FOS_T_F16 && intermediate_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
+    const int f32_product = intermediate_type == FOS_T_F32;
     if (dtype == FOS_DTYPE_MXFP4) {
         if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || ldo < cols) return FOS_E_BAD_SHAPE;
         if (sf_layout == FOS_SF_TILED_128X4 && rows_p % 128 != 0) return FOS_E_BAD_SHAPE;
         if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
         if (out_type != FOS_T_BF16 && out_type != FOS_T_F16 && out_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
-        return launch_dequantize_mxfp4(codes, sf, sf_layout, rows, cols, rows_p, cols_p, out, out_type, ldo, (hipStream_t)stream);
+        return launch_dequantize_mxfp4(codes, sf, sf_layout, rows, cols, rows_p, cols_p, out, out_type, ldo, f32_product,
+                                       (hipStream_t)stream);
     }
     if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || cols_p % 16 != 0 || ldo < cols) return FOS_E_BAD_SHAPE;
     if (sf_layout == FOS_SF_TILED_128X4 && (rows_p % 128 != 0 || cols_p % 64 != 0)) return FOS_E_BAD_SHAPE;
@@ -150,6 +155,7 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
     p.divisor = (float)divisor;
     p.sf_layout = sf_layout;
+    p.f32_product = f32_product;
     p.fast_div = p.divisor == 1536.0f || p.divisor == 1792.0f || p.divisor == 2688.0f;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;

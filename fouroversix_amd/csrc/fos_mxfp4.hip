@@ -180,6 +180,7 @@ struct MxDequantParams {
     int64_t rows, cols, rows_p, cols_p, ldo;
     int sf_layout;
     int vector_stores;
+    int f32_product;  // value * scale in fp32 (exact) instead of fp16
 };
 
 typedef _Float16 mx_half2_t __attribute__((ext_vector_type(2)));
@@ -200,14 +201,21 @@ __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantPa
                              ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
                              : r * sf_cols + cb;
     const uint32_t e = p.sf[sofs];
-    const _Float16 s16 = (_Float16)(e == 0u ? u2f(0x00400000u) : u2f(e << 23));
+    const float s32 = e == 0u ? u2f(0x00400000u) : u2f(e << 23);  // 2^(e - 127); e = 255 is a NaN, as in E8M0
+    const _Float16 s16 = (_Float16)s32;
     const mx_half2_t s2 = {s16, s16};
     float f[8];
     static_for<0, 4>([&](auto jc) {
         constexpr int j = decltype(jc)::value;
-        const mx_half2_t v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 1.0f, j) * s2;
-        f[2 * j] = (float)v.x;
-        f[2 * j + 1] = (float)v.y;
+        if (p.f32_product) {
+            const float2_t v = unpack_fp4<j>(q);
+            f[2 * j] = v.x * s32;
+            f[2 * j + 1] = v.y * s32;
+        } else {
+            const mx_half2_t v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(q, 1.0f, j) * s2;
+            f[2 * j] = (float)v.x;
+            f[2 * j + 1] = (float)v.y;
+        }
     });
     const int64_t c0 = oc * 8;
     const bool whole = p.vector_stores && c0 + 8 <= p.cols;
@@ -245,13 +253,15 @@ __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantPa
 }
 
 int launch_dequantize_mxfp4(const uint8_t *codes, const uint8_t *sf, int sf_layout, int64_t rows, int64_t cols,
-                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, hipStream_t s) {
+                            int64_t rows_p, int64_t cols_p, void *out, int out_type, int64_t ldo, int f32_product,
+                            hipStream_t s) {
     if (cols_p % 32 != 0 || (sf_layout == FOS_SF_TILED_128X4 && cols_p % 128 != 0)) return FOS_E_BAD_SHAPE;
     if ((uintptr_t)codes & 3) return FOS_E_BAD_ALIGNMENT;
     MxDequantParams p;
     p.codes = codes; p.sf = sf; p.out = out;
     p.rows = rows; p.cols = cols; p.rows_p = rows_p; p.cols_p = cols_p; p.ldo = ldo;
     p.sf_layout = sf_layout;
+    p.f32_product = f32_product;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
     const int64_t n_octets = rows * ((cols + 7) / 8);

@@ -169,8 +169,9 @@ def dequantize(
 ) -> torch.Tensor:
     """High-precision tensor of ``tensor.original_shape`` from a quantized tensor.
 
-    Value and block scale are multiplied in fp16 (exact for NVFP4, so
-    ``intermediate_dtype=float32`` gives the same result there), widened to fp32,
+    Value and block scale are multiplied in ``intermediate_dtype`` (fp16 or fp32; exact
+    either way for NVFP4, different for IF4's integer blocks and for MXFP4 scales outside
+    fp16's range), widened to fp32,
     scaled by ``amax / (qmax * smax * adjustment)`` and cast to ``dtype``.
     """
     del backend
@@ -180,8 +181,8 @@ def dequantize(
     if tensor.amax is None and tensor.dtype.scale_type != ScaleType.mx:
         msg = "dequantize needs the tensor-wide amax"
         raise ValueError(msg)
-    if intermediate_dtype != torch.float16 and tensor.dtype != DataType.nvfp4:
-        msg = "only intermediate_dtype=float16 is implemented for this format"
+    if intermediate_dtype not in (torch.float16, torch.float32):
+        msg = "intermediate_dtype must be float16 or float32"
         raise ValueError(msg)
     if dtype not in nat.TORCH_TO_T:
         msg = f"unsupported output dtype {dtype}"
@@ -198,4 +199,5 @@ def dequantize(
         rows,
         cols,
         dtype,
+        intermediate_dtype == torch.float32,
     )

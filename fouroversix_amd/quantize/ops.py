@@ -33,7 +33,7 @@ _LIB.define("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor 
 _LIB.define("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor")
 _LIB.define(
     "dequantize(Tensor values, Tensor scale_factors, Tensor amax, int dtype, int sf_layout, float divisor, "
-    "int rows, int cols, ScalarType out_dtype) -> Tensor"
+    "int rows, int cols, ScalarType out_dtype, bool f32_intermediate=False) -> Tensor"
 )
 
 
@@ -291,7 +291,7 @@ def _gemm_mxfp4_impl(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):
     return out
 
 
-def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype, f32_intermediate=False):
     nat.require_gpu_tensor(values, "values")
     rows_p, cols_p = values.shape[0], values.shape[1] * 2
     out = torch.empty(rows, cols, dtype=out_dtype, device=values.device)
@@ -302,7 +302,8 @@ def _dequantize_impl(values, scale_factors, amax, dtype, sf_layout, divisor, row
         rc = nat.lib().fos_dequantize(
             values.contiguous().data_ptr(), scale_factors.contiguous().data_ptr(), amax32.data_ptr(),
             dtype, sf_layout, divisor, rows, cols, rows_p, cols_p,
-            out.data_ptr(), nat.TORCH_TO_T[out_dtype], cols, nat.current_stream(values.device),
+            out.data_ptr(), nat.TORCH_TO_T[out_dtype], cols, nat.T_F32 if f32_intermediate else nat.T_F16,
+            nat.current_stream(values.device),
         )
     nat.check(rc, "fouroversix::dequantize")
     return out
@@ -366,7 +367,7 @@ def _(a, b, a_sf, b_sf, alpha):
 
 
 @torch.library.register_fake("fouroversix::dequantize")
-def _(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+def _(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype, f32_intermediate=False):
     return torch.empty(rows, cols, dtype=out_dtype, device=values.device)
 
 
@@ -429,7 +430,7 @@ def gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha, out_dtype=t
     return torch.ops.fouroversix.gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
-def dequantize(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype):
+def dequantize(values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype, f32_intermediate=False):
     return torch.ops.fouroversix.dequantize.default(
-        values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype
+        values, scale_factors, amax, dtype, sf_layout, divisor, rows, cols, out_dtype, f32_intermediate
     )

@@ -200,12 +200,15 @@ int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const
  *   codes u8 [rows_p, cols_p/2], sf in sf_layout over [rows_p, cols_p/16], amax f32[1]
  *   divisor = qmax * smax * adjustment of the tensor's scale rule and rounding style
  *   out_type FOS_T_BF16 / FOS_T_F16 / FOS_T_F32, leading dimension ldo
+ *   intermediate_type FOS_T_F16 (the reference's default) or FOS_T_F32: the type in which
+ *   value and block scale are multiplied (`intermediate_dtype`); it matters for IF4's
+ *   integer blocks (factor 6/7) and for MXFP4 scales outside fp16's range
  * FOS_DTYPE_MXFP4: blocks of 32, E8M0 scales, amax and divisor are ignored (amax may be NULL).
  */
 int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const float *amax,
                    int dtype, int sf_layout, double divisor,
                    int64_t rows, int64_t cols, int64_t rows_p, int64_t cols_p,
-                   void *out, int out_type, int64_t ldo, fos_stream_t stream);
+                   void *out, int out_type, int64_t ldo, int intermediate_type, fos_stream_t stream);
 
 #ifdef __cplusplus
 }

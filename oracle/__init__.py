@@ -78,6 +78,8 @@ def lib() -> ctypes.CDLL:
         L.fos_oracle_from_blocked.restype = None
         L.fos_oracle_dequantize.argtypes = [vp, vp, f32, i32, c.c_double, i64, i64, vp, i32]
         L.fos_oracle_dequantize.restype = i32
+        L.fos_oracle_dequantize_ex.argtypes = [vp, vp, f32, i32, c.c_double, i64, i64, vp, i32, i32]
+        L.fos_oracle_dequantize_ex.restype = i32
         L.fos_oracle_matmul_nt.argtypes = [vp, vp, i64, i64, i64, vp, vp, i32]
         L.fos_oracle_matmul_nt.restype = None
         L.fos_oracle_gemm_nvfp4.argtypes = [vp, vp, vp, vp, f32, i64, i64, i64, vp, vp, i32]
@@ -219,16 +221,17 @@ def from_blocked(flat: np.ndarray, rows: int, cols: int) -> np.ndarray:
 
 def dequantize(values: np.ndarray, scale_rows: np.ndarray, amax, *, dtype="nvfp4",
                scale_rule="mse", round_style="nearest", original_shape=None,
-               threads=None) -> np.ndarray:
-    """f32 [M, N] = the reference's ``dequantize(..., dtype=float32)`` (fp16 intermediate)."""
+               threads=None, f32_intermediate=False) -> np.ndarray:
+    """f32 [M, N] = the reference's ``dequantize(..., dtype=float32)``; value and block scale
+    meet in fp16 (its default intermediate dtype) or, with ``f32_intermediate``, in fp32."""
     values = np.ascontiguousarray(values)
     scale_rows = np.ascontiguousarray(scale_rows)
     mp, half = values.shape
     qmax, smax = qmax_smax(dtype, scale_rule)
     div = qmax * smax * adjustment(round_style)
     out = np.zeros((mp, half * 2), dtype=np.float32)
-    rc = lib().fos_oracle_dequantize(_ptr(values), _ptr(scale_rows), float(amax), DTYPE_IDS[dtype],
-                                     div, mp, half * 2, _ptr(out), threads or default_threads())
+    rc = lib().fos_oracle_dequantize_ex(_ptr(values), _ptr(scale_rows), float(amax), DTYPE_IDS[dtype],
+                                        div, mp, half * 2, _ptr(out), threads or default_threads(), int(f32_intermediate))
     assert rc == 0
     if original_shape is not None:
         out = out[: original_shape[0], : original_shape[1]]
@@ -327,15 +330,17 @@ def quantize_mxfp4(x, *, scale_rule="static_6") -> OracleQuantized:
                            orig, (mp, np_), True)
 
 
-def dequantize_mxfp4(values: np.ndarray, scale_rows: np.ndarray, original_shape=None) -> np.ndarray:
+def dequantize_mxfp4(values: np.ndarray, scale_rows: np.ndarray, original_shape=None, f32_intermediate=False) -> np.ndarray:
     """f32 [M, N]: fp16(value) * fp16(2^(e - 127)), the product rounded to fp16 (the reference's
-    intermediate dtype; scales outside fp16's range become 0 or inf there), widened."""
+    intermediate dtype; scales outside fp16's range become 0 or inf there), widened; with
+    ``f32_intermediate`` the product is formed in fp32 (exact short of overflow)."""
     code = np.empty((values.shape[0], values.shape[1] * 2), dtype=np.uint8)
     code[:, 0::2] = values & 0xF
     code[:, 1::2] = values >> 4
-    v16 = (E2M1_VALUES[code & 7] * np.where(code & 8, np.float32(-1), np.float32(1))).astype(np.float16)
+    inter = np.float32 if f32_intermediate else np.float16
+    v16 = (E2M1_VALUES[code & 7] * np.where(code & 8, np.float32(-1), np.float32(1))).astype(inter)
     with np.errstate(over="ignore", invalid="ignore"):  # 0 * inf = NaN, as in the reference's fp16 product
-        s16 = np.ldexp(np.float64(1.0), scale_rows.astype(np.int32) - 127).astype(np.float16)
+        s16 = np.ldexp(np.float64(1.0), scale_rows.astype(np.int32) - 127).astype(inter)
         out = (v16 * np.repeat(s16, 32, axis=1)).astype(np.float32)
     if original_shape is not None:
         out = out[: original_shape[0], : original_shape[1]]

@@ -522,8 +522,10 @@ void fos_oracle_from_blocked(const uint8_t *blk, int64_t rows, int64_t cols, uin
 /* codes u8[M,N/2], sf row-major u8[M,N/16], out f32[M,N].  div = qmax*smax*adj of the
  * tensor's scale rule, as a double (it is rounded to f32 for the division, as torch
  * does for a Python-scalar divisor). */
-int fos_oracle_dequantize(const uint8_t *codes, const uint8_t *sf, float amax, int dtype,
-                          double div, int64_t M, int64_t N, float *out, int nthreads) {
+/* `f32_intermediate`: value and block scale meet in fp32 instead of fp16
+ * (dequantize(..., intermediate_dtype=torch.float32), quantize/backend.py:89-160). */
+int fos_oracle_dequantize_ex(const uint8_t *codes, const uint8_t *sf, float amax, int dtype,
+                             double div, int64_t M, int64_t N, float *out, int nthreads, int f32_intermediate) {
     if (N % 16 != 0) return -1;
     float fdiv = (float)div;
     float six_sevenths = (float)(6.0 / 7.0);
@@ -540,16 +542,22 @@ int fos_oracle_dequantize(const uint8_t *codes, const uint8_t *sf, float amax, i
                 float v;
                 if (is_int) {
                     int iv = (int8_t)(code << 4) >> 4;
-                    v = round_to_f16((float)iv * six_sevenths);
+                    v = (float)iv * six_sevenths;
+                    if (!f32_intermediate) v = round_to_f16(v);
                 } else {
                     v = fos_oracle_e2m1_decode(code);
                 }
-                float r16 = round_to_f16(v * s);
-                out[r * N + cb * 16 + i] = (r16 * amax) / fdiv;
+                float prod = f32_intermediate ? v * s : round_to_f16(v * s);
+                out[r * N + cb * 16 + i] = (prod * amax) / fdiv;
             }
         }
     }
     return 0;
+}
+
+int fos_oracle_dequantize(const uint8_t *codes, const uint8_t *sf, float amax, int dtype,
+                          double div, int64_t M, int64_t N, float *out, int nthreads) {
+    return fos_oracle_dequantize_ex(codes, sf, amax, dtype, div, M, N, out, nthreads, 0);
 }
 
 /* ---- matmul oracle (matmul/pytorch.py:42-52) --------------------------------------- */

@@ -174,8 +174,35 @@ def write_mxfp4_vectors(quantize, dequantize, quantized_matmul, QuantizationConf
     print("wrote mxfp4", len(out))
 
 
+def write_f32_intermediate_vectors(quantize, dequantize, QuantizationConfig) -> None:  # noqa: N803
+    """dequantize(..., intermediate_dtype=torch.float32) -- value and block scale multiplied in
+    fp32 instead of fp16 (quantize/backend.py:89-160), which the reference's own pseudo-quantize
+    test relies on -- for the formats where that changes the result: IF4 (integer blocks carry
+    the factor 6/7) and MXFP4 (scales outside fp16's range), NVFP4 for completeness."""
+    out: dict[str, np.ndarray] = {}
+    for name, kind, shape, seed in [("randn_256x128", "randn", (256, 128), 51), ("tiny_blocks_128x128", "tiny_blocks", (128, 128), 52),
+                                    ("ragged_100x80", "randn", (100, 80), 53), ("outlier_128x384", "outlier", (128, 384), 54)]:
+        x = make_input(kind, shape, seed)
+        for dtype, rule in (("if4", "mse"), ("if4", "abs_max"), ("mxfp4", "static_6"), ("nvfp4", "mse")):
+            if kind == "tiny_blocks" and dtype == "mxfp4":
+                x = (x.float() * 2.0**-30).bfloat16()  # block scales below fp16's range
+            q = quantize(x.clone(), QuantizationConfig(backend="pytorch", dtype=dtype, scale_rule=rule))
+            key = f"{name}.{dtype}.{rule}"
+            out[key + ".values"] = u8(q.values)
+            out[key + ".sf"] = u8(q.scale_factors)
+            out[key + ".amax"] = np.array([float(q.amax)], dtype=np.float32)
+            out[key + ".shape"] = np.array(shape)
+            out[key + ".padded"] = np.array(q.padded_shape)
+            out[key + ".blocked"] = np.array([int(q.scale_factors_are_in_blackwell_layout)])
+            out[key + ".deq_bf16"] = bits(dequantize(q, torch.bfloat16, intermediate_dtype=torch.float32))
+            out[key + ".deq_f32"] = dequantize(q, torch.float32, intermediate_dtype=torch.float32).numpy().copy()
+    np.savez_compressed(os.path.join(HERE, "dequantize_f32_intermediate.npz"), **out)
+    print("wrote dequantize_f32_intermediate", len(out))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--only-dequant32", action="store_true", help="write only dequantize_f32_intermediate.npz")
     ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
     ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
     ap.add_argument("--only-mxfp4", action="store_true", help="write only mxfp4.npz")
@@ -185,6 +212,9 @@ def main() -> None:
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_f32_intermediate_vectors(quantize, dequantize, QuantizationConfig)
+    if args.only_dequant32:
+        return
     if not args.only_mxfp4:
         write_transform_vectors()
     if not args.only_transform:

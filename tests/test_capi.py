@@ -86,9 +86,10 @@ def test_argument_checks_need_no_device(native):
     assert g(out=2) == -3
     d = lambda **kw: L.fos_dequantize(  # noqa: E731
         kw.get("codes", p), p, p, kw.get("dtype", 0), 1, 1536.0, kw.get("rows", 128), 64,
-        kw.get("rows_p", 128), 64, p, kw.get("out", 0), 64, None)
+        kw.get("rows_p", 128), 64, p, kw.get("out", 0), 64, kw.get("inter", 1), None)
     assert d(codes=None) == -4
     assert d(rows=200) == -1
     assert d(rows_p=100, rows=100) == -1
     assert d(dtype=3) == -3
     assert d(out=9) == -3
+    assert d(inter=0) == -3  # value x scale meets in fp16 or fp32 only

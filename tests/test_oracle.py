@@ -262,3 +262,28 @@ def test_mxfp4_matches_reference_vectors(oracle, golden_dir):
         ref = d[f"mm.{tag}.out"]
         got = o16[:m, :nn]
         assert float((got != ref).mean()) <= 1e-3
+
+
+def test_dequantize_with_f32_intermediate_matches_reference_vectors(oracle, golden_dir):
+    """dequantize(..., intermediate_dtype=float32) of the reference on IF4 (integer blocks carry
+    6/7), MXFP4 (scales below fp16's range) and NVFP4 codes written by the reference itself."""
+    z = np.load(os.path.join(golden_dir, "dequantize_f32_intermediate.npz"))
+    keys = sorted({k.rsplit(".", 1)[0] for k in z.files})
+    assert len(keys) == 16
+    differs = 0
+    for key in keys:
+        _, dtype, rule = key.split(".")
+        values, sf, shape, padded = z[key + ".values"], z[key + ".sf"], z[key + ".shape"], z[key + ".padded"]
+        if dtype == "mxfp4":
+            rows = oracle.from_blocked(sf, int(padded[0]), int(padded[1]) // 32)
+            got = oracle.dequantize_mxfp4(values, rows, tuple(shape), f32_intermediate=True)
+            other = oracle.dequantize_mxfp4(values, rows, tuple(shape))
+        else:
+            rows = oracle.from_blocked(sf, int(padded[0]), int(padded[1]) // 16) if int(z[key + ".blocked"][0]) else sf.reshape(int(padded[0]), -1)
+            kw = dict(dtype=dtype, scale_rule=rule, original_shape=tuple(shape))
+            got = oracle.dequantize(values, rows, float(z[key + ".amax"][0]), f32_intermediate=True, **kw)
+            other = oracle.dequantize(values, rows, float(z[key + ".amax"][0]), **kw)
+        assert np.array_equal(got.view(np.uint32), z[key + ".deq_f32"].view(np.uint32)), key
+        assert np.array_equal(oracle.f32_to_bf16_bits(got), z[key + ".deq_bf16"]), key
+        differs += int(not np.array_equal(got.view(np.uint32), other.view(np.uint32)))
+    assert differs >= 4  # the option matters on the IF4 / out-of-range MXFP4 cases

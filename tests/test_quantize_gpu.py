@@ -300,6 +300,31 @@ def test_dequantize_bit_exact(oracle, dtype, rule, out):
                        expect.view(torch.int16 if out != torch.float32 else torch.int32))
 
 
+def test_dequantize_with_f32_intermediate_matches_reference_vectors(golden_dir):
+    """dequantize(..., intermediate_dtype=torch.float32) on codes and scales written by the
+    reference (IF4 with integer blocks, MXFP4 with scales below fp16's range, NVFP4), against
+    the reference's own outputs, bit for bit."""
+    from fouroversix_amd.utils import DataType, RoundStyle, ScaleRule
+
+    z = np.load(os.path.join(golden_dir, "dequantize_f32_intermediate.npz"))
+    keys = sorted({k.rsplit(".", 1)[0] for k in z.files})
+    assert len(keys) == 16
+    for key in keys:
+        _, dtype, rule = key.split(".")
+        sf = torch.from_numpy(z[key + ".sf"].reshape(-1).copy()).cuda()
+        sf = sf.view(torch.float8_e8m0fnu if dtype == "mxfp4" else torch.float8_e4m3fn)
+        q = fos.QuantizedTensor(
+            torch.from_numpy(z[key + ".values"].copy()).cuda(), sf,
+            torch.tensor(float(z[key + ".amax"][0]), device="cuda"), DataType(dtype), tuple(int(v) for v in z[key + ".shape"]),
+            ScaleRule(rule), RoundStyle.nearest, tuple(int(v) for v in z[key + ".padded"]),
+            scale_factors_are_in_blackwell_layout=bool(z[key + ".blocked"][0]),
+        )
+        got32 = fos.dequantize(q, torch.float32, intermediate_dtype=torch.float32).cpu().numpy()
+        assert np.array_equal(got32.view(np.uint32), z[key + ".deq_f32"].view(np.uint32)), key
+        got16 = fos.dequantize(q, torch.bfloat16, intermediate_dtype=torch.float32)
+        assert np.array_equal(bits16(got16), z[key + ".deq_bf16"]), key
+
+
 @pytest.mark.parametrize("two_d", [False, True])
 @pytest.mark.parametrize("rule", ["mse", "mae", "abs_max", "static_6", "static_4"])
 @pytest.mark.parametrize(
