@@ -95,6 +95,23 @@ FOS_DEVICE float row16_sum_lane0(float v) {
     return __shfl(v, lane & 48);
 }
 
+// Certified comparison of two candidates' errors h_a^2 S_a and h_b^2 S_b from their
+// scaled-domain sums (S already summed over the tile when TWO_D): returns +1 when the
+// second is surely smaller, -1 when it is surely not smaller (the first wins, also on a
+// tie), 0 when the two tolerance intervals overlap.
+// Tolerance 2^-14 (c1 sqrt(S) + c2 S) with sqrt(S) <= (1 + S) / 2.
+template <bool TWO_D>
+FOS_DEVICE int shortcut_compare(float SA, float hA, float SB, float hB) {
+    constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
+    constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
+    const float EA = hA * SA, EB = hB * SB;
+    const float tA = hA * __builtin_fmaf(k1, SA, k0);
+    const float tB = hB * __builtin_fmaf(k1, SB, k0);
+    if (EB + tB < EA - tA) return 1;
+    if (EB - tB > EA + tA) return -1;
+    return 0;
+}
+
 // The two rare paths are real function calls (arguments and results by value, in
 // registers) written as rolled loops over the eight column pairs (l, l + 8) -- the order
 // in which torch.sum consumes a block -- so that their register needs and code size stay
@@ -335,16 +352,9 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                         SA = row16_sum_lane0(SA);
                         SB = row16_sum_lane0(SB);
                     }
-                    constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
-                    constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
-                    const float hA = A.d1 * A.d1, hB = B.d1 * B.d1;
-                    const float EA = hA * SA, EB = hB * SB;
-                    const float tA = hA * __builtin_fmaf(k1, SA, k0);
-                    const float tB = hB * __builtin_fmaf(k1, SB, k0);
-                    const bool surely_b = EB + tB < EA - tA;
-                    const bool surely_a = EB - tB > EA + tA;
-                    certain = surely_a || surely_b;
-                    pickB = surely_b;
+                    const int cmp = shortcut_compare<TWO_D>(SA, A.d1 * A.d1, SB, B.d1 * B.d1);
+                    certain = cmp != 0;
+                    pickB = cmp > 0;
                 }
                 if (!certain) {
                     bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
@@ -394,17 +404,9 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     SA = row16_sum_lane0(SA);
                     SB = row16_sum_lane0(SB);
                 }
-                // tolerance 2^-14 (c1 sqrt(S) + c2 S) with sqrt(S) <= (1 + S) / 2
-                constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
-                constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
-                const float hA = A.d1 * A.d1, hB = B.d1 * B.d1;
-                const float EA = hA * SA, EB = hB * SB;
-                const float tA = hA * __builtin_fmaf(k1, SA, k0);
-                const float tB = hB * __builtin_fmaf(k1, SB, k0);
-                const bool surely_b = EB + tB < EA - tA;
-                const bool surely_a = EB - tB > EA + tA;
-                certain = surely_a || surely_b;
-                pickB = surely_b;
+                const int cmp = shortcut_compare<TWO_D>(SA, A.d1 * A.d1, SB, B.d1 * B.d1);
+                certain = cmp != 0;
+                pickB = cmp > 0;
             }
             if (!certain) {
                 // exact ties by construction first (cheap), the full evaluation otherwise
@@ -492,13 +494,9 @@ FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts
                 SA = row16_sum_lane0(SA);
                 SB = row16_sum_lane0(SB);
             }
-            constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
-            constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
-            const float tA = __builtin_fmaf(k1, SA, k0), tB = __builtin_fmaf(k1, SB, k0);
-            const bool surely_int = SB + tB < SA - tA;
-            const bool surely_fp = SB - tB > SA + tA;
-            if (surely_int) return BlockOut{b0, b1, s | 0x80u};
-            if (surely_fp) return BlockOut{a0, a1, s};
+            const int cmp = shortcut_compare<TWO_D>(SA, 1.0f, SB, 1.0f);  // same scale: compare the sums
+            if (cmp > 0) return BlockOut{b0, b1, s | 0x80u};
+            if (cmp < 0) return BlockOut{a0, a1, s};
             // undecided (uniform over the 16 lanes of a tile when TWO_D: both sums are tile sums)
         } else if (bmax == 0.0f) {
             return BlockOut{0, 0, 0};
