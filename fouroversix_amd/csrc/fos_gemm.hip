@@ -303,15 +303,19 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 // k = 256 step + 128 h ... of B row n0 + 32 t + r with the same codes of A rows r + 32 i.
 // The MFMA contraction index is thereby permuted (slice x pairs codes 8x..8x+7 of both
 // lane halves); A and B use the same permutation, so the sum is unchanged.
-//  * B codes come straight from global memory (64 contiguous bytes per lane).
 //  * A codes are re-read by every workgroup, so their path through the vector cache
 //    matters: a wavefront loads its A step with 8 lanes per 128-byte row segment (whole
 //    cache lines) and transposes it through a private LDS region into the per-row
 //    fragment order (LDS operations of one wavefront execute in order: no barrier).
+//  * B codes take the same route for M <= 64; a lane loading its own 64 bytes would
+//    touch every line with four instructions, and with a few thousand lines in flight per
+//    CU the vector cache refetches them.  For M = 128 the A regions leave no room and B
+//    goes straight from global memory to the lane that multiplies it.
 //  * Scales: the 128x4 tiled layout puts the four blocks of a 64-wide K group of rows r,
 //    r + 32, r + 64, r + 96 next to each other, so one 128-bit load per group fetches the
 //    scales of all A rows of a lane; B takes one 32-bit word per group.
 // The 8 partial accumulators are tree-reduced through LDS at the end (fixed order).
+constexpr int kSkinnyRotation = 5;  // K steps between the starting points of neighbouring workgroups (odd: 8 in a row are in flight)
 constexpr int kSkinnyPitch = 144;  // LDS bytes per A row (128 + 16: conflict-free 128-bit accesses)
 
 template <int MT, int WN>
@@ -324,7 +328,11 @@ struct SkinnyRegs {
 template <int MT, int WN, int OUT>
 __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
     constexpr int kWaves = 8, kAcc = MT * WN * 16;
-    constexpr int kRegion = MT * 32 * kSkinnyPitch;
+    // B through LDS as well (whole cache lines per load instruction, see above) where the
+    // second staging region fits next to A's
+    constexpr bool kBViaLds = MT <= 2;
+    constexpr int kRegionA = MT * 32 * kSkinnyPitch;
+    constexpr int kRegion = kRegionA + (kBViaLds ? WN * 32 * kSkinnyPitch : 0);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // the wave index steers loops and scalar buffer offsets: make its uniformity known
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 31, h = lane >> 5;
@@ -335,6 +343,17 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
     const int64_t s_end = OUT == kOutPartial ? (s_begin + p.ksteps_per_split < steps_all ? s_begin + p.ksteps_per_split : steps_all)
                                              : steps_all;
+
+    // Workgroups start at different K offsets and wrap around: started together at K = 0 they
+    // would all ask the same few memory channels for the same columns of their rows at the
+    // same time (rows are K / 2 bytes apart, typically a power of two).  The order of
+    // accumulation of a column block thereby depends on its index, and on nothing else.
+    const int64_t nsteps = s_end - s_begin;
+    const int64_t rot_wg = nsteps > 0 ? ((int64_t)blockIdx.x * kSkinnyRotation) % nsteps : 0;
+    auto phys = [&](int64_t j) -> int64_t {  // j-th step of this workgroup -> K step
+        const int64_t q = j + rot_wg;
+        return s_begin + (q >= nsteps ? q - nsteps : q);
+    };
 
     // rows of A past M read as zero codes (buffer range check), so A needs only M rows
     const BufferRsrc ra = make_rsrc(p.A, (uint32_t)(p.M * kbytes));
@@ -355,20 +374,29 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
             a_stage[j] = __builtin_bit_cast(
                 uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)(a_off + j * 8 * kbytes), (int)(step * 128), 0));
     };
-    auto fetch_b = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
-        const int kq = (int)(step * 128), ksf = (int)(step * 2048);
+    auto fetch_b_codes = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
+        const int kq = (int)(step * 128);
 #pragma unroll
-        for (int t = 0; t < WN; ++t) {
+        for (int t = 0; t < WN; ++t)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 s.b[t][q] = __builtin_bit_cast(
-                    uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
+                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(a_off + (t * 32 + q * 8) * kbytes), kq, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
+    };
+    auto fetch_scales = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
+        const int ksf = (int)(step * 2048);
+#pragma unroll
+        for (int t = 0; t < WN; ++t)
 #pragma unroll
             for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)(sb_off + t * 4 + u * 512), ksf, 0);
-        }
 #pragma unroll
         for (int u = 0; u < 2; ++u)
             s.sa[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsa, (int)(sa_off + u * 512), ksf, 0));
+    };
+    auto fetch_b = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
+        fetch_b_codes(step, s);
+        fetch_scales(step, s);
     };
 
     float16_t acc[MT][WN];
@@ -389,25 +417,46 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 #pragma unroll
         for (int i = 0; i < MT; ++i) fr[i] = *reinterpret_cast<const uint4 *>(region + lds_r + i * 32 * kSkinnyPitch + q * 16);
     };
-    // one step: A codes staged in `a_stage` go through LDS, the next step's A load is issued,
-    // then 16 K slices are multiplied
-    auto compute = [&](const SkinnyRegs<MT, WN> &s, int64_t next_step) {
+    auto read_frags_b = [&](int q, uint4 *fr) {
+#pragma unroll
+        for (int t = 0; t < WN; ++t)
+            fr[t] = *reinterpret_cast<const uint4 *>(region + kRegionA + lds_r + t * 32 * kSkinnyPitch + q * 16);
+    };
+    // one step: the staged codes go through LDS, the loads that refill the staging registers
+    // are issued (A for the wavefront's next step first: it is needed first and loads return
+    // in order; then, where B is staged too, the codes of this register set's step after
+    // next: the scales stay in use and follow after the multiplication), then 16 K slices
+    // are multiplied
+    auto compute = [&](SkinnyRegs<MT, WN> &s, int64_t next_step, int64_t refill_step) {
 #pragma unroll
         for (int j = 0; j < MT * 4; ++j) *reinterpret_cast<uint4 *>(region + lds_w + j * 8 * kSkinnyPitch) = a_stage[j];
+        if (kBViaLds) {
+#pragma unroll
+            for (int t = 0; t < WN; ++t)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<uint4 *>(region + kRegionA + lds_w + (t * 32 + q * 8) * kSkinnyPitch) = s.b[t][q];
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        uint4 fr[2][MT];
+        uint4 fr[2][MT], frb[2][WN];
         read_frags(0, fr[0]);
-        if (next_step < s_end) fetch_a(next_step);
+        if (kBViaLds) read_frags_b(0, frb[0]);
+        if (next_step < nsteps) fetch_a(phys(next_step));
+        if (kBViaLds && refill_step < nsteps) fetch_b_codes(phys(refill_step), s);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            if (q + 1 < 4) read_frags(q + 1, fr[(q + 1) & 1]);
+            if (q + 1 < 4) {
+                read_frags(q + 1, fr[(q + 1) & 1]);
+                if (kBViaLds) read_frags_b(q + 1, frb[(q + 1) & 1]);
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int x = q * 4 + j;
                 half8_t fb[WN], fa[MT];
 #pragma unroll
-                for (int t = 0; t < WN; ++t) fb[t] = dequant8(word_of(s.b[t][q], j), scale_of(s.sb[t][x >> 3], x));
+                for (int t = 0; t < WN; ++t)
+                    fb[t] = dequant8(word_of(kBViaLds ? frb[q & 1][t] : s.b[t][q], j), scale_of(s.sb[t][x >> 3], x));
 #pragma unroll
                 for (int i = 0; i < MT; ++i) fa[i] = dequant8(word_of(fr[q & 1][i], j), scale_of(word_of(s.sa[x >> 3], i), x));
 #pragma unroll
@@ -423,18 +472,24 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     };
 
     SkinnyRegs<MT, WN> st[2];
-    int64_t step = s_begin + wave;
-    if (step < s_end) {
-        fetch_a(step);
-        fetch_b(step, st[0]);
+    int64_t step = wave;
+    if (step < nsteps) {
+        fetch_a(phys(step));
+        fetch_b(phys(step), st[0]);
     }
-    if (step + kWaves < s_end) fetch_b(step + kWaves, st[1]);
-    for (; step < s_end; step += 2 * kWaves) {
-        compute(st[0], step + kWaves);
-        if (step + 2 * kWaves < s_end) fetch_b(step + 2 * kWaves, st[0]);
-        if (step + kWaves < s_end) {
-            compute(st[1], step + 2 * kWaves);
-            if (step + 3 * kWaves < s_end) fetch_b(step + 3 * kWaves, st[1]);
+    if (step + kWaves < nsteps) fetch_b(phys(step + kWaves), st[1]);
+    for (; step < nsteps; step += 2 * kWaves) {
+        compute(st[0], step + kWaves, step + 2 * kWaves);
+        if (step + 2 * kWaves < nsteps) {
+            if (!kBViaLds) fetch_b_codes(phys(step + 2 * kWaves), st[0]);
+            fetch_scales(phys(step + 2 * kWaves), st[0]);
+        }
+        if (step + kWaves < nsteps) {
+            compute(st[1], step + 2 * kWaves, step + 3 * kWaves);
+            if (step + 3 * kWaves < nsteps) {
+                if (!kBViaLds) fetch_b_codes(phys(step + 3 * kWaves), st[1]);
+                fetch_scales(phys(step + 3 * kWaves), st[1]);
+            }
         }
     }
 
@@ -572,7 +627,7 @@ static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
 
 template <int MT, int WN>
 static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
-    constexpr size_t stage_bytes = (size_t)8 * MT * 32 * kSkinnyPitch, red_bytes = (size_t)4 * (MT * WN * 16) * 64 * sizeof(float);
+    constexpr size_t stage_bytes = (size_t)8 * (MT * 32 + (MT <= 2 ? WN * 32 : 0)) * kSkinnyPitch, red_bytes = (size_t)4 * (MT * WN * 16) * 64 * sizeof(float);
     constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
     dim3 grid((unsigned)(p.N / (32 * WN)), (unsigned)p.splits);
     auto kernel = p.splits > 1 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutPartial>
