@@ -318,11 +318,26 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 constexpr int kSkinnyRotation = 5;  // K steps between the starting points of neighbouring workgroups (odd: 8 in a row are in flight)
 constexpr int kSkinnyPitch = 144;  // LDS bytes per A row (128 + 16: conflict-free 128-bit accesses)
 
+// N consecutive 32-bit words (N = 1, 2, 4) with one buffer load.
+template <int N>
+FOS_DEVICE void load_words(uint32_t (&dst)[N], BufferRsrc r, int voffset, int soffset) {
+    static_assert(N == 1 || N == 2 || N == 4, "one load instruction");
+    if constexpr (N == 1) {
+        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0);
+    } else if constexpr (N == 2) {
+        const auto v = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r, voffset, soffset, 0));
+        dst[0] = v.x, dst[1] = v.y;
+    } else {
+        const auto v = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, voffset, soffset, 0));
+        dst[0] = v.x, dst[1] = v.y, dst[2] = v.z, dst[3] = v.w;
+    }
+}
+
 template <int MT, int WN>
 struct SkinnyRegs {
     uint4 b[WN][4];     // 128 codes of each B row
     uint32_t sb[WN][2]; // their 8 block scales (two groups)
-    uint4 sa[2];        // block scales of the A rows: [group] word i = row r + 32 i
+    uint32_t sa[2][MT]; // block scales of the A rows: [group][i] = row r + 32 i
 };
 
 template <int MT, int WN, int OUT>
@@ -367,36 +382,43 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     const uint32_t lds_w = (uint32_t)((lane >> 3) * kSkinnyPitch + (lane & 7) * 16);
     const uint32_t lds_r = (uint32_t)(r * kSkinnyPitch + h * 64);
 
+    // Loads are issued unconditionally, so that the wait counts in the loop below are exact
+    // (a load under a branch makes the compiler wait for everything in flight, the prefetches
+    // just issued included): a step past the end reads through a descriptor of size zero,
+    // which returns zeros without touching memory.
+    const BufferRsrc r_none = make_rsrc(p.A, 0);
     uint4 a_stage[MT * 4];  // one A step in flight from global memory
-    auto fetch_a = [&](int64_t step) {
+    auto fetch_a = [&](int64_t j) {
+        const bool ok = j < nsteps;
+        const BufferRsrc r = ok ? ra : r_none;
+        const int kq = ok ? (int)(phys(j) * 128) : 0;
 #pragma unroll
-        for (int j = 0; j < MT * 4; ++j)
-            a_stage[j] = __builtin_bit_cast(
-                uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)(a_off + j * 8 * kbytes), (int)(step * 128), 0));
+        for (int i = 0; i < MT * 4; ++i)
+            a_stage[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + i * 8 * kbytes), kq, 0));
     };
-    auto fetch_b_codes = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
-        const int kq = (int)(step * 128);
+    auto fetch_b_codes = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
+        const bool ok = j < nsteps;
+        const BufferRsrc r = ok ? rb : r_none;
+        const int kq = ok ? (int)(phys(j) * 128) : 0;
 #pragma unroll
         for (int t = 0; t < WN; ++t)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 s.b[t][q] = __builtin_bit_cast(
-                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(a_off + (t * 32 + q * 8) * kbytes), kq, 0)
-                                    : __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
+                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (t * 32 + q * 8) * kbytes), kq, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
     };
-    auto fetch_scales = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
-        const int ksf = (int)(step * 2048);
+    auto fetch_scales = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
+        const bool ok = j < nsteps;
+        const BufferRsrc r_a = ok ? rsa : r_none, r_b = ok ? rsb : r_none;
+        const int ksf = ok ? (int)(phys(j) * 2048) : 0;
 #pragma unroll
         for (int t = 0; t < WN; ++t)
 #pragma unroll
-            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)(sb_off + t * 4 + u * 512), ksf, 0);
+            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(r_b, (int)(sb_off + t * 4 + u * 512), ksf, 0);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
-            s.sa[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsa, (int)(sa_off + u * 512), ksf, 0));
-    };
-    auto fetch_b = [&](int64_t step, SkinnyRegs<MT, WN> &s) {
-        fetch_b_codes(step, s);
-        fetch_scales(step, s);
+            load_words<MT>(s.sa[u], r_a, (int)(sa_off + u * 512), ksf);
     };
 
     float16_t acc[MT][WN];
@@ -442,8 +464,15 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
         uint4 fr[2][MT], frb[2][WN];
         read_frags(0, fr[0]);
         if (kBViaLds) read_frags_b(0, frb[0]);
-        if (next_step < nsteps) fetch_a(phys(next_step));
-        if (kBViaLds && refill_step < nsteps) fetch_b_codes(phys(refill_step), s);
+        // the refills go out here, ahead of the arithmetic: the scheduler may not sink them
+        if constexpr (kBViaLds) {
+            __builtin_amdgcn_sched_barrier(0);
+            fetch_a(next_step);
+            fetch_b_codes(refill_step, s);
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            if (next_step < nsteps) fetch_a(next_step);
+        }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             if (q + 1 < 4) {
@@ -458,7 +487,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
                 for (int t = 0; t < WN; ++t)
                     fb[t] = dequant8(word_of(kBViaLds ? frb[q & 1][t] : s.b[t][q], j), scale_of(s.sb[t][x >> 3], x));
 #pragma unroll
-                for (int i = 0; i < MT; ++i) fa[i] = dequant8(word_of(fr[q & 1][i], j), scale_of(word_of(s.sa[x >> 3], i), x));
+                for (int i = 0; i < MT; ++i) fa[i] = dequant8(word_of(fr[q & 1][i], j), scale_of(s.sa[x >> 3][i], x));
 #pragma unroll
                 for (int i = 0; i < MT; ++i)
 #pragma unroll
@@ -472,23 +501,38 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     };
 
     SkinnyRegs<MT, WN> st[2];
-    int64_t step = wave;
-    if (step < nsteps) {
-        fetch_a(phys(step));
-        fetch_b(phys(step), st[0]);
-    }
-    if (step + kWaves < nsteps) fetch_b(phys(step + kWaves), st[1]);
-    for (; step < nsteps; step += 2 * kWaves) {
-        compute(st[0], step + kWaves, step + 2 * kWaves);
-        if (step + 2 * kWaves < nsteps) {
-            if (!kBViaLds) fetch_b_codes(phys(step + 2 * kWaves), st[0]);
-            fetch_scales(phys(step + 2 * kWaves), st[0]);
-        }
-        if (step + kWaves < nsteps) {
+    int64_t step = wave;  // counts this workgroup's steps, see phys()
+    if constexpr (kBViaLds) {
+        fetch_a(step);
+        fetch_b_codes(step, st[0]);
+        fetch_scales(step, st[0]);
+        fetch_b_codes(step + kWaves, st[1]);
+        fetch_scales(step + kWaves, st[1]);
+        for (; step + kWaves < nsteps; step += 2 * kWaves) {
+            compute(st[0], step + kWaves, step + 2 * kWaves);
+            fetch_scales(step + 2 * kWaves, st[0]);
             compute(st[1], step + 2 * kWaves, step + 3 * kWaves);
-            if (step + 3 * kWaves < nsteps) {
-                if (!kBViaLds) fetch_b_codes(phys(step + 3 * kWaves), st[1]);
-                fetch_scales(phys(step + 3 * kWaves), st[1]);
+            fetch_scales(step + 3 * kWaves, st[1]);
+        }
+        if (step < nsteps) compute(st[0], nsteps, nsteps);  // odd count: the last step, nothing left to fetch
+    } else {
+        // 256 registers are in use here: the loads stay under branches, which costs the exact
+        // wait counts but keeps the accumulators out of scratch memory
+        auto fetch_b = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
+            fetch_b_codes(j, s);
+            fetch_scales(j, s);
+        };
+        if (step < nsteps) {
+            fetch_a(step);
+            fetch_b(step, st[0]);
+        }
+        if (step + kWaves < nsteps) fetch_b(step + kWaves, st[1]);
+        for (; step < nsteps; step += 2 * kWaves) {
+            compute(st[0], step + kWaves, 0);
+            if (step + 2 * kWaves < nsteps) fetch_b(step + 2 * kWaves, st[0]);
+            if (step + kWaves < nsteps) {
+                compute(st[1], step + 2 * kWaves, 0);
+                if (step + 3 * kWaves < nsteps) fetch_b(step + 3 * kWaves, st[1]);
             }
         }
     }
