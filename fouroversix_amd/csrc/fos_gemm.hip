@@ -31,6 +31,7 @@ namespace fos {
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
 
 struct GemmParams {
     const uint8_t *A, *B;      // [M, K/2], [N, K/2]
@@ -500,6 +501,9 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
         __builtin_amdgcn_wave_barrier();
     };
 
+    // read now, used in the epilogue: short launches would otherwise end on this latency
+    const float alpha = OUT == kOutPartial ? 0.0f : load_alpha(p);
+
     SkinnyRegs<MT, WN> st[2];
     int64_t step = wave;  // counts this workgroup's steps, see phys()
     if constexpr (kBViaLds) {
@@ -583,7 +587,6 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
         }
         return;
     }
-    const float alpha = load_alpha(p);
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
@@ -607,6 +610,163 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
                 *reinterpret_cast<uint2 *>(D + (int64_t)(32 * i + r) * p.ldd + n0 + 32 * t + 8 * g + 4 * h) =
                     make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
             }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// M <= 16 (decode batches).  Same decomposition as the weight-streaming kernel above (32 rows
+// of B per workgroup, 8 wavefronts share the K steps of 256, staggered start, tree reduction),
+// built on the 16 x 16 x 32 MFMA: a 32 x 32 tile would spend half of its rows, and half of
+// the activation conversions, on padding.
+//
+// Lane l = (c = l & 15, g = l >> 4).  Per step it holds the 64 codes k = 256 step + 64 g ...
+// of B rows n0 + c and n0 + 16 + c and of A row c: 32 contiguous bytes each, whose four
+// blocks are exactly one scale group (one 32-bit word of the tiled layout).  MFMA slice
+// s = 0..7 multiplies 32-bit word s of every lane, i.e. the contraction index is permuted
+// (slice s pairs codes 8 s ... 8 s + 7 of all four lane groups), identically for both
+// operands.  Operands go from global memory to registers to the MFMA: no LDS in the loop.
+// acc[b][e] is D[m = c][n = n0 + 16 b + 4 g + e].
+struct DecodeRegs {
+    uint4 b[2][2];   // 64 codes of two B rows
+    uint4 a[2];      // 64 codes of the A row
+    uint32_t sb[2];  // their scale groups
+    uint32_t sa;
+};
+
+template <int OUT>
+__global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams p) {
+    constexpr int kWaves = 8, kDepth = 3;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), c = lane & 15, g = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * 32;
+    const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
+    const int64_t steps_all = p.K >> 8;
+    const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
+    const int64_t s_end = OUT == kOutPartial ? (s_begin + p.ksteps_per_split < steps_all ? s_begin + p.ksteps_per_split : steps_all)
+                                             : steps_all;
+    // staggered start, as in the weight-streaming kernel
+    const int64_t nsteps = s_end - s_begin;
+    const int64_t rot_wg = nsteps > 0 ? ((int64_t)blockIdx.x * kSkinnyRotation) % nsteps : 0;
+    auto phys = [&](int64_t j) -> int64_t {
+        const int64_t q = j + rot_wg;
+        return s_begin + (q >= nsteps ? q - nsteps : q);
+    };
+
+    // rows of A past M read as zero codes (buffer range check); loads past the last step go
+    // through the empty descriptor, so that none of them sits under a branch
+    const BufferRsrc ra = make_rsrc(p.A, (uint32_t)(p.M * kbytes));
+    const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(32 * kbytes));
+    const BufferRsrc rsa = make_rsrc(p.sfA, (uint32_t)(sf_groups * 512));
+    const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
+    const BufferRsrc r_none = make_rsrc(p.A, 0);
+    const uint32_t q_off = (uint32_t)(c * kbytes + g * 32);
+    const uint32_t sa_off = (uint32_t)(g * 512 + c * 16);
+    const uint32_t sb_off = (uint32_t)(g * 512 + c * 16 + (((uint32_t)n0 & 127u) >> 5) * 4);
+
+    auto fetch = [&](int64_t j, DecodeRegs &s) {
+        const bool ok = j < nsteps;
+        const BufferRsrc qa = ok ? ra : r_none, qb = ok ? rb : r_none, fa = ok ? rsa : r_none, fb = ok ? rsb : r_none;
+        const int kq = ok ? (int)(phys(j) * 128) : 0, ksf = ok ? (int)(phys(j) * 2048) : 0;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                s.b[b][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qb, (int)(q_off + b * 16 * kbytes + u * 16), kq, 0));
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            s.a[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qa, (int)(q_off + u * 16), kq, 0));
+#pragma unroll
+        for (int b = 0; b < 2; ++b) s.sb[b] = __builtin_amdgcn_raw_buffer_load_b32(fb, (int)(sb_off + b * 256), ksf, 0);
+        s.sa = __builtin_amdgcn_raw_buffer_load_b32(fa, (int)sa_off, ksf, 0);
+    };
+
+    float4_t acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    auto word_of = [](const uint4 &v, int j) -> uint32_t { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; };
+    // scale of code word x (0..7) of a lane: block x >> 1 = byte x >> 1 of the group word
+    auto scale_of = [](uint32_t w, int x) -> half2_t {
+        const half2_t s2 = e4m3x2_to_half2((x & 4) ? w >> 16 : w);
+        return ((x >> 1) & 1) ? __builtin_shufflevector(s2, s2, 1, 1) : __builtin_shufflevector(s2, s2, 0, 0);
+    };
+    auto compute = [&](const DecodeRegs &s) {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const half8_t fa = dequant8(word_of(s.a[x >> 2], x & 3), scale_of(s.sa, x));
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const half8_t fb = dequant8(word_of(s.b[b][x >> 2], x & 3), scale_of(s.sb[b], x));
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, fa, acc[b], 0, 0, 0);
+            }
+        }
+    };
+
+    // read now, used in the epilogue: short launches would otherwise end on this latency
+    const float alpha = OUT == kOutPartial ? 0.0f : load_alpha(p);
+
+    DecodeRegs st[kDepth];
+    int64_t step = wave;  // counts this workgroup's steps, see phys()
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) fetch(step + d * kWaves, st[d]);
+    for (; step + (kDepth - 1) * kWaves < nsteps; step += kDepth * kWaves) {
+#pragma unroll
+        for (int d = 0; d < kDepth; ++d) {
+            compute(st[d]);
+            // the refill goes out here: the scheduler may not collect the loads at the loop's end
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(step + (d + kDepth) * kWaves, st[d]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d + 1 < kDepth; ++d)
+        if (step + d * kWaves < nsteps) compute(st[d]);  // the last, incomplete round
+
+    // tree reduction of the 8 wavefronts' accumulators (fixed order, hence deterministic)
+    float *red = reinterpret_cast<float *>(smem);
+#pragma unroll
+    for (int stride = kWaves / 2; stride >= 1; stride >>= 1) {
+        if (wave >= stride && wave < 2 * stride) {
+            float *slot = red + (wave - stride) * (8 * 64);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) slot[(b * 4 + e) * 64 + lane] = acc[b][e];
+        }
+        __syncthreads();
+        if (wave < stride) {
+            const float *slot = red + wave * (8 * 64);
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[b][e] += slot[(b * 4 + e) * 64 + lane];
+        }
+        __syncthreads();
+    }
+    if (wave != 0 || c >= p.M) return;
+
+    if (OUT == kOutPartial) {
+        float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+            *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n0 + 16 * b + 4 * g) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+        return;
+    }
+    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+        uint16_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float v = alpha * acc[b][e];
+            if (OUT == kOutBF16) {
+                uint32_t u = f2u(v);
+                u += 0x7fffu + ((u >> 16) & 1u);
+                o[e] = (uint16_t)(u >> 16);
+            } else {
+                o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
+            }
+        }
+        *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n0 + 16 * b + 4 * g) =
+            make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
     }
 }
 
@@ -690,6 +850,22 @@ static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
+static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
+    constexpr size_t lds_bytes = (size_t)4 * 8 * 64 * sizeof(float);
+    dim3 grid((unsigned)(p.N / 32), (unsigned)p.splits);
+    auto kernel = p.splits > 1 ? gemm_nvfp4_decode_kernel<kOutPartial>
+                  : out_type == FOS_T_BF16 ? gemm_nvfp4_decode_kernel<kOutBF16> : gemm_nvfp4_decode_kernel<kOutF16>;
+    hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
+    if (hipGetLastError() != hipSuccess) return FOS_E_LAUNCH;
+    if (p.splits > 1) {
+        const int64_t quads = p.M * (p.N >> 2);
+        dim3 rgrid((unsigned)((quads + 255) / 256));
+        if (out_type == FOS_T_BF16) hipLaunchKernelGGL(gemm_reduce_kernel<true>, rgrid, dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(gemm_reduce_kernel<false>, rgrid, dim3(256), 0, s, p);
+    }
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
 // Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
 // caller's workspace for splits * M * N FP32 partials).
 enum { kPlanBig, kPlanSmall, kPlanSkinny };
@@ -703,9 +879,9 @@ static int env_int(const char *name, int fallback) {
 }
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
-    const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no skinny kernel
+    const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
     int64_t steps, tiles;
-    if (M <= 128 && K % 256 == 0 && tile == 0) {
+    if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
         g.kind = kPlanSkinny;
         steps = K / 256;
@@ -797,6 +973,13 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     switch (g.kind) {
         case kPlanBig: return launch_gemm<2, 4, 4, 2>(p, out_type, s);
         case kPlanSkinny:
+            // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
+            // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);
+            // FOS_GEMM_TILE = 16 / 32 forces / forbids it (tuning, tests)
+            if (M <= 16) {
+                const int forced = env_int("FOS_GEMM_TILE", 0);
+                if (forced == 16 || (forced != 32 && g.ksteps_per_split >= 16)) return launch_decode(p, out_type, s);
+            }
             if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
             if (M <= 64) return launch_skinny<2, 1>(p, out_type, s);
             return launch_skinny<4, 1>(p, out_type, s);

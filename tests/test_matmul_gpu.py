@@ -99,6 +99,11 @@ def test_gemm_full_size_sampled(oracle, m, n, k):
         (100, 2048, 3328, {"FOS_GEMM_SPLITK": "5"}),            # ... 13 steps, idle waves, 100 of 128 rows
         (16, 1024, 4096, {}),                                   # ... one 32-row A tile
         (48, 512, 2048, {"FOS_GEMM_SPLITK": "2"}),              # ... two
+        (5, 512, 2304, {"FOS_GEMM_SPLITK": "3", "FOS_GEMM_TILE": "16"}),  # 16-row kernel: 9 steps, 5 of 16 rows
+        (16, 256, 768, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... fewer steps than wavefronts
+        (1, 128, 6400, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... 25 steps: full prefetch rounds + a tail
+        (16, 384, 12288, {"FOS_GEMM_SPLITK": "2"}),             # ... two full rounds per wavefront (its default range)
+        (16, 384, 12288, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "32"}),  # the same shape on 32-row tiles
         (128, 512, 1088, {}),                                   # K % 128 != 0: 128 x 128 tiles
         (384, 256, 14336, {}),
     ],
