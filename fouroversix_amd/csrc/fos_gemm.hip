@@ -296,12 +296,17 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 
 // ---------------------------------------------------------------------------------------
 // M <= 128 ("skinny": decode-sized batches, one 128-row band of A).  The weight matrix B is
-// streamed once from HBM; a workgroup owns 32 * WN rows of B and the first 32 * MT rows of A,
+// streamed once from HBM; a workgroup owns 32 rows of B and the first 32 * MT rows of A,
 // and its 8 wavefronts split the K steps of 256 between them (wave w takes steps w, w + 8,
 // ...), so no data is shared between wavefronts and the main loop has no barrier.
 //
+// The 32 rows are n128 + 32 q + r0 + i (q = 0..3, i = 0..7; tile row rho = 8 q + i): the tiled
+// scale layout keeps rows r, r + 32, r + 64, r + 96 in one 16-byte unit, so the scales of
+// these rows are 128 contiguous bytes per K group, where 32 consecutive rows would use 4
+// bytes of each of 32 units.
+//
 // Per step a lane (r = lane & 31, h = lane >> 5) multiplies the 128 codes
-// k = 256 step + 128 h ... of B row n0 + 32 t + r with the same codes of A rows r + 32 i.
+// k = 256 step + 128 h ... of B tile row r with the same codes of A rows r + 32 i.
 // The MFMA contraction index is thereby permuted (slice x pairs codes 8x..8x+7 of both
 // lane halves); A and B use the same permutation, so the sum is unchanged.
 //  * A codes are re-read by every workgroup, so their path through the vector cache
@@ -314,7 +319,8 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 //    goes straight from global memory to the lane that multiplies it.
 //  * Scales: the 128x4 tiled layout puts the four blocks of a 64-wide K group of rows r,
 //    r + 32, r + 64, r + 96 next to each other, so one 128-bit load per group fetches the
-//    scales of all A rows of a lane; B takes one 32-bit word per group.
+//    scales of the A rows of a lane (fewer words for fewer row tiles); B takes one 32-bit
+//    word per group.
 // The 8 partial accumulators are tree-reduced through LDS at the end (fixed order).
 constexpr int kSkinnyRotation = 5;  // K steps between the starting points of neighbouring workgroups (odd: 8 in a row are in flight)
 constexpr int kSkinnyPitch = 144;  // LDS bytes per A row (128 + 16: conflict-free 128-bit accesses)
@@ -353,7 +359,11 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     // the wave index steers loops and scalar buffer offsets: make its uniformity known
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 31, h = lane >> 5;
     uint8_t *region = smem + wave * kRegion;
-    const int64_t n0 = (int64_t)blockIdx.x * (32 * WN);
+    // rows n128 + 32 q + r0 + i (q = 0..3, i = 0..7): their scales are whole cache lines of the
+    // tiled layout (four rows 32 apart share a 16-byte unit); tile row rho = 8 q + i
+    static_assert(WN == 1, "one 32-row tile per workgroup: the row interleave below assumes it");
+    const int64_t n128 = (int64_t)(blockIdx.x >> 2) * 128;
+    const int r0 = (int)(blockIdx.x & 3) * 8;
     const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
     const int64_t steps_all = p.K >> 8;
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
@@ -373,13 +383,13 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 
     // rows of A past M read as zero codes (buffer range check), so A needs only M rows
     const BufferRsrc ra = make_rsrc(p.A, (uint32_t)(p.M * kbytes));
-    const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(32 * WN * kbytes));
+    const BufferRsrc rb = make_rsrc(p.B + n128 * kbytes, (uint32_t)(128 * kbytes));
     const BufferRsrc rsa = make_rsrc(p.sfA, (uint32_t)(sf_groups * 512));
-    const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
+    const BufferRsrc rsb = make_rsrc(p.sfB + (n128 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
     const uint32_t a_off = (uint32_t)((lane >> 3) * kbytes + (lane & 7) * 16);  // row 8 j + lane / 8, 16-byte column lane % 8
-    const uint32_t b_off = (uint32_t)(r * kbytes + h * 64);
+    const uint32_t b_off = (uint32_t)((32 * (r >> 3) + r0 + (r & 7)) * kbytes + h * 64);
     const uint32_t sa_off = (uint32_t)(h * 1024 + r * 16);
-    const uint32_t sb_off = (uint32_t)(h * 1024 + r * 16 + (((uint32_t)n0 & 127u) >> 5) * 4);
+    const uint32_t sb_off = (uint32_t)(h * 1024 + (r0 + (r & 7)) * 16 + (r >> 3) * 4);
     const uint32_t lds_w = (uint32_t)((lane >> 3) * kSkinnyPitch + (lane & 7) * 16);
     const uint32_t lds_r = (uint32_t)(r * kSkinnyPitch + h * 64);
 
@@ -406,8 +416,8 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 s.b[t][q] = __builtin_bit_cast(
-                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (t * 32 + q * 8) * kbytes), kq, 0)
-                                    : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + t * 32 * kbytes + q * 16), kq, 0));
+                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (q * 32 + r0) * kbytes), kq, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + q * 16), kq, 0));
     };
     auto fetch_scales = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
         const bool ok = j < nsteps;
@@ -416,7 +426,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 #pragma unroll
         for (int t = 0; t < WN; ++t)
 #pragma unroll
-            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(r_b, (int)(sb_off + t * 4 + u * 512), ksf, 0);
+            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(r_b, (int)(sb_off + u * 512), ksf, 0);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
             load_words<MT>(s.sa[u], r_a, (int)(sa_off + u * 512), ksf);
@@ -571,7 +581,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
     }
     if (wave != 0) return;
 
-    // acc[i][t][4 g + e] is D[m][n], m = 32 i + r, n = n0 + 32 t + 8 g + 4 h + e; rows m >= M
+    // acc[i][t][4 g + e] is D[m][n], m = 32 i + r, n = n128 + 32 g + r0 + 4 h + e (tile row 8 g + 4 h + e); rows m >= M
     // are padding of the band and are not written
     if (OUT == kOutPartial) {
         float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
@@ -582,7 +592,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
             for (int t = 0; t < WN; ++t)
 #pragma unroll
                 for (int g = 0; g < 4; ++g)
-                    *reinterpret_cast<float4 *>(P + (int64_t)(32 * i + r) * p.N + n0 + 32 * t + 8 * g + 4 * h) =
+                    *reinterpret_cast<float4 *>(P + (int64_t)(32 * i + r) * p.N + n128 + 32 * g + r0 + 4 * h) =
                         make_float4(acc[i][t][4 * g], acc[i][t][4 * g + 1], acc[i][t][4 * g + 2], acc[i][t][4 * g + 3]);
         }
         return;
@@ -607,7 +617,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
                         o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
                     }
                 }
-                *reinterpret_cast<uint2 *>(D + (int64_t)(32 * i + r) * p.ldd + n0 + 32 * t + 8 * g + 4 * h) =
+                *reinterpret_cast<uint2 *>(D + (int64_t)(32 * i + r) * p.ldd + n128 + 32 * g + r0 + 4 * h) =
                     make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
             }
     }
@@ -619,17 +629,23 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 // built on the 16 x 16 x 32 MFMA: a 32 x 32 tile would spend half of its rows, and half of
 // the activation conversions, on padding.
 //
+// A workgroup owns the rows n128 + 32 q + r0 + i (q = 0..3, i = 0..7) of one 128-row band,
+// r0 = 8 (blockIdx.x % 4): in the tiled scale layout the four rows r, r + 32, r + 64, r + 96
+// share a 16-byte unit, so the scales of these 32 rows are 128 contiguous bytes per K group
+// -- whole cache lines, one 64-bit load per lane -- where 32 consecutive rows would use 4
+// bytes of each of 32 units.
+//
 // Lane l = (c = l & 15, g = l >> 4).  Per step it holds the 64 codes k = 256 step + 64 g ...
-// of B rows n0 + c and n0 + 16 + c and of A row c: 32 contiguous bytes each, whose four
-// blocks are exactly one scale group (one 32-bit word of the tiled layout).  MFMA slice
-// s = 0..7 multiplies 32-bit word s of every lane, i.e. the contraction index is permuted
-// (slice s pairs codes 8 s ... 8 s + 7 of all four lane groups), identically for both
-// operands.  Operands go from global memory to registers to the MFMA: no LDS in the loop.
-// acc[b][e] is D[m = c][n = n0 + 16 b + 4 g + e].
+// of B rows n128 + 32 (2 (c >> 3) + b) + r0 + (c & 7), b = 0, 1, and of A row c: 32 contiguous
+// bytes each, whose four blocks are exactly one scale group (one 32-bit word of the tiled
+// layout).  MFMA slice s = 0..7 multiplies 32-bit word s of every lane, i.e. the contraction
+// index is permuted (slice s pairs codes 8 s ... 8 s + 7 of all four lane groups), identically
+// for both operands.  Operands go from global memory to registers to the MFMA: no LDS in the
+// loop.  acc[b][e] is D[m = c][n = n128 + 32 (2 (g >> 1) + b) + r0 + 4 (g & 1) + e].
 struct DecodeRegs {
     uint4 b[2][2];   // 64 codes of two B rows
     uint4 a[2];      // 64 codes of the A row
-    uint32_t sb[2];  // their scale groups
+    uint32_t sb[2];  // their scale groups (adjacent words of one 16-byte unit)
     uint32_t sa;
 };
 
@@ -638,7 +654,8 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     constexpr int kWaves = 8, kDepth = 3;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), c = lane & 15, g = lane >> 4;
-    const int64_t n0 = (int64_t)blockIdx.x * 32;
+    const int64_t n128 = (int64_t)(blockIdx.x >> 2) * 128;
+    const int r0 = (int)(blockIdx.x & 3) * 8;
     const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
     const int64_t steps_all = p.K >> 8;
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
@@ -655,13 +672,14 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     // rows of A past M read as zero codes (buffer range check); loads past the last step go
     // through the empty descriptor, so that none of them sits under a branch
     const BufferRsrc ra = make_rsrc(p.A, (uint32_t)(p.M * kbytes));
-    const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(32 * kbytes));
+    const BufferRsrc rb = make_rsrc(p.B + n128 * kbytes, (uint32_t)(128 * kbytes));
     const BufferRsrc rsa = make_rsrc(p.sfA, (uint32_t)(sf_groups * 512));
-    const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
+    const BufferRsrc rsb = make_rsrc(p.sfB + (n128 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
     const BufferRsrc r_none = make_rsrc(p.A, 0);
-    const uint32_t q_off = (uint32_t)(c * kbytes + g * 32);
+    const uint32_t qa_off = (uint32_t)(c * kbytes + g * 32);
+    const uint32_t qb_off = (uint32_t)((64 * (c >> 3) + r0 + (c & 7)) * kbytes + g * 32);  // b = 1: 32 rows further
     const uint32_t sa_off = (uint32_t)(g * 512 + c * 16);
-    const uint32_t sb_off = (uint32_t)(g * 512 + c * 16 + (((uint32_t)n0 & 127u) >> 5) * 4);
+    const uint32_t sb_off = (uint32_t)(g * 512 + (r0 + (c & 7)) * 16 + (c >> 3) * 8);
 
     auto fetch = [&](int64_t j, DecodeRegs &s) {
         const bool ok = j < nsteps;
@@ -671,12 +689,11 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
-                s.b[b][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qb, (int)(q_off + b * 16 * kbytes + u * 16), kq, 0));
+                s.b[b][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qb, (int)(qb_off + b * 32 * kbytes + u * 16), kq, 0));
 #pragma unroll
         for (int u = 0; u < 2; ++u)
-            s.a[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qa, (int)(q_off + u * 16), kq, 0));
-#pragma unroll
-        for (int b = 0; b < 2; ++b) s.sb[b] = __builtin_amdgcn_raw_buffer_load_b32(fb, (int)(sb_off + b * 256), ksf, 0);
+            s.a[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qa, (int)(qa_off + u * 16), kq, 0));
+        load_words<2>(s.sb, fb, (int)sb_off, ksf);
         s.sa = __builtin_amdgcn_raw_buffer_load_b32(fa, (int)sa_off, ksf, 0);
     };
 
@@ -743,11 +760,12 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     }
     if (wave != 0 || c >= p.M) return;
 
+    const int64_t n_out = n128 + 64 * (g >> 1) + r0 + 4 * (g & 1);  // column of acc[0][0]; acc[1] is 32 further
     if (OUT == kOutPartial) {
         float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
 #pragma unroll
         for (int b = 0; b < 2; ++b)
-            *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n0 + 16 * b + 4 * g) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+            *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n_out + 32 * b) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
         return;
     }
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
@@ -765,7 +783,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
                 o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
             }
         }
-        *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n0 + 16 * b + 4 * g) =
+        *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n_out + 32 * b) =
             make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
     }
 }
