@@ -916,7 +916,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
         tiles = ((M + 127) / 128) * (N / 128);
     }
     // split so that about kTargetWorkgroups workgroups run, each with a useful share of K
-    const int64_t min_steps = g.kind == kPlanSkinny ? 8 : 4;
+    // (at M <= 32 a split must leave two steps per wavefront: 16 x 4096 x 4096 takes 6.4 us
+    // unsplit and 7.1 us in two halves plus their reduction)
+    const int64_t min_steps = g.kind == kPlanSkinny ? (M <= 32 ? 16 : 8) : 4;
     // (the weight-streaming kernel also splits in two when its workgroups would cover exactly
     // half of the compute units: measured 18.8 -> 15.1 us at M = 16, N = 4096, K = 14336)
     const int64_t enough = g.kind == kPlanSkinny ? kTargetWorkgroups / 2 + 1 : kTargetWorkgroups / 2;

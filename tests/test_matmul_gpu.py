@@ -97,7 +97,8 @@ def test_gemm_full_size_sampled(oracle, m, n, k):
         (128, 1024, 4096, {}),                                  # weight-streaming kernel, split 2
         (128, 4096, 4096, {"FOS_GEMM_SPLITK": "3"}),            # ... ragged last split
         (100, 2048, 3328, {"FOS_GEMM_SPLITK": "5"}),            # ... 13 steps, idle waves, 100 of 128 rows
-        (16, 1024, 4096, {}),                                   # ... one 32-row A tile
+        (16, 1024, 4096, {"FOS_GEMM_SPLITK": "2"}),             # ... one 32-row A tile (unsplit by default: 16 steps)
+        (32, 1024, 8192, {}),                                   # ... split by default
         (48, 512, 2048, {"FOS_GEMM_SPLITK": "2"}),              # ... two
         (5, 512, 2304, {"FOS_GEMM_SPLITK": "3", "FOS_GEMM_TILE": "16"}),  # 16-row kernel: 9 steps, 5 of 16 rows
         (16, 256, 768, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... fewer steps than wavefronts
