@@ -312,6 +312,21 @@ FOS_DEVICE MxRsrc mx_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
+// N consecutive 32-bit words (N = 1, 2, 4) with one buffer load.
+template <int N>
+FOS_DEVICE void mx_load_words(uint32_t (&dst)[N], MxRsrc r, int voffset, int soffset) {
+    static_assert(N == 1 || N == 2 || N == 4, "one load instruction");
+    if constexpr (N == 1) {
+        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voffset, soffset, 0);
+    } else if constexpr (N == 2) {
+        const auto v = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r, voffset, soffset, 0));
+        dst[0] = v.x, dst[1] = v.y;
+    } else {
+        const auto v = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, voffset, soffset, 0));
+        dst[0] = v.x, dst[1] = v.y, dst[2] = v.z, dst[3] = v.w;
+    }
+}
+
 FOS_DEVICE mx_v8i frag_of(const uint4 &q) {
     mx_v8i v = {(int)q.x, (int)q.y, (int)q.z, (int)q.w, 0, 0, 0, 0};  // FP4 operands use the first four registers
     return v;
@@ -381,12 +396,12 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
             s.b[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)q_off, kq + (int)(i * kRowsPerPass * kbytes), 0));
     };
     // raw scale words of step ks (bytes = the four K blocks of the chunk)
+    // (the words of a wavefront's row tiles are adjacent in the 16-byte unit of row r: one
+    // load per operand instead of one per row tile)
     auto fetch_scales = [&](int64_t ks, Scales &s) {
         const int ksf = (int)(ks * 512);
-#pragma unroll
-        for (int i = 0; i < WM; ++i) s.a[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)sa_off, ksf + i * 4, 0);
-#pragma unroll
-        for (int j = 0; j < WN; ++j) s.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)sb_off, ksf + j * 4, 0);
+        mx_load_words<WM>(s.a, rsa, (int)sa_off, ksf);
+        mx_load_words<WN>(s.b, rsb, (int)sb_off, ksf);
     };
     // half q of the staged registers -> LDS stage `buf`
     auto stage_part = [&](const Staged &s, int buf, int q) {
