@@ -540,6 +540,198 @@ static int launch_gemm_mxfp4(MxGemmParams &p, int out_type, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
+// ---------------------------------------------------------------------------------------
+// The same 256 x 256 x 128 tile with the operands loaded from global memory straight into
+// LDS (buffer_load ... lds: lane i of a wavefront fills the i-th 16-byte unit of a 1 KiB
+// run), so no registers stage them and four LDS stages keep three K steps in flight -- the
+// register-staged kernel above has one step of latency cover, and a step then lasts as long
+// as a load takes whatever the matrix pipe could do.
+//
+// A stage holds 256 rows x 64 bytes of each operand without padding and the four 512-byte
+// scale tiles of the step (fetched the same way, 4 bytes per lane); the 16-byte unit c of
+// row rho sits at unit c ^ ((rho >> 2) & 3).  A 128-bit LDS read serves 16 lanes per cycle
+// from 64 banks, i.e. the 16 rows a quarter-wave reads must differ in address bits 7:4:
+// those are 4 (rho & 3) + (c ^ ((rho >> 2) & 3)), all 16 values.  (With (rho >> 1) & 3, which
+// serves 8 lanes from 32 banks, the counters showed every fragment read taking twice as
+// long.)  The load of lane i therefore fetches unit (i & 3) ^ ((i >> 4) & 3) of row i >> 2 of
+// its 16-row run.
+constexpr int kDmaStages = 4;
+constexpr int kDmaOperandBytes = 256 * 64;
+constexpr int kDmaStageBytes = 2 * kDmaOperandBytes + 2048;  // + the step's scales: A tiles 0, 1, B tiles 0, 1
+typedef __attribute__((address_space(3))) void *MxLdsPtr;
+typedef int mx_v4i __attribute__((ext_vector_type(4)));
+
+// Buffer descriptor as four plain words (for inline assembly): base, stride 0, size in
+// bytes, raw 32-bit offsets with range checking -- the words mx_rsrc() makes.
+FOS_DEVICE mx_v4i mx_raw_rsrc(const void *base, uint32_t bytes) {
+    const uint64_t a = (uint64_t)(uintptr_t)base;
+    mx_v4i v = {(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+    return v;
+}
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maxima)
+#define MX_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+template <bool OUT_BF16>
+__global__ __launch_bounds__(512) void gemm_mxfp4_dma_kernel(const MxGemmParams p) {
+    constexpr int WAVES_N = 4, WM = 4, WN = 2, BM = 256, BN = 256;
+    extern __shared__ __attribute__((aligned(16))) uint8_t mx_lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 31, h = lane >> 5;
+    int tile_m, tile_n;
+    mx_tile_of(blockIdx.x, p.tiles_m, p.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int64_t kbytes = p.K >> 1;
+    const int64_t ksteps = p.K / kMxBK;
+
+    // The loads into LDS are written as inline assembly: the compiler orders a wait for ALL
+    // loads in flight before any LDS read that follows such a load it knows about, which would
+    // undo the pipelining.  Every global load of the loop is of this kind (the scales too), so
+    // the compiler places no vector-memory waits of its own there and the one wait per step
+    // is placed by hand in kstep().
+    const mx_v4i ra = mx_raw_rsrc(p.A + m0 * kbytes, (uint32_t)(BM * kbytes));
+    const mx_v4i rb = mx_raw_rsrc(p.B + n0 * kbytes, (uint32_t)(BN * kbytes));
+    // wavefront w loads rows 32 w ... 32 w + 31 of both operands, 16 rows per instruction
+    const int ld_row = lane >> 2;
+    const uint32_t ld_off = (uint32_t)((wave * 32 + ld_row) * kbytes + (((lane & 3) ^ ((ld_row >> 2) & 3)) * 16));
+    const int ld_half = (int)(16 * kbytes);
+    // ... and 256 of the step's 2 KiB of scales (a 512-byte tile per 128 rows and K step):
+    // waves 0-3 those of A (row tile w >> 1, half w & 1), waves 4-7 those of B
+    const uint8_t *sf_src = (wave < 4 ? p.sfA + (m0 >> 7) * ksteps * 512 : p.sfB + (n0 >> 7) * ksteps * 512) + ((wave >> 1) & 1) * ksteps * 512;
+    const mx_v4i rs = mx_raw_rsrc(sf_src, (uint32_t)(ksteps * 512));
+    const uint32_t sf_off = (uint32_t)((wave & 1) * 256 + lane * 4);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(MxLdsPtr)mx_lds;
+    auto issue = [&](int64_t ks, int stage) {
+        const int kq = (int)(ks * (kMxBK / 2)), ksf = (int)(ks * 512);
+        const uint32_t base = lds_base + (uint32_t)(stage * kDmaStageBytes);
+        const uint32_t run = base + (uint32_t)(wave * 2048), sf_run = base + (uint32_t)(2 * kDmaOperandBytes + wave * 256);
+        // m0 = LDS address of the run a wavefront fills (lane i: unit i); one wait state
+        // between a write of m0 and its use.  (m0 is reserved: the compiler never keeps a
+        // value in it across other code, it writes it right before each use of its own.)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :
+                         : "s"(run + t * 1024), "v"(ld_off), "s"(ra), "s"(kq + t * ld_half)
+                         : "memory");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :
+                         : "s"(run + kDmaOperandBytes + t * 1024), "v"(ld_off), "s"(rb), "s"(kq + t * ld_half)
+                         : "memory");
+        }
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                     :
+                     : "s"(sf_run), "v"(sf_off), "s"(rs), "s"(ksf)
+                     : "memory");
+    };
+    constexpr int kLoadsPerStep = 5;
+
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    mx_v16f acc[WM][WN];
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    const uint32_t fa_off = (uint32_t)((wm * WM * 32 + r) * 64), fb_off = (uint32_t)(kDmaOperandBytes + (wn * WN * 32 + r) * 64);
+    const int swz = (r >> 2) & 3;
+    auto read_frags = [&](int stage, int kk, uint4 *fa, uint4 *fb) {
+        const uint8_t *base = mx_lds + stage * kDmaStageBytes + (((kk * 2 + h) ^ swz) * 16);
+#pragma unroll
+        for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const uint4 *>(base + fa_off + i * 32 * 64);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const uint4 *>(base + fb_off + j * 32 * 64);
+    };
+    // scale words of this wavefront's row tiles: the 16-byte unit of row r holds those of rows
+    // r, r + 32, r + 64, r + 96 of a 128-row tile (A: all four; B: two of them)
+    const uint32_t sa_off = (uint32_t)(2 * kDmaOperandBytes + wm * 512 + r * 16);
+    const uint32_t sb_off = (uint32_t)(2 * kDmaOperandBytes + 1024 + (wn >> 1) * 512 + r * 16 + (wn & 1) * 8);
+
+    // steps 0 .. 2 in flight (past the end: the last step once more, into stages nobody reads)
+#pragma unroll
+    for (int s = 0; s < kDmaStages - 1; ++s) issue(s < ksteps ? s : ksteps - 1, s);
+
+    // One K step.  On entry the loads of step ks are the oldest in flight; behind them are
+    // those of steps ks + 1 and ks + 2.  After the barrier every wavefront has its share of
+    // step ks in LDS and has read the last fragments of step ks - 1, whose stage the loads of
+    // step ks + 3 may overwrite.  (Moving the barrier between the two slices, with the next
+    // step's first fragments read behind it, measured slower -- 341 against 320 us at 8192^3:
+    // it asks for a step's operands half a step earlier, and their arrival is what a step
+    // waits for.)
+    for (int64_t ks = 0; ks < ksteps; ++ks) {
+        const int stage = (int)(ks & (kDmaStages - 1));
+        MX_WAIT_VMCNT(2 * kLoadsPerStep);
+        __syncthreads();
+        issue(ks + 3 < ksteps ? ks + 3 : ksteps - 1, (stage + 3) & (kDmaStages - 1));
+        const uint8_t *st = mx_lds + stage * kDmaStageBytes;
+        const uint4 wa = *reinterpret_cast<const uint4 *>(st + sa_off);
+        const uint2 wb = *reinterpret_cast<const uint2 *>(st + sb_off);
+        // lanes of the upper half use the next byte: after the shift, byte 0 / byte 2 of every
+        // lane's register are the scales of the K blocks it feeds in slice 0 / slice 1
+        const uint32_t sha[WM] = {wa.x >> (8 * h), wa.y >> (8 * h), wa.z >> (8 * h), wa.w >> (8 * h)};
+        const uint32_t shb[WN] = {wb.x >> (8 * h), wb.y >> (8 * h)};
+        uint4 fa[2][WM], fb[2][WN];
+        read_frags(stage, 0, fa[0], fb[0]);
+        read_frags(stage, 1, fa[1], fb[1]);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+            for (int i = 0; i < WM; ++i)
+#pragma unroll
+                for (int j = 0; j < WN; ++j) {
+                    if (kk == 1)
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            frag_of(fb[1][j]), frag_of(fa[1][i]), acc[i][j], 4, 4, 2, (int)shb[j], 2, (int)sha[i]);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            frag_of(fb[0][j]), frag_of(fa[0][i]), acc[i][j], 4, 4, 0, (int)shb[j], 0, (int)sha[i]);
+                }
+        }
+    }
+    // loads still in flight write LDS: drain them before the workgroup gives its LDS up
+    MX_WAIT_VMCNT(0);
+
+    const float alpha = *p.alpha;
+    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+        const int64_t m = m0 + wm * WM * 32 + i * 32 + r;
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * h;
+                uint32_t w[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float2_t v = {alpha * acc[i][j][4 * g + 2 * e], alpha * acc[i][j][4 * g + 2 * e + 1]};
+                    if (OUT_BF16) {
+                        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+                    } else {
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
+                    }
+                }
+                *reinterpret_cast<uint2 *>(D + m * p.ldd + n) = make_uint2(w[0], w[1]);
+            }
+        }
+    }
+}
+
+static int launch_gemm_mxfp4_dma(MxGemmParams &p, int out_type, hipStream_t s) {
+    constexpr size_t lds_bytes = (size_t)kDmaStages * kDmaStageBytes;
+    p.tiles_m = (int)(p.M / 256);
+    p.tiles_n = (int)(p.N / 256);
+    auto kernel = out_type == FOS_T_BF16 ? gemm_mxfp4_dma_kernel<true> : gemm_mxfp4_dma_kernel<false>;
+    if (hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
+        return FOS_E_LAUNCH;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(p.tiles_m * p.tiles_n)), dim3(512), lds_bytes, s, p);
+    return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
 }  // namespace fos
 
 using namespace fos;
@@ -559,7 +751,10 @@ extern "C" int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
     bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256;
-    if (const char *e = getenv("FOS_MX_TILE")) big = big && atoi(e) != 128;  // tuning / tests
+    int forced = 0;
+    if (const char *e = getenv("FOS_MX_TILE")) forced = atoi(e);  // tuning / tests: 128 small tile, 256 register-staged big tile
+    big = big && forced != 128;
+    if (big && forced != 256) return launch_gemm_mxfp4_dma(p, out_type, s);
     if (big) return launch_gemm_mxfp4<2, 4, 4, 2>(p, out_type, s);
     return launch_gemm_mxfp4<2, 2, 2, 2>(p, out_type, s);
 }

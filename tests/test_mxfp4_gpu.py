@@ -112,3 +112,24 @@ def test_mxfp4_gemm(oracle, m, n, k, out_dtype):
     frac = float((got != expect).mean())
     rel = float(np.abs(got - expect).max() / max(np.abs(expect).max(), 1e-30))
     assert frac <= MISMATCH_BUDGET and rel <= MAX_REL, f"{frac:.2e} of outputs differ, max rel {rel:.2e}"
+
+
+@pytest.mark.parametrize("k", [128, 256, 384, 1152, 4224])
+def test_mxfp4_gemm_kernels_agree_bitwise(monkeypatch, k):
+    """The big-tile kernel that loads operands straight into LDS (four stages), the
+    register-staged big-tile kernel and the small-tile kernel contract K in the same order
+    with the same matrix instruction: whole outputs are bit-identical.  K covers fewer steps
+    than stages, a partial last round of stages, and many rounds."""
+    m = n = 4096
+    qa = fos.quantize(make_input("randn", (m, k), 21).cuda(), mx_config())
+    qb = fos.quantize(make_input("outlier", (n, k), 22).cuda(), mx_config("static_4"))
+    outs = []
+    for tile in (None, "256", "128"):
+        if tile is None:
+            monkeypatch.delenv("FOS_MX_TILE", raising=False)
+        else:
+            monkeypatch.setenv("FOS_MX_TILE", tile)
+        outs.append(fos.quantized_matmul(qa, qb))
+        torch.cuda.synchronize()
+    assert not torch.isnan(outs[0].float()).any()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
