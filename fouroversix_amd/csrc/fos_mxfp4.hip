@@ -83,7 +83,10 @@ FOS_DEVICE void quantize_octet_mxfp4(const uint4 &x, float qmax, uint32_t &codes
 // the tile per load instruction (512 elements = 1 KiB), four rows per step; 8 wavefronts,
 // four steps of 32 rows; the four complete 128x4 scale tiles are staged in LDS and leave as
 // one contiguous 2 KiB run.
+// FULL: the tensor is whole tiles and 16-byte aligned, so every load is an unconditional
+// 128-bit load (loads under a branch make the compiler wait for all of them at once).
 constexpr int kMxQuantThreads = 512;
+template <bool FULL>
 __global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const MxQuantParams p) {
     __shared__ uint32_t sf_stage[4 * 128];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -92,12 +95,12 @@ __global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const M
     const int64_t tile_y = blockIdx.x / p.tiles_x, tile_x = blockIdx.x - tile_y * p.tiles_x;
     const int64_t cb = tile_x * 16 + lb;
     const int64_t c0 = tile_x * 512 + lane * 8;  // first column of this lane's 8 elements
-    const bool col_ok = cb < sf_cols;
+    const bool col_ok = FULL || cb < sf_cols;
     const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
     if (blockIdx.x == 0 && threadIdx.x == 0) *p.amax = 1.0f;  // the reference reports amax = 1 (reference.py:573-578)
 
     auto load = [&](int64_t r, uint4 &v) {
-        if (r < p.rows && c0 + 8 <= p.cols && p.vector_loads) {
+        if (FULL || (r < p.rows && c0 + 8 <= p.cols && p.vector_loads)) {
             v = *reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
         } else {
             uint32_t w[4];
@@ -144,7 +147,7 @@ __global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const M
         __syncthreads();
         const int t = threadIdx.x >> 6;  // wavefronts 0-3: one scale tile each, 512 bytes, 8 per lane
         const int64_t group = tile_x * 4 + t;
-        if (t < 4 && group < (sf_cols >> 2)) {
+        if (t < 4 && (FULL || group < (sf_cols >> 2))) {
             uint2 *out = reinterpret_cast<uint2 *>(p.sf + (tile_y * (sf_cols >> 2) + group) * 512);
             out[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
         }
@@ -166,7 +169,10 @@ int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld,
     const int64_t grid = (p.rows_p / 128) * p.tiles_x;
     if (grid > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     p.amax = amax;
-    hipLaunchKernelGGL(quantize_mxfp4_kernel, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
+    if (p.vector_loads && rows % 128 == 0 && cols % 512 == 0)
+        hipLaunchKernelGGL(quantize_mxfp4_kernel<true>, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(quantize_mxfp4_kernel<false>, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
