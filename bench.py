@@ -128,6 +128,32 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
     }
 
 
+def c_abi_gemm(qa, qb, m: int, dev):
+    """A closure that calls fos_gemm_nvfp4 on two quantized operands (first m rows of A)."""
+    import torch
+
+    import fouroversix_amd as fos
+    from fouroversix_amd import _native as nat
+
+    lib = nat.lib()
+    n, k = qb.values.shape[0], qa.values.shape[1] * 2
+    alpha = fos.matmul.frontend.gemm_alpha(qa, qb).reshape(1).float().to(dev)
+    ws_bytes = int(lib.fos_gemm_workspace_bytes(m, n, k))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    out = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    args = (qa.values.data_ptr(), qb.values.data_ptr(), qa.scale_factors.data_ptr(), qb.scale_factors.data_ptr(),
+            alpha.data_ptr(), m, n, k, out.data_ptr(), nat.T_BF16, n, ws.data_ptr() if ws_bytes else None, ws_bytes,
+            nat.current_stream(dev))
+    keep = (alpha, ws, out)
+
+    def call(_keep=keep):
+        rc = lib.fos_gemm_nvfp4(*args)
+        if rc != 0:
+            raise RuntimeError(f"fos_gemm_nvfp4 returned {rc}")
+
+    return call
+
+
 def extras(dev, steps: int) -> dict:
     """Timings of the rows built around the headline path (whole calls through the public
     API, microseconds): small-M GEMMs, fused pseudo-quantize, dequantize, the transpose /
@@ -166,6 +192,10 @@ def extras(dev, steps: int) -> dict:
         qa = fos.quantize(make_activation(m, k, 7).to(dev), mse)
         qb = fos.quantize(make_activation(nn, k, 8).to(dev), mse)
         out[f"gemm_nvfp4_{m}x{nn}x{k}_us"] = us(lambda: fos.quantized_matmul(qa, qb))
+        if m <= 128:
+            # the same GEMM through the C entry point alone (output and workspace allocated once):
+            # at these sizes the Python frontend costs more than the kernels
+            out[f"gemm_nvfp4_{m}x{nn}x{k}_c_abi_us"] = us(c_abi_gemm(qa, qb, m, dev))
     mx = fos.QuantizationConfig(dtype="mxfp4", scale_rule="static_6")
     qa = fos.quantize(make_activation(8192, 8192, 5).to(dev), mx)
     qb = fos.quantize(make_activation(8192, 8192, 6).to(dev), mx)
