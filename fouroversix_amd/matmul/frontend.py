@@ -50,6 +50,19 @@ def _dequantize_form_applies(input: QuantizedTensor, other: QuantizedTensor, out
     )
 
 
+_UNIT_ALPHA: dict = {}
+
+
+def _unit_alpha(device: torch.device) -> torch.Tensor:
+    """A device f32[1] holding 1.0, made once per device (never written afterwards)."""
+    if torch.compiler.is_compiling():
+        return torch.ones(1, dtype=torch.float32, device=device)
+    one = _UNIT_ALPHA.get(device)
+    if one is None:
+        one = _UNIT_ALPHA[device] = torch.ones(1, dtype=torch.float32, device=device)
+    return one
+
+
 def gemm_alpha(input: QuantizedTensor, other: QuantizedTensor) -> torch.Tensor:
     """``(amaxA * amaxB) / (qA sA qB sB adjA adjB)`` as a device f32[1] (reference
     matmul/cutlass/backend.py:86-98); one small kernel when both maxima are f32 GPU tensors."""
@@ -100,7 +113,7 @@ def quantized_matmul(
     out_shape = (input.original_shape[0], other.original_shape[0])
     if input.dtype == DataType.mxfp4:
         # no tensor scale: alpha = 1 (src/fouroversix/matmul/cutlass/backend.py:79-85)
-        alpha = torch.ones(1, dtype=torch.float32, device=input.values.device)
+        alpha = _unit_alpha(input.values.device)
         out = ops.gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(
             input.values, other.values, input.scale_factors, other.scale_factors, alpha,
             torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16,
