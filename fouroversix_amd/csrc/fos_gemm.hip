@@ -642,20 +642,25 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 // index is permuted (slice s pairs codes 8 s ... 8 s + 7 of all four lane groups), identically
 // for both operands.  Operands go from global memory to registers to the MFMA: no LDS in the
 // loop.  acc[b][e] is D[m = c][n = n128 + 32 (2 (g >> 1) + b) + r0 + 4 (g & 1) + e].
+//
+// NB = 1 halves the workgroup to 16 rows (n128 + 32 q + r0 + i, i = 0..3, r0 = 4 (blockIdx.x % 8);
+// lane row c: q = c >> 2, i = c & 3): twice the workgroups for narrow outputs (N <= 4096), which
+// would otherwise split K and pay a reduction kernel.  acc[0][e] is then D[c][n128 + 32 g + r0 + e].
+template <int NB>
 struct DecodeRegs {
-    uint4 b[2][2];   // 64 codes of two B rows
-    uint4 a[2];      // 64 codes of the A row
-    uint32_t sb[2];  // their scale groups (adjacent words of one 16-byte unit)
+    uint4 b[NB][2];   // 64 codes of NB rows of B
+    uint4 a[2];       // 64 codes of the A row
+    uint32_t sb[NB];  // their scale groups (NB = 2: adjacent words of one 16-byte unit)
     uint32_t sa;
 };
 
-template <int OUT>
+template <int NB, int OUT>
 __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams p) {
     constexpr int kWaves = 8, kDepth = 3;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), c = lane & 15, g = lane >> 4;
-    const int64_t n128 = (int64_t)(blockIdx.x >> 2) * 128;
-    const int r0 = (int)(blockIdx.x & 3) * 8;
+    const int64_t n128 = (int64_t)(blockIdx.x >> (NB == 2 ? 2 : 3)) * 128;
+    const int r0 = NB == 2 ? (int)(blockIdx.x & 3) * 8 : (int)(blockIdx.x & 7) * 4;
     const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
     const int64_t steps_all = p.K >> 8;
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
@@ -677,39 +682,43 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     const BufferRsrc rsb = make_rsrc(p.sfB + (n128 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
     const BufferRsrc r_none = make_rsrc(p.A, 0);
     const uint32_t qa_off = (uint32_t)(c * kbytes + g * 32);
-    const uint32_t qb_off = (uint32_t)((64 * (c >> 3) + r0 + (c & 7)) * kbytes + g * 32);  // b = 1: 32 rows further
+    const uint32_t qb_off = NB == 2 ? (uint32_t)((64 * (c >> 3) + r0 + (c & 7)) * kbytes + g * 32)  // b = 1: 32 rows further
+                                    : (uint32_t)((32 * (c >> 2) + r0 + (c & 3)) * kbytes + g * 32);
     const uint32_t sa_off = (uint32_t)(g * 512 + c * 16);
-    const uint32_t sb_off = (uint32_t)(g * 512 + (r0 + (c & 7)) * 16 + (c >> 3) * 8);
+    const uint32_t sb_off = NB == 2 ? (uint32_t)(g * 512 + (r0 + (c & 7)) * 16 + (c >> 3) * 8)
+                                    : (uint32_t)(g * 512 + (r0 + (c & 3)) * 16 + (c >> 2) * 4);
 
-    auto fetch = [&](int64_t j, DecodeRegs &s) {
+    auto fetch = [&](int64_t j, DecodeRegs<NB> &s) {
         const bool ok = j < nsteps;
         const BufferRsrc qa = ok ? ra : r_none, qb = ok ? rb : r_none, fa = ok ? rsa : r_none, fb = ok ? rsb : r_none;
         const int kq = ok ? (int)(phys(j) * 128) : 0, ksf = ok ? (int)(phys(j) * 2048) : 0;
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 s.b[b][u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qb, (int)(qb_off + b * 32 * kbytes + u * 16), kq, 0));
 #pragma unroll
         for (int u = 0; u < 2; ++u)
             s.a[u] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(qa, (int)(qa_off + u * 16), kq, 0));
-        load_words<2>(s.sb, fb, (int)sb_off, ksf);
+        load_words<NB>(s.sb, fb, (int)sb_off, ksf);
         s.sa = __builtin_amdgcn_raw_buffer_load_b32(fa, (int)sa_off, ksf, 0);
     };
 
-    float4_t acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+    float4_t acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     auto word_of = [](const uint4 &v, int j) -> uint32_t { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; };
     // scale of code word x (0..7) of a lane: block x >> 1 = byte x >> 1 of the group word
     auto scale_of = [](uint32_t w, int x) -> half2_t {
         const half2_t s2 = e4m3x2_to_half2((x & 4) ? w >> 16 : w);
         return ((x >> 1) & 1) ? __builtin_shufflevector(s2, s2, 1, 1) : __builtin_shufflevector(s2, s2, 0, 0);
     };
-    auto compute = [&](const DecodeRegs &s) {
+    auto compute = [&](const DecodeRegs<NB> &s) {
 #pragma unroll
         for (int x = 0; x < 8; ++x) {
             const half8_t fa = dequant8(word_of(s.a[x >> 2], x & 3), scale_of(s.sa, x));
 #pragma unroll
-            for (int b = 0; b < 2; ++b) {
+            for (int b = 0; b < NB; ++b) {
                 const half8_t fb = dequant8(word_of(s.b[b][x >> 2], x & 3), scale_of(s.sb[b], x));
                 acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, fa, acc[b], 0, 0, 0);
             }
@@ -719,7 +728,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     // read now, used in the epilogue: short launches would otherwise end on this latency
     const float alpha = OUT == kOutPartial ? 0.0f : load_alpha(p);
 
-    DecodeRegs st[kDepth];
+    DecodeRegs<NB> st[kDepth];
     int64_t step = wave;  // counts this workgroup's steps, see phys()
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) fetch(step + d * kWaves, st[d]);
@@ -742,17 +751,17 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
 #pragma unroll
     for (int stride = kWaves / 2; stride >= 1; stride >>= 1) {
         if (wave >= stride && wave < 2 * stride) {
-            float *slot = red + (wave - stride) * (8 * 64);
+            float *slot = red + (wave - stride) * (4 * NB * 64);
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) slot[(b * 4 + e) * 64 + lane] = acc[b][e];
         }
         __syncthreads();
         if (wave < stride) {
-            const float *slot = red + wave * (8 * 64);
+            const float *slot = red + wave * (4 * NB * 64);
 #pragma unroll
-            for (int b = 0; b < 2; ++b)
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[b][e] += slot[(b * 4 + e) * 64 + lane];
         }
@@ -760,17 +769,18 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
     }
     if (wave != 0 || c >= p.M) return;
 
-    const int64_t n_out = n128 + 64 * (g >> 1) + r0 + 4 * (g & 1);  // column of acc[0][0]; acc[1] is 32 further
+    const int64_t n_out = NB == 2 ? n128 + 64 * (g >> 1) + r0 + 4 * (g & 1)  // column of acc[0][0]; acc[1] is 32 further
+                                  : n128 + 32 * g + r0;
     if (OUT == kOutPartial) {
         float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < NB; ++b)
             *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n_out + 32 * b) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
         return;
     }
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
+    for (int b = 0; b < NB; ++b) {
         uint16_t o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -868,11 +878,12 @@ static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
 
+template <int NB>
 static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
-    constexpr size_t lds_bytes = (size_t)4 * 8 * 64 * sizeof(float);
-    dim3 grid((unsigned)(p.N / 32), (unsigned)p.splits);
-    auto kernel = p.splits > 1 ? gemm_nvfp4_decode_kernel<kOutPartial>
-                  : out_type == FOS_T_BF16 ? gemm_nvfp4_decode_kernel<kOutBF16> : gemm_nvfp4_decode_kernel<kOutF16>;
+    constexpr size_t lds_bytes = (size_t)4 * (4 * NB) * 64 * sizeof(float);
+    dim3 grid((unsigned)(p.N / (16 * NB)), (unsigned)p.splits);
+    auto kernel = p.splits > 1 ? gemm_nvfp4_decode_kernel<NB, kOutPartial>
+                  : out_type == FOS_T_BF16 ? gemm_nvfp4_decode_kernel<NB, kOutBF16> : gemm_nvfp4_decode_kernel<NB, kOutF16>;
     hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
     if (hipGetLastError() != hipSuccess) return FOS_E_LAUNCH;
     if (p.splits > 1) {
@@ -889,6 +900,7 @@ static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
 enum { kPlanBig, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
+    int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
 };
 constexpr int kTargetWorkgroups = 256;
 static int env_int(const char *name, int fallback) {
@@ -897,6 +909,7 @@ static int env_int(const char *name, int fallback) {
 }
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
+    g.narrow = 0;
     const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
     int64_t steps, tiles;
     if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32)) {
@@ -904,6 +917,12 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
         g.kind = kPlanSkinny;
         steps = K / 256;
         tiles = N / 32;
+        if (M <= 16 && tiles <= kTargetWorkgroups / 2 && (tile == 16 || (tile == 0 && steps >= 16))) {
+            // narrow outputs on the 16-row kernel: 16 rows of B per workgroup give twice the
+            // workgroups, instead of a split of K and its reduction kernel
+            g.narrow = 1;
+            tiles = N / 16;
+        }
     } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
         g.kind = kPlanBig;
@@ -998,7 +1017,8 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
             // FOS_GEMM_TILE = 16 / 32 forces / forbids it (tuning, tests)
             if (M <= 16) {
                 const int forced = env_int("FOS_GEMM_TILE", 0);
-                if (forced == 16 || (forced != 32 && g.ksteps_per_split >= 16)) return launch_decode(p, out_type, s);
+                if (forced == 16 || (forced != 32 && g.ksteps_per_split >= 16))
+                    return g.narrow ? launch_decode<1>(p, out_type, s) : launch_decode<2>(p, out_type, s);
             }
             if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
             if (M <= 64) return launch_skinny<2, 1>(p, out_type, s);

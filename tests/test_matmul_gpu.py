@@ -100,10 +100,12 @@ def test_gemm_full_size_sampled(oracle, m, n, k):
         (16, 1024, 4096, {"FOS_GEMM_SPLITK": "2"}),             # ... one 32-row A tile (unsplit by default: 16 steps)
         (32, 1024, 8192, {}),                                   # ... split by default
         (48, 512, 2048, {"FOS_GEMM_SPLITK": "2"}),              # ... two
-        (5, 512, 2304, {"FOS_GEMM_SPLITK": "3", "FOS_GEMM_TILE": "16"}),  # 16-row kernel: 9 steps, 5 of 16 rows
+        (5, 512, 2304, {"FOS_GEMM_SPLITK": "3", "FOS_GEMM_TILE": "16"}),  # 16-row kernel (16 rows of B per workgroup up to N = 4096): 9 steps, 5 of 16 rows
         (16, 256, 768, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... fewer steps than wavefronts
         (1, 128, 6400, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... 25 steps: full prefetch rounds + a tail
         (16, 384, 12288, {"FOS_GEMM_SPLITK": "2"}),             # ... two full rounds per wavefront (its default range)
+        (16, 4224, 4096, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "16"}),  # ... 32 rows of B per workgroup (N > 4096)
+        (9, 8192, 8192, {"FOS_GEMM_SPLITK": "2"}),              # ... the same by default
         (16, 384, 12288, {"FOS_GEMM_SPLITK": "2", "FOS_GEMM_TILE": "32"}),  # the same shape on 32-row tiles
         (128, 512, 1088, {}),                                   # K % 128 != 0: 128 x 128 tiles
         (384, 256, 14336, {}),
