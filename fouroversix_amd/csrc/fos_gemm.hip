@@ -347,23 +347,28 @@ struct SkinnyRegs {
     uint32_t sa[2][MT]; // block scales of the A rows: [group][i] = row r + 32 i
 };
 
+// Wavefronts of a workgroup: 8 with one 32-row tile of B each; 4 with two (WN = 2), which then
+// have a SIMD and its 512 registers to themselves (128 of them accumulators).
+constexpr int skinny_waves(int WN) { return WN == 2 ? 4 : 8; }
+
 template <int MT, int WN, int OUT>
-__global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
-    constexpr int kWaves = 8, kAcc = MT * WN * 16;
+__global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
+    constexpr int kWaves = skinny_waves(WN), kAcc = MT * WN * 16;
     // B through LDS as well (whole cache lines per load instruction, see above) where the
     // second staging region fits next to A's
-    constexpr bool kBViaLds = MT <= 2;
+    constexpr bool kBViaLds = MT <= 2 || WN == 2;
     constexpr int kRegionA = MT * 32 * kSkinnyPitch;
     constexpr int kRegion = kRegionA + (kBViaLds ? WN * 32 * kSkinnyPitch : 0);
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // the wave index steers loops and scalar buffer offsets: make its uniformity known
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), r = lane & 31, h = lane >> 5;
     uint8_t *region = smem + wave * kRegion;
-    // rows n128 + 32 q + r0 + i (q = 0..3, i = 0..7): their scales are whole cache lines of the
-    // tiled layout (four rows 32 apart share a 16-byte unit); tile row rho = 8 q + i
-    static_assert(WN == 1, "one 32-row tile per workgroup: the row interleave below assumes it");
-    const int64_t n128 = (int64_t)(blockIdx.x >> 2) * 128;
-    const int r0 = (int)(blockIdx.x & 3) * 8;
+    // tile t holds rows n128 + 32 q + r0 + 8 t + i (q = 0..3, i = 0..7): their scales are whole
+    // cache lines of the tiled layout (four rows 32 apart share a 16-byte unit); tile row rho = 8 q + i
+    static_assert(WN == 1 || WN == 2, "32 or 64 of the 128 rows of a band per workgroup");
+    constexpr int kPerBand = 4 / WN;
+    const int64_t n128 = (int64_t)(blockIdx.x / kPerBand) * 128;
+    const int r0 = (int)(blockIdx.x % kPerBand) * 8 * WN;
     const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
     const int64_t steps_all = p.K >> 8;
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
@@ -416,8 +421,8 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 #pragma unroll
             for (int q = 0; q < 4; ++q)
                 s.b[t][q] = __builtin_bit_cast(
-                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (q * 32 + r0) * kbytes), kq, 0)
-                                    : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + q * 16), kq, 0));
+                    uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (q * 32 + r0 + 8 * t) * kbytes), kq, 0)
+                                    : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + 8 * t * kbytes + q * 16), kq, 0));
     };
     auto fetch_scales = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
         const bool ok = j < nsteps;
@@ -426,7 +431,7 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
 #pragma unroll
         for (int t = 0; t < WN; ++t)
 #pragma unroll
-            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(r_b, (int)(sb_off + u * 512), ksf, 0);
+            for (int u = 0; u < 2; ++u) s.sb[t][u] = __builtin_amdgcn_raw_buffer_load_b32(r_b, (int)(sb_off + t * 128 + u * 512), ksf, 0);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
             load_words<MT>(s.sa[u], r_a, (int)(sa_off + u * 512), ksf);
@@ -551,75 +556,76 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_skinny_kernel(const GemmParams
         }
     }
 
-    // tree reduction of the 8 wavefronts' accumulators: waves [stride, 2 stride) hand theirs
-    // to waves [0, stride) through LDS slot (wave - stride); fixed order, hence deterministic.
-    // The slots overlay the staging regions, so every wavefront must have left the main loop.
+    // Reduction of the wavefronts' accumulators, scattered: every wavefront writes all of its
+    // registers to its LDS slot, then wavefront w sums registers [w R, (w + 1) R) of all slots in
+    // slot order (fixed, hence deterministic) and stores that share of the output, so the
+    // conversion and the stores are spread over the workgroup as well.  Register f = (i WN + t) 16 + e
+    // of a lane sits at float (slot (kAcc / 4) + f / 4) 256 + 4 lane + f % 4: 128-bit accesses,
+    // consecutive lanes 16 bytes apart.  The slots overlay the staging regions, so every wavefront
+    // must have left the main loop.
+    constexpr int R = kAcc / kWaves;  // 2 (MT = 1), 4, 8, 16 or 32
+    static_assert(R == 2 || R % 4 == 0, "whole groups of four columns, or half of one");
     __syncthreads();
     float *red = reinterpret_cast<float *>(smem);
 #pragma unroll
-    for (int stride = kWaves / 2; stride >= 1; stride >>= 1) {
-        if (wave >= stride && wave < 2 * stride) {
-            float *slot = red + (wave - stride) * (kAcc * 64);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int t = 0; t < WN; ++t)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) slot[((i * WN + t) * 16 + e) * 64 + lane] = acc[i][t][e];
-        }
-        __syncthreads();
-        if (wave < stride) {
-            const float *slot = red + wave * (kAcc * 64);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int t = 0; t < WN; ++t)
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) acc[i][t][e] += slot[((i * WN + t) * 16 + e) * 64 + lane];
-        }
-        __syncthreads();
-    }
-    if (wave != 0) return;
-
-    // acc[i][t][4 g + e] is D[m][n], m = 32 i + r, n = n128 + 32 g + r0 + 4 h + e (tile row 8 g + 4 h + e); rows m >= M
-    // are padding of the band and are not written
-    if (OUT == kOutPartial) {
-        float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            if (32 * i + r >= p.M) continue;
-#pragma unroll
-            for (int t = 0; t < WN; ++t)
-#pragma unroll
-                for (int g = 0; g < 4; ++g)
-                    *reinterpret_cast<float4 *>(P + (int64_t)(32 * i + r) * p.N + n128 + 32 * g + r0 + 4 * h) =
-                        make_float4(acc[i][t][4 * g], acc[i][t][4 * g + 1], acc[i][t][4 * g + 2], acc[i][t][4 * g + 3]);
-        }
-        return;
-    }
-    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        if (32 * i + r >= p.M) continue;
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int t = 0; t < WN; ++t)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint16_t o[4];
+            for (int g = 0; g < 4; ++g)
+                *reinterpret_cast<float4 *>(red + ((wave * (kAcc / 4) + (i * WN + t) * 4 + g) * 64 + lane) * 4) =
+                    make_float4(acc[i][t][4 * g], acc[i][t][4 * g + 1], acc[i][t][4 * g + 2], acc[i][t][4 * g + 3]);
+    __syncthreads();
+    float mine[R];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float v = alpha * acc[i][t][4 * g + e];
-                    if (OUT == kOutBF16) {
-                        uint32_t u = f2u(v);
-                        u += 0x7fffu + ((u >> 16) & 1u);
-                        o[e] = (uint16_t)(u >> 16);
-                    } else {
-                        o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
-                    }
-                }
-                *reinterpret_cast<uint2 *>(D + (int64_t)(32 * i + r) * p.ldd + n128 + 32 * g + r0 + 4 * h) =
-                    make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+    for (int k = 0; k < R; ++k) mine[k] = 0.0f;
+#pragma unroll
+    for (int v = 0; v < kWaves; ++v) {
+        const float *slot = red + (v * (kAcc / 4) * 64 + lane) * 4 + (R == 2 ? (wave >> 1) * 256 + (wave & 1) * 2 : wave * (R / 4) * 256);
+        if constexpr (R == 2) {
+            const float2 x = *reinterpret_cast<const float2 *>(slot);
+            mine[0] += x.x, mine[1] += x.y;
+        } else {
+#pragma unroll
+            for (int c = 0; c < R / 4; ++c) {
+                const float4 x = *reinterpret_cast<const float4 *>(slot + c * 256);
+                mine[4 * c] += x.x, mine[4 * c + 1] += x.y, mine[4 * c + 2] += x.z, mine[4 * c + 3] += x.w;
             }
+        }
+    }
+
+    // Register f is D[m][n], m = 32 i + r, n = n128 + 32 g + r0 + 8 t + 4 h + e % 4 (tile row 8 g + 4 h + e % 4),
+    // g = (f % 16) / 4; rows m >= M are padding of the band and are not written.  This wavefront's
+    // registers are groups of four columns c4 = w R / 4 ... (or, for R = 2, half of group w / 2).
+    constexpr int kGroups = R == 2 ? 1 : R / 4;
+    float *P = OUT == kOutPartial ? p.partials + (int64_t)blockIdx.y * p.M * p.N : nullptr;
+    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+    auto to16 = [&](float v) -> uint32_t {
+        v *= alpha;
+        if (OUT == kOutBF16) {
+            uint32_t u = f2u(v);
+            u += 0x7fffu + ((u >> 16) & 1u);
+            return u >> 16;
+        }
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
+    };
+#pragma unroll
+    for (int c = 0; c < kGroups; ++c) {
+        const int c4 = R == 2 ? (wave >> 1) : wave * (R / 4) + c;  // group of four columns: c4 = (i WN + t) 4 + g
+        const int g = c4 & 3, t = (c4 >> 2) % WN, i = (c4 >> 2) / WN;
+        const int m = 32 * i + r;
+        if (m >= p.M) continue;
+        const int64_t n = n128 + 32 * g + r0 + 8 * t + 4 * h + (R == 2 ? (wave & 1) * 2 : 0);
+        if constexpr (R == 2) {
+            if (OUT == kOutPartial) *reinterpret_cast<float2 *>(P + (int64_t)m * p.N + n) = make_float2(mine[0], mine[1]);
+            else *reinterpret_cast<uint32_t *>(D + (int64_t)m * p.ldd + n) = to16(mine[0]) | (to16(mine[1]) << 16);
+        } else {
+            if (OUT == kOutPartial)
+                *reinterpret_cast<float4 *>(P + (int64_t)m * p.N + n) = make_float4(mine[4 * c], mine[4 * c + 1], mine[4 * c + 2], mine[4 * c + 3]);
+            else
+                *reinterpret_cast<uint2 *>(D + (int64_t)m * p.ldd + n) =
+                    make_uint2(to16(mine[4 * c]) | (to16(mine[4 * c + 1]) << 16), to16(mine[4 * c + 2]) | (to16(mine[4 * c + 3]) << 16));
+        }
     }
 }
 
@@ -859,7 +865,9 @@ static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
 
 template <int MT, int WN>
 static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
-    constexpr size_t stage_bytes = (size_t)8 * (MT * 32 + (MT <= 2 ? WN * 32 : 0)) * kSkinnyPitch, red_bytes = (size_t)4 * (MT * WN * 16) * 64 * sizeof(float);
+    constexpr int kWaves = skinny_waves(WN);
+    constexpr size_t stage_bytes = (size_t)kWaves * (MT * 32 + (MT <= 2 || WN == 2 ? WN * 32 : 0)) * kSkinnyPitch,
+                     red_bytes = (size_t)kWaves * (MT * WN * 16) * 64 * sizeof(float);
     constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
     dim3 grid((unsigned)(p.N / (32 * WN)), (unsigned)p.splits);
     auto kernel = p.splits > 1 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutPartial>
@@ -867,7 +875,7 @@ static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
     if (lds_bytes > 64 * 1024 &&
         hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes) != hipSuccess)
         return FOS_E_LAUNCH;
-    hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * kWaves), lds_bytes, s, p);
     if (hipGetLastError() != hipSuccess) return FOS_E_LAUNCH;
     if (p.splits > 1) {
         const int64_t quads = p.M * (p.N >> 2);
@@ -901,6 +909,7 @@ enum { kPlanBig, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
+    int wide;    // M > 32: workgroups of 64 rows of B, four wavefronts with two tiles each
 };
 constexpr int kTargetWorkgroups = 256;
 static int env_int(const char *name, int fallback) {
@@ -909,10 +918,10 @@ static int env_int(const char *name, int fallback) {
 }
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
-    g.narrow = 0;
+    g.narrow = g.wide = 0;
     const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
     int64_t steps, tiles;
-    if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32)) {
+    if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32 || tile == 64)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
         g.kind = kPlanSkinny;
         steps = K / 256;
@@ -922,6 +931,10 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
             // workgroups, instead of a split of K and its reduction kernel
             g.narrow = 1;
             tiles = N / 16;
+        }
+        if (M > 32 && tile == 64) {
+            g.wide = 1;
+            tiles = N / 64;
         }
     } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
@@ -1021,8 +1034,8 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
                     return g.narrow ? launch_decode<1>(p, out_type, s) : launch_decode<2>(p, out_type, s);
             }
             if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
-            if (M <= 64) return launch_skinny<2, 1>(p, out_type, s);
-            return launch_skinny<4, 1>(p, out_type, s);
+            if (M <= 64) return g.wide ? launch_skinny<2, 2>(p, out_type, s) : launch_skinny<2, 1>(p, out_type, s);
+            return g.wide ? launch_skinny<4, 2>(p, out_type, s) : launch_skinny<4, 1>(p, out_type, s);
         default: return launch_gemm<2, 2, 2, 2>(p, out_type, s);
     }
 }
