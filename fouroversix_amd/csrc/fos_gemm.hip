@@ -342,17 +342,16 @@ FOS_DEVICE void load_words(uint32_t (&dst)[N], BufferRsrc r, int voffset, int so
 
 template <int MT, int WN>
 struct SkinnyRegs {
-    uint4 b[WN][4];     // 128 codes of each B row
-    uint32_t sb[WN][2]; // their 8 block scales (two groups)
+    uint32_t sb[WN][2]; // the 8 block scales of each B row (two groups)
     uint32_t sa[2][MT]; // block scales of the A rows: [group][i] = row r + 32 i
 };
 
-// Wavefronts of a workgroup: 8 with one 32-row tile of B each; 4 with two (WN = 2), which then
-// have a SIMD and its 512 registers to themselves (128 of them accumulators).
+// Wavefronts of a workgroup: 8 with one 32-row tile of B each; 4 with two (WN = 2), and then two
+// workgroups per compute unit.
 constexpr int skinny_waves(int WN) { return WN == 2 ? 4 : 8; }
 
 template <int MT, int WN, int OUT>
-__global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
+__global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1) void gemm_nvfp4_skinny_kernel(const GemmParams p) {
     constexpr int kWaves = skinny_waves(WN), kAcc = MT * WN * 16;
     // B through LDS as well (whole cache lines per load instruction, see above) where the
     // second staging region fits next to A's
@@ -365,10 +364,12 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
     uint8_t *region = smem + wave * kRegion;
     // tile t holds rows n128 + 32 q + r0 + 8 t + i (q = 0..3, i = 0..7): their scales are whole
     // cache lines of the tiled layout (four rows 32 apart share a 16-byte unit); tile row rho = 8 q + i
-    static_assert(WN == 1 || WN == 2, "32 or 64 of the 128 rows of a band per workgroup");
+    static_assert(WN == 1 || (WN == 2 && MT <= 2), "32 or 64 of the 128 rows of a band per workgroup");
     constexpr int kPerBand = 4 / WN;
     const int64_t n128 = (int64_t)(blockIdx.x / kPerBand) * 128;
     const int r0 = (int)(blockIdx.x % kPerBand) * 8 * WN;
+    // a launch with gridDim.z > 1 gives every 32 MT rows of A workgroups of their own
+    const int m_base = (int)blockIdx.z * 32 * MT;
     const int64_t kbytes = p.K >> 1, sf_groups = p.K >> 6;
     const int64_t steps_all = p.K >> 8;
     const int64_t s_begin = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
@@ -392,8 +393,9 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
     const BufferRsrc rsa = make_rsrc(p.sfA, (uint32_t)(sf_groups * 512));
     const BufferRsrc rsb = make_rsrc(p.sfB + (n128 >> 7) * sf_groups * 512, (uint32_t)(sf_groups * 512));
     const uint32_t a_off = (uint32_t)((lane >> 3) * kbytes + (lane & 7) * 16);  // row 8 j + lane / 8, 16-byte column lane % 8
+    const uint32_t a_row0 = (uint32_t)(m_base * kbytes);
     const uint32_t b_off = (uint32_t)((32 * (r >> 3) + r0 + (r & 7)) * kbytes + h * 64);
-    const uint32_t sa_off = (uint32_t)(h * 1024 + r * 16);
+    const uint32_t sa_off = (uint32_t)(h * 1024 + r * 16 + (m_base >> 5) * 4);
     const uint32_t sb_off = (uint32_t)(h * 1024 + (r0 + (r & 7)) * 16 + (r >> 3) * 4);
     const uint32_t lds_w = (uint32_t)((lane >> 3) * kSkinnyPitch + (lane & 7) * 16);
     const uint32_t lds_r = (uint32_t)(r * kSkinnyPitch + h * 64);
@@ -410,9 +412,13 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
         const int kq = ok ? (int)(phys(j) * 128) : 0;
 #pragma unroll
         for (int i = 0; i < MT * 4; ++i)
-            a_stage[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + i * 8 * kbytes), kq, 0));
+            a_stage[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_row0 + a_off + i * 8 * kbytes), kq, 0));
     };
-    auto fetch_b_codes = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
+    // 128 codes of each B row; two register sets (loaded two steps ahead), one with two tiles
+    constexpr int kBSets = WN == 2 ? 1 : 2;
+    typedef uint4 BCodes[WN][4];
+    BCodes bst[kBSets];
+    auto fetch_b_codes = [&](int64_t j, BCodes &b) {
         const bool ok = j < nsteps;
         const BufferRsrc r = ok ? rb : r_none;
         const int kq = ok ? (int)(phys(j) * 128) : 0;
@@ -420,7 +426,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
         for (int t = 0; t < WN; ++t)
 #pragma unroll
             for (int q = 0; q < 4; ++q)
-                s.b[t][q] = __builtin_bit_cast(
+                b[t][q] = __builtin_bit_cast(
                     uint4, kBViaLds ? __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_off + (q * 32 + r0 + 8 * t) * kbytes), kq, 0)
                                     : __builtin_amdgcn_raw_buffer_load_b128(r, (int)(b_off + 8 * t * kbytes + q * 16), kq, 0));
     };
@@ -465,7 +471,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
     // in order; then, where B is staged too, the codes of this register set's step after
     // next: the scales stay in use and follow after the multiplication), then 16 K slices
     // are multiplied
-    auto compute = [&](SkinnyRegs<MT, WN> &s, int64_t next_step, int64_t refill_step) {
+    auto compute = [&](SkinnyRegs<MT, WN> &s, BCodes &b, int64_t next_step, int64_t refill_step) {
 #pragma unroll
         for (int j = 0; j < MT * 4; ++j) *reinterpret_cast<uint4 *>(region + lds_w + j * 8 * kSkinnyPitch) = a_stage[j];
         if (kBViaLds) {
@@ -473,7 +479,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
             for (int t = 0; t < WN; ++t)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    *reinterpret_cast<uint4 *>(region + kRegionA + lds_w + (t * 32 + q * 8) * kSkinnyPitch) = s.b[t][q];
+                    *reinterpret_cast<uint4 *>(region + kRegionA + lds_w + (t * 32 + q * 8) * kSkinnyPitch) = b[t][q];
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -484,7 +490,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
         if constexpr (kBViaLds) {
             __builtin_amdgcn_sched_barrier(0);
             fetch_a(next_step);
-            fetch_b_codes(refill_step, s);
+            fetch_b_codes(refill_step, b);
             __builtin_amdgcn_sched_barrier(0);
         } else {
             if (next_step < nsteps) fetch_a(next_step);
@@ -501,7 +507,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
                 half8_t fb[WN], fa[MT];
 #pragma unroll
                 for (int t = 0; t < WN; ++t)
-                    fb[t] = dequant8(word_of(kBViaLds ? frb[q & 1][t] : s.b[t][q], j), scale_of(s.sb[t][x >> 3], x));
+                    fb[t] = dequant8(word_of(kBViaLds ? frb[q & 1][t] : b[t][q], j), scale_of(s.sb[t][x >> 3], x));
 #pragma unroll
                 for (int i = 0; i < MT; ++i) fa[i] = dequant8(word_of(fr[q & 1][i], j), scale_of(s.sa[x >> 3][i], x));
 #pragma unroll
@@ -522,36 +528,38 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
     SkinnyRegs<MT, WN> st[2];
     int64_t step = wave;  // counts this workgroup's steps, see phys()
     if constexpr (kBViaLds) {
+        // a register set of codes is refilled for the step kBSets steps after the one it held
+        constexpr int kAhead = (kBSets - 1) * kWaves;
         fetch_a(step);
-        fetch_b_codes(step, st[0]);
+        fetch_b_codes(step, bst[0]);
         fetch_scales(step, st[0]);
-        fetch_b_codes(step + kWaves, st[1]);
+        if (kBSets == 2) fetch_b_codes(step + kWaves, bst[kBSets - 1]);
         fetch_scales(step + kWaves, st[1]);
         for (; step + kWaves < nsteps; step += 2 * kWaves) {
-            compute(st[0], step + kWaves, step + 2 * kWaves);
+            compute(st[0], bst[0], step + kWaves, step + kWaves + kAhead);
             fetch_scales(step + 2 * kWaves, st[0]);
-            compute(st[1], step + 2 * kWaves, step + 3 * kWaves);
+            compute(st[1], bst[kBSets - 1], step + 2 * kWaves, step + 2 * kWaves + kAhead);
             fetch_scales(step + 3 * kWaves, st[1]);
         }
-        if (step < nsteps) compute(st[0], nsteps, nsteps);  // odd count: the last step, nothing left to fetch
+        if (step < nsteps) compute(st[0], bst[0], nsteps, nsteps);  // odd count: the last step, nothing left to fetch
     } else {
         // 256 registers are in use here: the loads stay under branches, which costs the exact
         // wait counts but keeps the accumulators out of scratch memory
-        auto fetch_b = [&](int64_t j, SkinnyRegs<MT, WN> &s) {
-            fetch_b_codes(j, s);
-            fetch_scales(j, s);
+        auto fetch_b = [&](int64_t j, int set) {
+            fetch_b_codes(j, bst[set]);
+            fetch_scales(j, st[set]);
         };
         if (step < nsteps) {
             fetch_a(step);
-            fetch_b(step, st[0]);
+            fetch_b(step, 0);
         }
-        if (step + kWaves < nsteps) fetch_b(step + kWaves, st[1]);
+        if (step + kWaves < nsteps) fetch_b(step + kWaves, 1);
         for (; step < nsteps; step += 2 * kWaves) {
-            compute(st[0], step + kWaves, 0);
-            if (step + 2 * kWaves < nsteps) fetch_b(step + 2 * kWaves, st[0]);
+            compute(st[0], bst[0], step + kWaves, 0);
+            if (step + 2 * kWaves < nsteps) fetch_b(step + 2 * kWaves, 0);
             if (step + kWaves < nsteps) {
-                compute(st[1], step + 2 * kWaves, 0);
-                if (step + 3 * kWaves < nsteps) fetch_b(step + 3 * kWaves, st[1]);
+                compute(st[1], bst[kBSets - 1], step + 2 * kWaves, 0);
+                if (step + 3 * kWaves < nsteps) fetch_b(step + 3 * kWaves, 1);
             }
         }
     }
@@ -594,7 +602,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
         }
     }
 
-    // Register f is D[m][n], m = 32 i + r, n = n128 + 32 g + r0 + 8 t + 4 h + e % 4 (tile row 8 g + 4 h + e % 4),
+    // Register f is D[m][n], m = m_base + 32 i + r, n = n128 + 32 g + r0 + 8 t + 4 h + e % 4 (tile row 8 g + 4 h + e % 4),
     // g = (f % 16) / 4; rows m >= M are padding of the band and are not written.  This wavefront's
     // registers are groups of four columns c4 = w R / 4 ... (or, for R = 2, half of group w / 2).
     constexpr int kGroups = R == 2 ? 1 : R / 4;
@@ -613,7 +621,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN)) void gemm_nvfp4_skinny_kerne
     for (int c = 0; c < kGroups; ++c) {
         const int c4 = R == 2 ? (wave >> 1) : wave * (R / 4) + c;  // group of four columns: c4 = (i WN + t) 4 + g
         const int g = c4 & 3, t = (c4 >> 2) % WN, i = (c4 >> 2) / WN;
-        const int m = 32 * i + r;
+        const int m = m_base + 32 * i + r;
         if (m >= p.M) continue;
         const int64_t n = n128 + 32 * g + r0 + 8 * t + 4 * h + (R == 2 ? (wave & 1) * 2 : 0);
         if constexpr (R == 2) {
@@ -864,12 +872,12 @@ static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
 }
 
 template <int MT, int WN>
-static int launch_skinny(GemmParams &p, int out_type, hipStream_t s) {
+static int launch_skinny(GemmParams &p, int out_type, hipStream_t s, int row_groups = 1) {
     constexpr int kWaves = skinny_waves(WN);
     constexpr size_t stage_bytes = (size_t)kWaves * (MT * 32 + (MT <= 2 || WN == 2 ? WN * 32 : 0)) * kSkinnyPitch,
                      red_bytes = (size_t)kWaves * (MT * WN * 16) * 64 * sizeof(float);
     constexpr size_t lds_bytes = stage_bytes > red_bytes ? stage_bytes : red_bytes;
-    dim3 grid((unsigned)(p.N / (32 * WN)), (unsigned)p.splits);
+    dim3 grid((unsigned)(p.N / (32 * WN)), (unsigned)p.splits, (unsigned)row_groups);
     auto kernel = p.splits > 1 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutPartial>
                   : out_type == FOS_T_BF16 ? gemm_nvfp4_skinny_kernel<MT, WN, kOutBF16> : gemm_nvfp4_skinny_kernel<MT, WN, kOutF16>;
     if (lds_bytes > 64 * 1024 &&
@@ -909,7 +917,7 @@ enum { kPlanBig, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
-    int wide;    // M > 32: workgroups of 64 rows of B, four wavefronts with two tiles each
+    int wide;    // M > 32: workgroups of 64 rows of B and 64 rows of A, four wavefronts with two by two tiles each
 };
 constexpr int kTargetWorkgroups = 256;
 static int env_int(const char *name, int fallback) {
@@ -932,9 +940,13 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
             g.narrow = 1;
             tiles = N / 16;
         }
-        if (M > 32 && tile == 64) {
+        if (M > 32 && (tile == 64 || (tile == 0 && (M > 64 || tiles > kTargetWorkgroups)))) {
+            // 64 rows of B per workgroup of four wavefronts, two workgroups per compute unit, and
+            // workgroups of their own for rows 64 ... of A: half the reads of A per multiplication.
+            // At M <= 64 it pays once the 32-row workgroups no longer run all at once (N = 14336,
+            // K = 4096: 22.4 -> 13.9 us at M = 64; N = 8192: 11.3 against 14.3 us)
             g.wide = 1;
-            tiles = N / 64;
+            tiles = (N / 64) * (M > 64 ? 2 : 1);
         }
     } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
@@ -950,7 +962,8 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     // split so that about kTargetWorkgroups workgroups run, each with a useful share of K
     // (at M <= 32 a split must leave two steps per wavefront: 16 x 4096 x 4096 takes 6.4 us
     // unsplit and 7.1 us in two halves plus their reduction)
-    const int64_t min_steps = g.kind == kPlanSkinny ? (M <= 32 ? 16 : 8) : 4;
+    // (with row groups, M > 64: 128 x 4096 x 4096 takes 12.3 us unsplit, 13.4 us in two halves)
+    const int64_t min_steps = g.kind == kPlanSkinny ? (M <= 32 || (g.wide && M > 64) ? 16 : 8) : 4;
     // (the weight-streaming kernel also splits in two when its workgroups would cover exactly
     // half of the compute units: measured 18.8 -> 15.1 us at M = 16, N = 4096, K = 14336)
     const int64_t enough = g.kind == kPlanSkinny ? kTargetWorkgroups / 2 + 1 : kTargetWorkgroups / 2;
@@ -1035,7 +1048,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
             }
             if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
             if (M <= 64) return g.wide ? launch_skinny<2, 2>(p, out_type, s) : launch_skinny<2, 1>(p, out_type, s);
-            return g.wide ? launch_skinny<4, 2>(p, out_type, s) : launch_skinny<4, 1>(p, out_type, s);
+            return g.wide ? launch_skinny<2, 2>(p, out_type, s, 2) : launch_skinny<4, 1>(p, out_type, s);
         default: return launch_gemm<2, 2, 2, 2>(p, out_type, s);
     }
 }

@@ -69,7 +69,7 @@ def test_gemm_fp16_output_and_mixed_rules(oracle):
 
 
 @pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), (16, 4096, 4096), (128, 14336, 4096), (2048, 4096, 14336),
-                                           (128, 4096, 14336), (256, 384, 2368)])
+                                           (128, 4096, 14336), (256, 384, 2368), (64, 14336, 4096), (96, 11008, 4096)])
 def test_gemm_full_size_sampled(oracle, m, n, k):
     """Headline and Llama-3-8B shapes: 192 sampled rows of each operand are multiplied by
     the oracle (fp64 accumulation) and compared with the same entries of the GPU result."""
@@ -94,9 +94,14 @@ def test_gemm_full_size_sampled(oracle, m, n, k):
 @pytest.mark.parametrize(
     ("m", "n", "k", "env"),
     [
-        (128, 1024, 4096, {}),                                  # weight-streaming kernel, split 2
+        (128, 1024, 8192, {}),                                  # weight-streaming kernel, 64-row workgroups, two row groups, split 2
         (128, 4096, 4096, {"FOS_GEMM_SPLITK": "3"}),            # ... ragged last split
         (100, 2048, 3328, {"FOS_GEMM_SPLITK": "5"}),            # ... 13 steps, idle waves, 100 of 128 rows
+        (65, 256, 1024, {"FOS_GEMM_SPLITK": "2"}),              # ... one row in the second row group
+        (48, 8448, 1024, {"FOS_GEMM_SPLITK": "2"}),             # ... one row group (more than 256 32-row tiles)
+        (64, 384, 2560, {"FOS_GEMM_SPLITK": "3", "FOS_GEMM_TILE": "64"}),  # ... forced; 10 steps over 4 wavefronts, ragged split
+        (128, 1024, 4096, {"FOS_GEMM_TILE": "32"}),             # 32-row workgroups, four A tiles per wavefront, split 2
+        (100, 2048, 3328, {"FOS_GEMM_SPLITK": "5", "FOS_GEMM_TILE": "32"}),  # ... 13 steps, idle waves, 100 of 128 rows
         (16, 1024, 4096, {"FOS_GEMM_SPLITK": "2"}),             # ... one 32-row A tile (unsplit by default: 16 steps)
         (32, 1024, 8192, {}),                                   # ... split by default
         (48, 512, 2048, {"FOS_GEMM_SPLITK": "2"}),              # ... two
