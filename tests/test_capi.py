@@ -65,7 +65,9 @@ def test_argument_checks_need_no_device(native):
     assert q(x=None) == -4
     assert q(rows=0) == -1
     assert q(ld=32) == -1
-    assert q(x_type=2) == -3
+    assert q(x_type=3) == -3
+    assert q(x_type=2, x=p + 2) == -2  # fp32 elements: 4-byte aligned
+    assert q(x_type=1, dtype=2, rule=0) == -3  # MXFP4 reads bf16 only
     assert q(dtype=7) == -3
     assert q(rule=9) == -3
     assert q(dtype=1, rule=0) == -3  # IF4 has no static rule
@@ -79,7 +81,8 @@ def test_argument_checks_need_no_device(native):
     assert g(A=None) == -4
     assert g(M=100) == -1  # fewer than 128 rows need K % 256 == 0
     assert L.fos_gemm_workspace_bytes(100, 128, 64) == 0
-    assert L.fos_gemm_workspace_bytes(128, 1024, 4096) == 2 * 128 * 1024 * 4
+    assert L.fos_gemm_workspace_bytes(128, 1024, 8192) == 2 * 128 * 1024 * 4  # two splits of 16 K steps
+    assert L.fos_gemm_workspace_bytes(128, 1024, 4096) == 0  # 16 steps: unsplit
     assert L.fos_gemm_workspace_bytes(8192, 8192, 8192) == 0
     assert g(K=32) == -1
     assert g(ldd=64) == -1
