@@ -90,6 +90,28 @@ __global__ __launch_bounds__(kThreads) void amax_rows_kernel(const uint16_t *__r
     }
 }
 
+// fp32 input, any strides: one workgroup per row, strided over the rows.
+__global__ __launch_bounds__(kThreads) void amax_rows_f32_kernel(const uint32_t *__restrict__ x, int64_t rows,
+                                                                 int64_t cols, int64_t ld,
+                                                                 uint32_t *__restrict__ partials) {
+    __shared__ uint32_t smem[4];
+    uint32_t m = 0, z = 0;
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+        const uint32_t *row = x + r * ld;
+        for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
+            const uint32_t u = row[c], v = u & 0x7fffffffu;  // magnitudes order like their bit patterns
+            m = m > v ? m : v;
+            z |= (u == 0x80000000u) ? 1u : 0u;
+        }
+    }
+    m = block_max_u32(m, smem);
+    z = block_max_u32(z, smem);
+    if (threadIdx.x == 0) {
+        partials[2 * blockIdx.x] = m;
+        partials[2 * blockIdx.x + 1] = z;
+    }
+}
+
 // partials -> one f32 (single workgroup)
 __global__ __launch_bounds__(kThreads) void amax_finalize_kernel(const uint32_t *__restrict__ partials, int n,
                                                                  float *__restrict__ amax) {
@@ -120,8 +142,19 @@ extern "C" size_t fos_quantize_workspace_bytes(int64_t, int64_t) { return 2 * kM
 namespace {
 
 // Launch pass 1; returns the number of partial maxima written to `partials`.
-int launch_amax(const void *x, int64_t rows, int64_t cols, int64_t ld, bool aligned, uint32_t *partials, hipStream_t s) {
+int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, bool aligned, uint32_t *partials,
+                hipStream_t s) {
     int n_partials;
+    if (x_type != FOS_T_BF16) {
+        n_partials = (int)(rows < kMaxPartials ? rows : kMaxPartials);
+        if (x_type == FOS_T_F32)
+            hipLaunchKernelGGL(amax_rows_f32_kernel, dim3(n_partials), dim3(kThreads), 0, s, (const uint32_t *)x, rows, cols, ld,
+                               partials);
+        else
+            hipLaunchKernelGGL((amax_rows_kernel<false>), dim3(n_partials), dim3(kThreads), 0, s, (const uint16_t *)x, rows,
+                               cols, ld, partials);
+        return n_partials;
+    }
     if (ld == cols && aligned) {
         const int64_t n_vec = rows * cols / 8;
         // each thread keeps 8 independent 128-bit loads in flight
@@ -147,8 +180,22 @@ void dispatch_2d(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     else launch_quantize<false, DT, RULE, ROUND, false>(p, aligned, s);
 }
 
+// fp16 / fp32 inputs: the element-wise kernel, whatever the alignment
+template <int DT, int RULE, int ROUND>
+void launch_typed(QuantParams &p, bool two_d, hipStream_t s) {
+    p.tiles_x = (int)(p.cols_p / 64);
+    const dim3 grid((unsigned)((p.rows_p / 128) * p.tiles_x));
+    if (two_d) hipLaunchKernelGGL((quantize_kernel<false, DT, RULE, ROUND, true, 1, false>), grid, dim3(kThreads), 0, s, p);
+    else hipLaunchKernelGGL((quantize_kernel<false, DT, RULE, ROUND, false, 1, false>), grid, dim3(kThreads), 0, s, p);
+}
+
 template <int DT, int RULE>
 void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, hipStream_t s) {
+    if (p.x_type != FOS_T_BF16) {
+        if (round_style == FOS_ROUND_NEAREST) launch_typed<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, s);
+        else launch_typed<DT, RULE, FOS_ROUND_STOCHASTIC>(p, two_d, s);
+        return;
+    }
     if (round_style == FOS_ROUND_NEAREST) {
         // NVFP4 round-to-nearest lives in fos_quantize_fast.hip
         if constexpr (DT == FOS_DTYPE_NVFP4) {
@@ -181,13 +228,13 @@ extern "C" int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, i
                         void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!x || !amax) return FOS_E_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
-    if (x_type != FOS_T_BF16) return FOS_E_UNSUPPORTED;
+    if (x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < fos_quantize_workspace_bytes(rows, cols)) return FOS_E_WORKSPACE;
-    if (((uintptr_t)x & 1) || ((uintptr_t)workspace & 3) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
+    if (((uintptr_t)x & (x_type == FOS_T_F32 ? 3 : 1)) || ((uintptr_t)workspace & 3) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
     hipStream_t s = (hipStream_t)stream;
     const bool aligned = (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0);
     uint32_t *partials = (uint32_t *)workspace;
-    const int n = launch_amax(x, rows, cols, ld, aligned, partials, s);
+    const int n = launch_amax(x, x_type, rows, cols, ld, aligned, partials, s);
     hipLaunchKernelGGL(amax_finalize_kernel, dim3(1), dim3(kThreads), 0, s, partials, n, amax);
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
 }
@@ -215,22 +262,24 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         return launch_quantize_mxfp4(x, rows, cols, ld, rule, sf_layout, codes, sf, amax, (hipStream_t)stream);
     }
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
-    if (x_type != FOS_T_BF16) return FOS_E_UNSUPPORTED;
+    if (x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
+    if (x_type != FOS_T_BF16 && pseudo_out) return FOS_E_UNSUPPORTED;  // the fused round trip reads bf16 only
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;
     if (rule < FOS_RULE_STATIC_6 || rule > FOS_RULE_ABS_MAX) return FOS_E_UNSUPPORTED;
     if (round_style < FOS_ROUND_NEAREST || round_style > FOS_ROUND_STOCHASTIC_UNBIASED) return FOS_E_UNSUPPORTED;
     if (dtype == FOS_DTYPE_IF4 && (rule == FOS_RULE_STATIC_6 || rule == FOS_RULE_STATIC_4)) return FOS_E_UNSUPPORTED;
     if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
     if (!workspace || workspace_bytes < fos_quantize_workspace_bytes(rows, cols)) return FOS_E_WORKSPACE;
-    if (((uintptr_t)x & 1) || ((uintptr_t)codes & 7) || ((uintptr_t)sf & 3) || ((uintptr_t)workspace & 3) ||
-        ((uintptr_t)amax & 3))
+    if (((uintptr_t)x & (x_type == FOS_T_F32 ? 3 : 1)) || ((uintptr_t)codes & 7) || ((uintptr_t)sf & 3) ||
+        ((uintptr_t)workspace & 3) || ((uintptr_t)amax & 3))
         return FOS_E_BAD_ALIGNMENT;
     const int64_t rows_p = fos_padded_rows(rows), cols_p = fos_padded_cols(cols);
     if (rows_p * (cols_p / 64) > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
 
     hipStream_t s = (hipStream_t)stream;
     uint32_t *partials = (uint32_t *)workspace;
-    const bool aligned = (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0);
+    // (fp16 / fp32 inputs take the element-wise kernel: treat them as unaligned throughout)
+    const bool aligned = x_type == FOS_T_BF16 && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0);
     if (pseudo_out) {
         // only the NVFP4 round-to-nearest kernels have the fused epilogue
         if (dtype != FOS_DTYPE_NVFP4 || round_style != FOS_ROUND_NEAREST || !aligned) return FOS_E_UNSUPPORTED;
@@ -242,6 +291,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     p.pseudo_out = pseudo_out;
     p.ldo = ldo;
     p.x = (const uint16_t *)x;
+    p.x_type = x_type;
     p.rows = rows; p.cols = cols; p.ld = ld;
     p.rows_p = rows_p; p.cols_p = cols_p;
     p.codes = codes; p.sf = sf;
@@ -259,7 +309,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         p.amax_out = amax;
     } else {
         p.partials = partials;
-        p.n_partials = launch_amax(x, rows, cols, ld, aligned, partials, s);
+        p.n_partials = launch_amax(x, x_type, rows, cols, ld, aligned, partials, s);
         p.amax_out = amax;
     }
 

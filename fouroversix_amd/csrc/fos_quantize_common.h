@@ -17,7 +17,8 @@ constexpr int kThreads = 256;
 constexpr int kMaxPartials = 1024;  // pairs of 32-bit words in the workspace
 
 struct QuantParams {
-    const uint16_t *x;
+    const uint16_t *x;           // bf16 / fp16 elements, or (x_type == FOS_T_F32) really const float *
+    int x_type = FOS_T_BF16;     // fp16 and fp32 inputs go through the element-wise kernel only
     int64_t rows, cols, ld;      // logical input
     int64_t rows_p, cols_p;      // padded output extents
     uint8_t *codes;              // [rows_p, cols_p / 2]
@@ -246,17 +247,13 @@ FOS_DEVICE Philox4 second_candidate_words(const Philox4 &p) { return Philox4{{p.
 
 // One 1x16 block (one row of a 16x16 tile when TWO_D): 8 input words -> 2 code words
 // and the scale byte.  `blk` = row * (cols_p / 16) + block column keys the dither.
+// The block arrives as 16 fp32 values (the reference converts its input with `.float()`,
+// reference.py:577,593,596, so bf16, fp16 and fp32 inputs meet here).
 template <int DT, int RULE, int ROUND, bool TWO_D>
-FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t seed, uint64_t offset,
-                               uint64_t blk, uint32_t *codes, uint32_t &sbyte) {
+FOS_DEVICE void quantize_block_f32(const float *x, const QuantConsts &k, uint64_t seed, uint64_t offset,
+                                   uint64_t blk, uint32_t *codes, uint32_t &sbyte) {
     constexpr bool SR = ROUND != FOS_ROUND_NEAREST;
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
-    float x[16];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        x[2 * i] = u2f(w[i] << 16);
-        x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
-    }
     float bmax = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i += 2) bmax = fmaxf(fmaxf(fabsf(x[i]), fabsf(x[i + 1])), bmax);
@@ -382,6 +379,28 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
     codes[0] = pickB ? b0 : a0;
     codes[1] = pickB ? b1 : a1;
     sbyte = pickB ? sB : sA;
+}
+
+// The same for 8 words of bf16 pairs.
+template <int DT, int RULE, int ROUND, bool TWO_D>
+FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t seed, uint64_t offset,
+                               uint64_t blk, uint32_t *codes, uint32_t &sbyte) {
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        x[2 * i] = u2f(w[i] << 16);
+        x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+    }
+    quantize_block_f32<DT, RULE, ROUND, TWO_D>(x, k, seed, offset, blk, codes, sbyte);
+}
+
+// Element (r, c) of the input as fp32 (exact for each of the three input types).
+FOS_DEVICE float load_element(const QuantParams &p, int64_t r, int64_t c) {
+    const int64_t i = r * p.ld + c;
+    if (p.x_type == FOS_T_F32) return reinterpret_cast<const float *>(p.x)[i];
+    const uint16_t h = p.x[i];
+    if (p.x_type == FOS_T_F16) return (float)__builtin_bit_cast(_Float16, h);
+    return u2f((uint32_t)h << 16);
 }
 
 // Offset of scale (r, c) inside the 128x4-tile layout (quantize/utils.py:88-96).

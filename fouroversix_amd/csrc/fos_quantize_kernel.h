@@ -55,13 +55,19 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
     const int64_t cb_base = (int64_t)tile_x * (4 * T) + (lane >> 4);
 
     constexpr int NB = 2 * T;  // blocks per lane: T column groups x 2 row halves
+    // the element-wise form (any alignment) is also the one that reads fp16 and fp32 inputs
+    constexpr bool TYPED = !FAST && !ALIGNED;
     uint32_t w[NB][8];
+    float xf[TYPED ? NB : 1][16];
 #pragma unroll
     for (int it = 0; it < NB; ++it) {
         const int64_t r = row_base + (it & 1) * 64;
         const int64_t cb = cb_base + (it >> 1) * 4;
         const int64_t c0 = cb * 16;
-        if (ALIGNED) {
+        if (TYPED) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) xf[it][i] = (r < p.rows && c0 + i < p.cols) ? load_element(p, r, c0 + i) : 0.0f;
+        } else if (ALIGNED) {
             if (r < p.rows && c0 < p.cols) {
                 const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
                 uint4 lo = src[0], hi = src[1];
@@ -101,7 +107,10 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
             codes[0] = o.c0;
             codes[1] = o.c1;
             sbyte = o.s;
-        } else
+        } else if (TYPED)
+            quantize_block_f32<DT, RULE, ROUND, TWO_D>(xf[it], k, p.seed, p.offset, (uint64_t)(r * sf_cols + cb), codes,
+                                                       sbyte);
+        else
             quantize_block<DT, RULE, ROUND, TWO_D>(w[it], k, p.seed, p.offset, (uint64_t)(r * sf_cols + cb), codes,
                                                    sbyte);
         *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(codes[0], codes[1]);

@@ -32,8 +32,12 @@ def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | Non
         return f"format {config.dtype.value} has no gfx950 kernel"
     if x.device.type != "cuda":
         return f"input must live on the GPU, got {x.device}"
-    if x.dtype != torch.bfloat16:
-        return f"input must be bfloat16, got {x.dtype}"
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        return f"input must be bfloat16, float16 or float32, got {x.dtype}"
+    if x.dtype != torch.bfloat16 and (config.dtype == DataType.mxfp4 or config.rht or config.transpose):
+        # the reference converts any input with `.float()` (quantize/pytorch/reference.py:577,593,596);
+        # here the element-wise nvfp4 / if4 kernel reads the other two types
+        return f"mxfp4, rht and transpose take bfloat16 input only, got {x.dtype}"
     if config.dtype == DataType.mxfp4 and (config.block_scale_2d or config.round_style.is_stochastic):
         return "mxfp4 has kernels for 1x32 blocks with round-to-nearest only"
     if config.rht or config.transpose:
@@ -74,7 +78,7 @@ def quantize(
     x: torch.Tensor,
     config: QuantizationConfig | None = None,
 ) -> QuantizedTensor | torch.Tensor:
-    """Quantize a 2-D bf16 GPU tensor to a block-scaled 4-bit format.
+    """Quantize a 2-D bf16 (nvfp4 / if4: also fp16 or fp32) GPU tensor to a block-scaled 4-bit format.
 
     With no config: NVFP4, 1x16 blocks, round-to-nearest, 4/6 selection by block MSE.
     ``config.kwargs`` may carry ``seed`` / ``offset`` (ints) keying the dither of the

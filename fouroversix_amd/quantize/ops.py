@@ -83,8 +83,8 @@ class _on_device:
 def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
     if x.dim() != 2:
         raise RuntimeError("quantize: x must be 2-D")
-    if x.dtype != torch.bfloat16:
-        raise RuntimeError("quantize: x must be bfloat16")
+    if x.dtype not in nat.TORCH_TO_T or (dtype == MXFP4 and x.dtype != torch.bfloat16):
+        raise RuntimeError(f"quantize: x must be bfloat16 (float16 / float32 for nvfp4 and if4), got {x.dtype}")
     if x.stride(-1) != 1:
         raise RuntimeError("quantize: x must be contiguous on the last dim")
     nat.require_gpu_tensor(x, "x")
@@ -111,7 +111,7 @@ def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, s
         stream = nat.current_stream(dev)
         workspace = _workspace(dev, stream)
         rc = L.fos_quantize(
-            x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), dtype, selection_rule, round_style, int(is_2d),
+            x.data_ptr(), nat.TORCH_TO_T[x.dtype], rows, cols, x.stride(0), dtype, selection_rule, round_style, int(is_2d),
             seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF, sf_layout,
             values.data_ptr(), sf.data_ptr(), amax_buf.data_ptr(), int(amax_is_input),
             workspace.data_ptr(), workspace.numel(), stream,
@@ -198,6 +198,9 @@ def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selec
         raise RuntimeError("quantize: only the NVFP4 format is implemented by this op (use quantize_ex for IF4)")
     if not 0 <= selection_rule <= 4:
         raise RuntimeError(f"Invalid selection_rule: {selection_rule}")
+    # the reference's native op takes fp16 and bf16 (csrc/quantize/fp4_quant.cu:134-136)
+    if x.dtype not in (torch.float16, torch.bfloat16) or (x.dtype != torch.bfloat16 and (is_rht or is_transpose)):
+        raise RuntimeError(f"quantize: x must be bfloat16 (or float16 without rht / transpose), got {x.dtype}")
     seed = 0 if rbits < 0 else rbits
     amax = None
     if is_rht or is_transpose:

@@ -62,8 +62,8 @@ int64_t fos_padded_cols_for(int dtype, int64_t cols);
 size_t fos_quantize_workspace_bytes(int64_t rows, int64_t cols);
 
 /*
- * amax[0] = max |x| over a row-major 16-bit float matrix (pass 1 of fos_quantize on its
- * own).  Stands in for `x.abs().max().float()` of the reference quantizer
+ * amax[0] = max |x| over a row-major matrix of x_type (FOS_T_BF16, FOS_T_F16 or FOS_T_F32)
+ * elements (pass 1 of fos_quantize on its own).  Stands in for `x.abs().max().float()` of the reference quantizer
  * (src/fouroversix/quantize/pytorch/reference.py:573-578; the prologue kernel of the
  * native op, src/fouroversix/csrc/include/fp4_quant_kernel.h:195-215).  Same workspace
  * as fos_quantize.
@@ -72,7 +72,7 @@ int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, 
              void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
- * Quantize a row-major 16-bit float matrix x[rows, cols] (leading dimension ld elements)
+ * Quantize a row-major matrix x[rows, cols] (leading dimension ld elements)
  * to packed 4-bit codes with one E4M3 scale per 1x16 block and one FP32 tensor scale.
  * Stands in for torch.ops.fouroversix.quantize (src/fouroversix/csrc/bindings.cpp:28,
  * csrc/quantize/fp4_quant.cu:99-239) with the semantics of the reference's PyTorch
@@ -80,8 +80,10 @@ int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, 
  * quantize/pytorch/reference.py:555-679): the input is zero-padded to
  * (fos_padded_rows, fos_padded_cols) and every padded output element is written.
  *
- *   x_type      FOS_T_BF16 (the only input type implemented; anything else returns
- *               FOS_E_UNSUPPORTED)
+ *   x_type      FOS_T_BF16; FOS_T_F16 and FOS_T_F32 (the reference converts its input with
+ *               `.float()`, reference.py:577,593,596; its native op takes bf16 and fp16,
+ *               csrc/quantize/fp4_quant.cu:134-136) are read by an element-wise kernel: same
+ *               results, below the bf16 kernels' speed
  *   dtype       FOS_DTYPE_*; rule FOS_RULE_* (IF4 takes only the adaptive rules)
  *   round_style FOS_ROUND_*; seed/offset key the Philox dither of the stochastic styles
  *   block2d     non-zero: one scale and one decision per 16x16 tile

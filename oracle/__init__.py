@@ -70,6 +70,8 @@ def lib() -> ctypes.CDLL:
         L.fos_oracle_quantize.restype = i32
         L.fos_oracle_quantize_with_amax.argtypes = [vp, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, vp, i32]
         L.fos_oracle_quantize_with_amax.restype = i32
+        L.fos_oracle_quantize_typed.argtypes = [vp, i32, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, vp, i32]
+        L.fos_oracle_quantize_typed.restype = i32
         L.fos_oracle_blocked_offset.argtypes = [i64, i64, i64]
         L.fos_oracle_blocked_offset.restype = i64
         L.fos_oracle_to_blocked.argtypes = [vp, i64, i64, vp]
@@ -138,9 +140,27 @@ def pad_bits(xb: np.ndarray) -> np.ndarray:
     mp, np_ = -(-m // 128) * 128, -(-n // 64) * 64
     if (mp, np_) == (m, n):
         return xb
-    out = np.zeros((mp, np_), dtype=np.uint16)
+    out = np.zeros((mp, np_), dtype=xb.dtype)
     out[:m, :n] = xb
     return out
+
+
+def input_bits(x) -> tuple[np.ndarray, int]:
+    """(array, input type id) of a quantize input: bf16 (torch tensor or uint16 bit patterns) -> uint16, 0;
+    fp16 (torch or numpy) -> uint16 bit patterns, 1; fp32 -> float32, 2."""
+    if isinstance(x, np.ndarray):
+        if x.dtype == np.float32:
+            return np.ascontiguousarray(x), 2
+        if x.dtype == np.float16:
+            return np.ascontiguousarray(x).view(np.uint16), 1
+        return bf16_bits(x), 0
+    import torch
+
+    if x.dtype == torch.float32:
+        return x.detach().cpu().contiguous().numpy(), 2
+    if x.dtype == torch.float16:
+        return x.detach().cpu().contiguous().numpy().view(np.uint16), 1
+    return bf16_bits(x), 0
 
 
 # Hard-coded sign vector and Sylvester-ordered 16-point Hadamard matrix of the reference's
@@ -181,9 +201,10 @@ def transform(xb: np.ndarray, *, transpose=False, rht=False) -> np.ndarray:
 def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
              block_scale_2d=False, seed=0, offset=0, threads=None,
              transpose=False, rht=False, amax=None) -> OracleQuantized:
-    xb = bf16_bits(x)
+    xb, x_type = input_bits(x)
     assert xb.ndim == 2
     if transpose or rht:
+        assert x_type == 0, "transpose / rht: bf16 input only"
         xb = transform(xb, transpose=transpose, rht=rht)
     orig = tuple(int(v) for v in xb.shape)
     xp = np.ascontiguousarray(pad_bits(xb))
@@ -192,8 +213,8 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
     sf = np.zeros((mp, np_ // 16), dtype=np.uint8)
     amax_in = None if amax is None else np.array([amax], dtype=np.float32)
     amax = np.zeros(1, dtype=np.float32)
-    rc = lib().fos_oracle_quantize_with_amax(
-        _ptr(xp), mp, np_, DTYPE_IDS[dtype], RULE_IDS[scale_rule], ROUND_IDS[round_style],
+    rc = lib().fos_oracle_quantize_typed(
+        _ptr(xp), x_type, mp, np_, DTYPE_IDS[dtype], RULE_IDS[scale_rule], ROUND_IDS[round_style],
         int(block_scale_2d), seed, offset, _ptr(codes), _ptr(sf), _ptr(amax),
         None if amax_in is None else _ptr(amax_in), threads or default_threads(),
     )

@@ -410,10 +410,29 @@ static double adj_of(int round_style) {
  */
 /* `amax_in` (may be NULL) is the reference function's x_amax argument (reference.py:557,
  * 573-578): the tensor scale to use instead of max|x|. */
-int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,
-                                  int round_style, int block2d, uint64_t seed, uint64_t offset,
-                                  uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
-                                  int nthreads) {
+/* fp16 bits -> fp32 (exact). */
+static inline float f16_to_f32(uint16_t h) {
+    const uint32_t e = (h >> 10) & 31u, m = h & 1023u;
+    float v;
+    if (e == 0) v = ldexpf((float)m, -24);
+    else if (e == 31) v = m ? NAN : INFINITY;
+    else v = ldexpf((float)(m | 1024u), (int)e - 25);
+    return (h & 0x8000u) ? -v : v;
+}
+
+/* Element i of an input of type x_type (0 bf16, 1 fp16: 16-bit patterns; 2 fp32) as fp32:
+ * the reference converts whatever it is given with `.float()` (reference.py:577,593,596). */
+static inline float load_x(const void *x, int x_type, int64_t i) {
+    if (x_type == 2) return ((const float *)x)[i];
+    const uint16_t h = ((const uint16_t *)x)[i];
+    return x_type == 1 ? f16_to_f32(h) : bf16_to_f32(h);
+}
+
+int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, int dtype, int rule,
+                              int round_style, int block2d, uint64_t seed, uint64_t offset,
+                              uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                              int nthreads) {
+    if (x_type < 0 || x_type > 2) return -1;
     if (N % 16 != 0 || (block2d && M % 16 != 0)) return -1;
     if (dtype != FOS_NVFP4 && dtype != FOS_IF4) return -1;
     if (dtype == FOS_IF4 && (rule == RULE_STATIC6 || rule == RULE_STATIC4)) return -1;
@@ -424,7 +443,7 @@ int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int d
         amax = *amax_in;
     } else {
         for (int64_t i = 0; i < M * N; ++i) {
-            float a = fabsf(bf16_to_f32(x[i]));
+            float a = fabsf(load_x(x, x_type, i));
             if (a > amax) amax = a;
         }
     }
@@ -451,8 +470,7 @@ int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int d
         for (int64_t r = 0; r < M; ++r) {
             float xb[16], fq[16];
             for (int64_t cb = 0; cb < bpr; ++cb) {
-                const uint16_t *src = x + r * N + cb * 16;
-                for (int i = 0; i < 16; ++i) xb[i] = bf16_to_f32(src[i]);
+                for (int i = 0; i < 16; ++i) xb[i] = load_x(x, x_type, r * N + cb * 16 + i);
                 int is_int; uint8_t s;
                 quantize_block(&q, xb, 16, (uint64_t)(r * bpr + cb), fq, &is_int, &s);
                 sf[r * bpr + cb] = s;
@@ -471,7 +489,7 @@ int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int d
             for (int64_t cb = 0; cb < bpr; ++cb) {
                 for (int r = 0; r < 16; ++r)
                     for (int i = 0; i < 16; ++i)
-                        xb[16 * r + i] = bf16_to_f32(x[(rt * 16 + r) * N + cb * 16 + i]);
+                        xb[16 * r + i] = load_x(x, x_type, (rt * 16 + r) * N + cb * 16 + i);
                 int is_int; uint8_t s;
                 quantize_block(&q, xb, 256, (uint64_t)(rt * 16 * bpr + cb), fq, &is_int, &s);
                 for (int r = 0; r < 16; ++r) {
@@ -488,6 +506,14 @@ int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int d
         }
     }
     return 0;
+}
+
+int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,
+                                  int round_style, int block2d, uint64_t seed, uint64_t offset,
+                                  uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                                  int nthreads) {
+    return fos_oracle_quantize_typed(x, 0, M, N, dtype, rule, round_style, block2d, seed, offset, codes, sf, amax_out,
+                                     amax_in, nthreads);
 }
 
 int fos_oracle_quantize(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,

@@ -200,8 +200,35 @@ def write_f32_intermediate_vectors(quantize, dequantize, QuantizationConfig) -> 
     print("wrote dequantize_f32_intermediate", len(out))
 
 
+def write_input_dtype_vectors(quantize, QuantizationConfig) -> None:  # noqa: N803
+    """fp32 and fp16 inputs: the reference converts whatever it is given with `.float()`
+    (quantize/pytorch/reference.py:577,593,596), so an input with more significant bits than
+    bf16 reaches the block arithmetic unrounded."""
+    out: dict[str, np.ndarray] = {}
+    for name, kind, shape, seed in [("randn_128x128", "randn", (128, 128), 61), ("ragged_100x80", "randn", (100, 80), 62),
+                                    ("outlier_128x256", "outlier", (128, 256), 63)]:
+        g = torch.Generator("cpu").manual_seed(seed)
+        base = torch.randn(*shape, generator=g)
+        if kind == "outlier":
+            base[:, 7] *= 50.0
+        for tname, x in (("f32", base), ("f16", base.half())):
+            out[f"{name}.{tname}.x"] = x.numpy().copy() if tname == "f32" else x.numpy().view(np.uint16).copy()
+            for dtype, rule, two_d in (("nvfp4", "mse", False), ("nvfp4", "static_6", False), ("nvfp4", "mse", True),
+                                       ("nvfp4", "abs_max", False), ("if4", "mse", False)):
+                if two_d and shape[0] % 16:
+                    continue
+                q = quantize(x.clone(), QuantizationConfig(backend="pytorch", dtype=dtype, scale_rule=rule, block_scale_2d=two_d))
+                key = f"{name}.{tname}.{dtype}.{rule}.{'2d' if two_d else '1d'}"
+                out[key + ".values"] = u8(q.values)
+                out[key + ".sf"] = u8(q.scale_factors)
+                out[key + ".amax"] = np.array([float(q.amax)], dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "input_dtypes.npz"), **out)
+    print("wrote input_dtypes", len(out))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--only-input-dtypes", action="store_true", help="write only input_dtypes.npz")
     ap.add_argument("--only-dequant32", action="store_true", help="write only dequantize_f32_intermediate.npz")
     ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
     ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
@@ -212,6 +239,9 @@ def main() -> None:
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_input_dtype_vectors(quantize, QuantizationConfig)
+    if args.only_input_dtypes:
+        return
     write_f32_intermediate_vectors(quantize, dequantize, QuantizationConfig)
     if args.only_dequant32:
         return

@@ -37,6 +37,36 @@ def test_quantize_matches_reference_vectors(oracle, path):
         assert np.array_equal(q.scale_factors, d[k + ".sf"].reshape(-1)), k
 
 
+def _typed_input(d, name, tname):
+    x = d[f"{name}.{tname}.x"]
+    return x if tname == "f32" else x.view(np.float16)
+
+
+def test_quantize_of_fp32_and_fp16_inputs_matches_reference_vectors(oracle, golden_dir):
+    """The reference converts any input with `.float()`: inputs with more significant bits than
+    bf16 (fp32 randn, fp16 randn, ragged and outlier shapes) against its PyTorch backend's bytes."""
+    d = np.load(os.path.join(golden_dir, "input_dtypes.npz"))
+    keys = _keys(d)
+    assert len(keys) >= 24
+    for k in keys:
+        name, tname, dt, rule, dim = k.split(".")
+        q = oracle.quantize(_typed_input(d, name, tname), dtype=dt, scale_rule=rule, block_scale_2d=(dim == "2d"))
+        assert q.amax == d[k + ".amax"][0], k
+        assert np.array_equal(q.values, d[k + ".values"]), k
+        assert np.array_equal(q.scale_factors, d[k + ".sf"].reshape(-1)), k
+
+
+def test_quantize_input_type_does_not_matter_for_bf16_values(oracle):
+    """bf16 values handed over as fp32 (and fp16 values as fp32) give the same bytes."""
+    g = torch.Generator("cpu").manual_seed(71)
+    x = torch.randn(128, 192, generator=g)
+    for narrow in (x.bfloat16(), x.half()):
+        for kw in (dict(scale_rule="mse"), dict(scale_rule="mae", block_scale_2d=True), dict(dtype="if4", scale_rule="mse"),
+                   dict(scale_rule="static_6", round_style="stochastic", seed=5)):
+            a, b = oracle.quantize(narrow, **kw), oracle.quantize(narrow.float(), **kw)
+            assert a.amax == b.amax and np.array_equal(a.values, b.values) and np.array_equal(a.scale_factors, b.scale_factors), kw
+
+
 def test_quantize_config1_digest(oracle, golden_dir):
     """1024x1024 randn seed 0, static_6 and mse: SHA-256 of codes and scales."""
     d = np.load(os.path.join(golden_dir, "quantize_config1_1024x1024.npz"))

@@ -57,6 +57,72 @@ def test_matches_reference_vectors(path):
             assert np.array_equal(bits16(fos.dequantize(q)), d[k + ".deq_bf16"]), k
 
 
+def test_fp32_and_fp16_inputs_match_reference_vectors(golden_dir):
+    """Inputs with more significant bits than bf16, which the reference converts with `.float()`:
+    bytes written by its PyTorch backend for fp32 and fp16 tensors (ragged and outlier shapes too)."""
+    d = np.load(os.path.join(golden_dir, "input_dtypes.npz"))
+    keys = sorted({k.rsplit(".", 1)[0] for k in d.files if k.endswith(".values")})
+    assert len(keys) >= 24
+    for k in keys:
+        name, tname, dt, rule, dim = k.split(".")
+        raw = d[f"{name}.{tname}.x"]
+        x = torch.from_numpy(raw.copy()) if tname == "f32" else torch.from_numpy(raw.view(np.int16).copy()).view(torch.float16)
+        q = hip_quantize(x, dtype=dt, scale_rule=rule, block_scale_2d=(dim == "2d"))
+        assert tuple(q.original_shape) == tuple(x.shape), k
+        assert float(q.amax) == float(d[k + ".amax"][0]), k
+        assert np.array_equal(u8(q.values), d[k + ".values"]), k
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), d[k + ".sf"].reshape(-1)), k
+
+
+@pytest.mark.parametrize("in_dtype", [torch.float32, torch.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize(("cfg"), [
+    dict(scale_rule="mse"), dict(scale_rule="mae", block_scale_2d=True), dict(scale_rule="abs_max"),
+    dict(scale_rule="static_4", block_scale_2d=True), dict(dtype="if4", scale_rule="mse"), dict(dtype="if4", scale_rule="mae", block_scale_2d=True),
+    dict(scale_rule="mse", round_style="stochastic"), dict(scale_rule="static_6", round_style="stochastic_unbiased"),
+    dict(dtype="if4", scale_rule="abs_max", round_style="stochastic"),
+], ids=str)
+def test_fp32_and_fp16_inputs_match_oracle(oracle, in_dtype, cfg):
+    """Every rule / format / rounding style on fp32 and fp16 data (element-wise kernel), aligned and
+    ragged shapes, strided rows; bf16 values handed over in the wider type give the bf16 kernels' bytes."""
+    g = torch.Generator("cpu").manual_seed(17)
+    kwargs = {"seed": 7, "offset": 1} if "round_style" in cfg else {}
+    okw = dict(seed=7, offset=1) if "round_style" in cfg else {}
+    for shape in ((256, 320), (100, 80), (16, 4096)):
+        x = (torch.randn(*shape, generator=g) * 3.0).to(in_dtype)
+        q = hip_quantize(x, kwargs=kwargs, **cfg)
+        assert_same_quantization(q, oracle.quantize(x, **okw, **cfg), f"{in_dtype} {shape} {cfg}")
+    wide = (torch.randn(64, 512, generator=g)).to(in_dtype).cuda()
+    view = wide[:, 64:320]  # row stride 512 elements, offset start
+    q = fos.quantize(view, fos.QuantizationConfig(kwargs=kwargs, **cfg))
+    assert_same_quantization(q, oracle.quantize(view.cpu().contiguous(), **okw, **cfg), f"strided {in_dtype} {cfg}")
+    xb = torch.randn(128, 256, generator=g).bfloat16()
+    if in_dtype == torch.float32:
+        same = hip_quantize(xb.float(), kwargs=kwargs, **cfg)
+        base = hip_quantize(xb, kwargs=kwargs, **cfg)
+        assert torch.equal(same.values, base.values) and torch.equal(same.scale_factors.view(torch.uint8), base.scale_factors.view(torch.uint8))
+        assert float(same.amax) == float(base.amax)
+
+
+def test_fp32_and_fp16_inputs_other_paths(oracle):
+    """pseudo-quantize composes quantize -> dequantize in the input's type; amax can be supplied; formats and
+    options without a kernel for these types say so."""
+    g = torch.Generator("cpu").manual_seed(3)
+    x = torch.randn(128, 128, generator=g)
+    for t in (torch.float32, torch.float16):
+        xt = x.to(t).cuda()
+        out = fos.quantize(xt, fos.QuantizationConfig(pseudo_quantize=True))
+        assert out.dtype == t and out.shape == xt.shape
+        q = fos.quantize(xt)
+        assert torch.equal(out, fos.dequantize(q, dtype=t))
+        q2 = fos.quantize(xt, fos.QuantizationConfig(kwargs={"amax": q.amax}))
+        assert torch.equal(q2.values, q.values)
+        for bad in (dict(dtype="mxfp4", scale_rule="static_6"), dict(rht=True), dict(transpose=True)):
+            with pytest.raises(ValueError, match="bfloat16 input only"):
+                fos.quantize(xt, fos.QuantizationConfig(**bad))
+    with pytest.raises(ValueError, match="bfloat16, float16 or float32"):
+        fos.quantize(x.double().cuda())
+
+
 @pytest.mark.parametrize(("shape", "kind", "cfg"), [
     ((8192, 4096), "outlier", dict(scale_rule="mse")),            # activation-style
     ((8192, 8192), "randn", dict(scale_rule="mse")),              # headline size
@@ -201,6 +267,11 @@ def test_reference_op_schema(oracle):
         ops.quantize(x.cuda(), True, True, False, False, False, 9, -1)
     with pytest.raises(RuntimeError):
         ops.quantize(x.cuda().float(), True, True, False, False, False, 0, -1)
+    # fp16 is the other input type of the reference's op (csrc/quantize/fp4_quant.cu:134-136)
+    h = make_input("randn", (256, 128), 7).half()
+    values, sf, amax = ops.quantize(h.cuda(), True, True, False, True, False, fos.ScaleRule.mae.cuda_id, -1)
+    ref = oracle.quantize(h, scale_rule="mae", block_scale_2d=True)
+    assert np.array_equal(u8(values), ref.values) and np.array_equal(u8(sf), ref.scale_factors) and float(amax) == float(ref.amax)
 
 
 @pytest.mark.parametrize(("dtype", "rule", "two_d"), [
