@@ -191,6 +191,28 @@ def test_linear_layer_forward(oracle):
     assert torch.equal(keep(x.cuda()), y)
 
 
+def test_linear_layer_forward_in_fp16(oracle):
+    """An fp16 model: fp16 activations and weights are quantized from their own values (the
+    reference converts with `.float()`), fp16 output."""
+    torch.manual_seed(1)
+    lin = nn.Linear(256, 384, bias=True, dtype=torch.float16)
+    w, bias = lin.weight.detach().clone(), lin.bias.detach().clone()
+    layer = fos.FourOverSixLinear(lin.cuda(), fos.ModuleQuantizationConfig(weight_scale_2d=True, output_dtype="float16"))
+    layer.quantize_weight_()
+    x = make_input("randn", (96, 256), 36).half()
+    y = layer(x.cuda())
+    assert y.shape == (96, 384) and y.dtype == torch.float16
+    rx = oracle.quantize(x, scale_rule="mse")
+    rw = oracle.quantize(w, scale_rule="mse", block_scale_2d=True)
+    _, f32 = oracle.gemm_nvfp4(rx.values, rx.scale_rows, rw.values, rw.scale_rows, oracle.gemm_alpha(rx, rw))
+    expect = torch.from_numpy(f32[:96, :384].copy()).half() + bias
+    got = y.detach().cpu()
+    # fp16's grid is 8x finer than bf16's, so FP32 re-association shows on 8x as many outputs: the
+    # budget scales with it (a unit in the last place of the product, before the bias is added)
+    assert float((got != expect).float().mean()) <= 8 * MISMATCH_BUDGET
+    assert float((got.float() - expect.float()).abs().max() / expect.float().abs().max()) <= MAX_REL
+
+
 def test_formats_without_a_native_gemm_take_the_dequantize_form(oracle):
     """IF4 operands (and an fp32 result) go through dequantize + matmul, the reference's
     PyTorch matmul backend (src/fouroversix/matmul/pytorch.py:33-52); compared with the
