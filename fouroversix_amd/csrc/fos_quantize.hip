@@ -90,6 +90,38 @@ __global__ __launch_bounds__(kThreads) void amax_rows_kernel(const uint16_t *__r
     }
 }
 
+// fp32 input, contiguous and 16-byte aligned, viewed as n_vec 128-bit vectors.
+__global__ __launch_bounds__(kThreads) void amax_flat_f32_kernel(const uint4 *__restrict__ x, int64_t n_vec,
+                                                                 uint32_t *__restrict__ partials) {
+    __shared__ uint32_t smem[4];
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    uint32_t m = 0, z = 0;
+    auto take = [&](uint32_t u) {
+        const uint32_t v = u & 0x7fffffffu;
+        m = m > v ? m : v;
+        z |= (u == 0x80000000u) ? 1u : 0u;
+    };
+    constexpr int U = 8;
+    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    for (; i + (U - 1) * stride < n_vec; i += U * stride) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = x[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < U; ++u) take(v[u].x), take(v[u].y), take(v[u].z), take(v[u].w);
+    }
+    for (; i < n_vec; i += stride) {
+        const uint4 v = x[i];
+        take(v.x), take(v.y), take(v.z), take(v.w);
+    }
+    m = block_max_u32(m, smem);
+    z = block_max_u32(z, smem);
+    if (threadIdx.x == 0) {
+        partials[2 * blockIdx.x] = m;
+        partials[2 * blockIdx.x + 1] = z;
+    }
+}
+
 // fp32 input, any strides: one workgroup per row, strided over the rows.
 __global__ __launch_bounds__(kThreads) void amax_rows_f32_kernel(const uint32_t *__restrict__ x, int64_t rows,
                                                                  int64_t cols, int64_t ld,
@@ -145,6 +177,18 @@ namespace {
 int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, bool aligned, uint32_t *partials,
                 hipStream_t s) {
     int n_partials;
+    if (x_type != FOS_T_BF16 && ld == cols && ((uintptr_t)x & 15) == 0 && (rows * cols) % 8 == 0) {
+        // contiguous: the flat scans (fp16 shares the bf16 one, magnitudes order like bit patterns)
+        const int64_t n_vec = rows * cols / (x_type == FOS_T_F32 ? 4 : 8);
+        const int64_t want = (n_vec + kThreads * 8 - 1) / (kThreads * 8);
+        n_partials = (int)(want > 256 ? 256 : (want < 1 ? 1 : want));
+        if (x_type == FOS_T_F32)
+            hipLaunchKernelGGL(amax_flat_f32_kernel, dim3(n_partials), dim3(kThreads), 0, s, (const uint4 *)x, n_vec, partials);
+        else
+            hipLaunchKernelGGL((amax_flat_kernel<false>), dim3(n_partials), dim3(kThreads), 0, s, (const uint4 *)x, n_vec,
+                               partials);
+        return n_partials;
+    }
     if (x_type != FOS_T_BF16) {
         n_partials = (int)(rows < kMaxPartials ? rows : kMaxPartials);
         if (x_type == FOS_T_F32)
@@ -292,6 +336,10 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     p.ldo = ldo;
     p.x = (const uint16_t *)x;
     p.x_type = x_type;
+    {
+        const int64_t esize = x_type == FOS_T_F32 ? 4 : 2;
+        p.x_vec = x_type != FOS_T_BF16 && ((uintptr_t)x & 15) == 0 && (ld * esize) % 16 == 0 && cols % 16 == 0;
+    }
     p.rows = rows; p.cols = cols; p.ld = ld;
     p.rows_p = rows_p; p.cols_p = cols_p;
     p.codes = codes; p.sf = sf;

@@ -19,6 +19,7 @@ constexpr int kMaxPartials = 1024;  // pairs of 32-bit words in the workspace
 struct QuantParams {
     const uint16_t *x;           // bf16 / fp16 elements, or (x_type == FOS_T_F32) really const float *
     int x_type = FOS_T_BF16;     // fp16 and fp32 inputs go through the element-wise kernel only
+    int x_vec = 0;               // ... with 128-bit loads when base, row pitch and width allow (16-byte aligned rows, cols % 16 == 0)
     int64_t rows, cols, ld;      // logical input
     int64_t rows_p, cols_p;      // padded output extents
     uint8_t *codes;              // [rows_p, cols_p / 2]
@@ -392,6 +393,32 @@ FOS_DEVICE void quantize_block(const uint32_t *w, const QuantConsts &k, uint64_t
         x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
     }
     quantize_block_f32<DT, RULE, ROUND, TWO_D>(x, k, seed, offset, blk, codes, sbyte);
+}
+
+// The 16 elements of block column cb of row r as fp32, 128-bit loads (QuantParams::x_vec).
+FOS_DEVICE void load_block16(const QuantParams &p, int64_t r, int64_t c0, float *x) {
+    if (p.x_type == FOS_T_F32) {
+        const float4 *src = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.x) + r * p.ld + c0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float4 v = src[i];
+            x[4 * i] = v.x, x[4 * i + 1] = v.y, x[4 * i + 2] = v.z, x[4 * i + 3] = v.w;
+        }
+        return;
+    }
+    const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
+    const uint4 lo = src[0], hi = src[1];
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        if (p.x_type == FOS_T_F16) {
+            x[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xffffu));
+            x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+        } else {
+            x[2 * i] = u2f(w[i] << 16);
+            x[2 * i + 1] = u2f(w[i] & 0xffff0000u);
+        }
+    }
 }
 
 // Element (r, c) of the input as fp32 (exact for each of the three input types).

@@ -65,8 +65,12 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
         const int64_t cb = cb_base + (it >> 1) * 4;
         const int64_t c0 = cb * 16;
         if (TYPED) {
+            if (p.x_vec && r < p.rows && c0 < p.cols) {
+                load_block16(p, r, c0, xf[it]);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) xf[it][i] = (r < p.rows && c0 + i < p.cols) ? load_element(p, r, c0 + i) : 0.0f;
+                for (int i = 0; i < 16; ++i) xf[it][i] = (r < p.rows && c0 + i < p.cols) ? load_element(p, r, c0 + i) : 0.0f;
+            }
         } else if (ALIGNED) {
             if (r < p.rows && c0 < p.cols) {
                 const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
