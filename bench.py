@@ -188,7 +188,8 @@ def extras(dev, steps: int) -> dict:
         out[f"{name}_8192x8192_us"] = us(lambda: fos.quantize(nxt(), cfg))
     del xs
     mse = fos.QuantizationConfig(scale_rule="mse")
-    for m, nn, k in ((16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336), (128, 4096, 4096), (2048, 14336, 4096)):
+    for m, nn, k in ((16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336), (128, 4096, 4096), (128, 14336, 4096),
+                     (128, 4096, 14336), (2048, 14336, 4096)):
         qa = fos.quantize(make_activation(m, k, 7).to(dev), mse)
         qb = fos.quantize(make_activation(nn, k, 8).to(dev), mse)
         out[f"gemm_nvfp4_{m}x{nn}x{k}_us"] = us(lambda: fos.quantized_matmul(qa, qb))
