@@ -127,7 +127,7 @@ int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t
  * codes or scales.  Stands in for QuantizeBackendBase.pseudo_quantize
  * (src/fouroversix/quantize/backend.py:213-234; fused Triton kernel
  * src/fouroversix/kernels/triton/ops.py:212-374).  Arguments as fos_quantize.  Fused
- * kernels exist for FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST, x and out 16-byte aligned,
+ * kernels exist for FOS_T_BF16 input, FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST, x and out 16-byte aligned,
  * ld and ldo multiples of 8 and cols a multiple of 16; anything else returns
  * FOS_E_UNSUPPORTED (compose fos_quantize and fos_dequantize instead).
  */
