@@ -72,6 +72,8 @@ def lib() -> ctypes.CDLL:
         L.fos_oracle_quantize_with_amax.restype = i32
         L.fos_oracle_quantize_typed.argtypes = [vp, i32, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, vp, i32]
         L.fos_oracle_quantize_typed.restype = i32
+        L.fos_oracle_quantize_errors.argtypes = [vp, i32, i64, i64, i32, i32, i32, i32, u64, u64, vp, vp, vp, vp, i32, vp]
+        L.fos_oracle_quantize_errors.restype = i32
         L.fos_oracle_blocked_offset.argtypes = [i64, i64, i64]
         L.fos_oracle_blocked_offset.restype = i64
         L.fos_oracle_to_blocked.argtypes = [vp, i64, i64, vp]
@@ -224,6 +226,26 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
     flat = to_blocked(sf) if blocked else sf.reshape(-1).copy()
     return OracleQuantized(codes, flat, sf, amax[0], dtype, scale_rule, round_style,
                            orig, (mp, np_), blocked)
+
+
+def selection_errors(x, *, dtype="nvfp4", scale_rule="mse", block_scale_2d=False, amax=None, threads=None) -> np.ndarray:
+    """f32 [M, N/16, 2]: the two errors the adaptive rule compared for every 1x16 block of an
+    unpadded-or-padded bf16 input (round to nearest), first the "6" / E2M1 candidate, second
+    the "4" / INT4 one; the second wins when strictly smaller."""
+    xb, x_type = input_bits(x)
+    xp = np.ascontiguousarray(xb)
+    m, n = xp.shape
+    codes = np.zeros((m, n // 2), dtype=np.uint8)
+    sf = np.zeros((m, n // 16), dtype=np.uint8)
+    errors = np.zeros((m, n // 16, 2), dtype=np.float32)
+    amax_in = None if amax is None else np.array([amax], dtype=np.float32)
+    amax_out = np.zeros(1, dtype=np.float32)
+    rc = lib().fos_oracle_quantize_errors(
+        _ptr(xp), x_type, m, n, DTYPE_IDS[dtype], RULE_IDS[scale_rule], 0, int(block_scale_2d), 0, 0,
+        _ptr(codes), _ptr(sf), _ptr(amax_out), None if amax_in is None else _ptr(amax_in),
+        threads or default_threads(), _ptr(errors))
+    assert rc == 0
+    return errors
 
 
 def to_blocked(sf_rows: np.ndarray) -> np.ndarray:

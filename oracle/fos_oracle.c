@@ -21,8 +21,12 @@
  * Parity pins (tests/test_oracle.py): E4M3 cast vs torch's own cast over a full sweep;
  * E2M1 rounding vs the reference's threshold table over every bf16 value; the 16- and
  * 256-element summation orders vs torch.sum; closed forms for zeros / ones / rand01;
- * golden vectors written by the reference itself (tests/golden); the if4_mac golden
- * dot products for decode + scale arithmetic.
+ * golden vectors written by the reference itself (tests/golden); the dot products of the
+ * reference's MAC test benches (if4_mac/tb/*.svh, transcribed to tests/golden/if4_mac.npz)
+ * for code decode, E4M3 decode and IF4 integer blocks; Philox4x32-10 against the published
+ * Random123 known answers; the reference's stochastic-rounding known answers for NVFP4
+ * (137 / 122 / 158 / 139) and IF4 (110 / 122), which is what holds int4_sr and the IF4
+ * stochastic branch.
  * Stochastic rounding is "parity unpinned" bit-wise by construction: the reference draws
  * from torch's global generator; here the dither comes from Philox4x32-10 keyed by
  * (seed, block, candidate) so that this file and the GPU kernel agree bit-for-bit, and
@@ -324,7 +328,8 @@ static void e2m1_sr_block(const float *x, int n, uint8_t s, float inv, const uin
 /* One block (16 or 256 floats): writes fake-quantized values fq[n], whether they are
  * integer coded, and the scale byte. */
 static void quantize_block(const qctx *q, const float *x, int n, uint64_t blk0,
-                           float *fq, int *is_int, uint8_t *s_out) {
+                           float *fq, int *is_int, uint8_t *s_out, float *err2) {
+    if (err2) err2[0] = err2[1] = 0.0f;
     float bmax = 0.0f;
     for (int i = 0; i < n; ++i) { float a = fabsf(x[i]); if (a > bmax) bmax = a; }
     float xs6[256], xs4[256], f6[256], f4[256], d6[256], d4[256], u[256], inv6, inv4;
@@ -366,6 +371,7 @@ static void quantize_block(const qctx *q, const float *x, int n, uint64_t blk0,
         float err_fp = block_error(q->rule, d6, x, n);
         float err_int = block_error(q->rule, d4, x, n);
         int pick_int = err_int < err_fp;
+        if (err2) { err2[0] = err_fp; err2[1] = err_int; }
         memcpy(fq, pick_int ? f4 : f6, sizeof(float) * (size_t)n);
         *is_int = pick_int;
         *s_out = pick_int ? (uint8_t)(s6 + 128) : s6;
@@ -392,6 +398,7 @@ static void quantize_block(const qctx *q, const float *x, int n, uint64_t blk0,
     float e4 = block_error(q->rule, d4, x, n);
     float e6 = block_error(q->rule, d6, x, n);
     int pick4 = e4 < e6;
+    if (err2) { err2[0] = e6; err2[1] = e4; }
     memcpy(fq, pick4 ? f4 : f6, sizeof(float) * (size_t)n);
     *s_out = pick4 ? s4 : s6;
 }
@@ -428,10 +435,14 @@ static inline float load_x(const void *x, int x_type, int64_t i) {
     return x_type == 1 ? f16_to_f32(h) : bf16_to_f32(h);
 }
 
-int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, int dtype, int rule,
-                              int round_style, int block2d, uint64_t seed, uint64_t offset,
-                              uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
-                              int nthreads) {
+/* `errors` (may be NULL): f32 [M, N/16, 2], the two selection errors the adaptive rules
+ * compared for each 1x16 block (first candidate "6" / E2M1, second "4" / INT4; a 16x16
+ * tile repeats its pair on its 16 rows; zeros for the static rules) -- what the tests use to
+ * find blocks whose candidates nearly tie. */
+static int quantize_typed(const void *x, int x_type, int64_t M, int64_t N, int dtype, int rule,
+                          int round_style, int block2d, uint64_t seed, uint64_t offset,
+                          uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                          int nthreads, float *errors) {
     if (x_type < 0 || x_type > 2) return -1;
     if (N % 16 != 0 || (block2d && M % 16 != 0)) return -1;
     if (dtype != FOS_NVFP4 && dtype != FOS_IF4) return -1;
@@ -472,7 +483,8 @@ int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, i
             for (int64_t cb = 0; cb < bpr; ++cb) {
                 for (int i = 0; i < 16; ++i) xb[i] = load_x(x, x_type, r * N + cb * 16 + i);
                 int is_int; uint8_t s;
-                quantize_block(&q, xb, 16, (uint64_t)(r * bpr + cb), fq, &is_int, &s);
+                quantize_block(&q, xb, 16, (uint64_t)(r * bpr + cb), fq, &is_int, &s,
+                               errors ? errors + 2 * (r * bpr + cb) : NULL);
                 sf[r * bpr + cb] = s;
                 uint8_t *dst = codes + r * (N / 2) + cb * 8;
                 for (int i = 0; i < 8; ++i) {
@@ -491,8 +503,13 @@ int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, i
                     for (int i = 0; i < 16; ++i)
                         xb[16 * r + i] = load_x(x, x_type, (rt * 16 + r) * N + cb * 16 + i);
                 int is_int; uint8_t s;
-                quantize_block(&q, xb, 256, (uint64_t)(rt * 16 * bpr + cb), fq, &is_int, &s);
+                float e2[2];
+                quantize_block(&q, xb, 256, (uint64_t)(rt * 16 * bpr + cb), fq, &is_int, &s, e2);
                 for (int r = 0; r < 16; ++r) {
+                    if (errors) {
+                        errors[2 * ((rt * 16 + r) * bpr + cb)] = e2[0];
+                        errors[2 * ((rt * 16 + r) * bpr + cb) + 1] = e2[1];
+                    }
                     sf[(rt * 16 + r) * bpr + cb] = s;
                     uint8_t *dst = codes + (rt * 16 + r) * (N / 2) + cb * 8;
                     const float *f = fq + 16 * r;
@@ -506,6 +523,23 @@ int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, i
         }
     }
     return 0;
+}
+
+int fos_oracle_quantize_typed(const void *x, int x_type, int64_t M, int64_t N, int dtype, int rule,
+                              int round_style, int block2d, uint64_t seed, uint64_t offset,
+                              uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                              int nthreads) {
+    return quantize_typed(x, x_type, M, N, dtype, rule, round_style, block2d, seed, offset, codes, sf, amax_out,
+                          amax_in, nthreads, NULL);
+}
+
+/* fos_oracle_quantize_typed that also reports the selection errors (see quantize_typed). */
+int fos_oracle_quantize_errors(const void *x, int x_type, int64_t M, int64_t N, int dtype, int rule,
+                               int round_style, int block2d, uint64_t seed, uint64_t offset,
+                               uint8_t *codes, uint8_t *sf, float *amax_out, const float *amax_in,
+                               int nthreads, float *errors) {
+    return quantize_typed(x, x_type, M, N, dtype, rule, round_style, block2d, seed, offset, codes, sf, amax_out,
+                          amax_in, nthreads, errors);
 }
 
 int fos_oracle_quantize_with_amax(const uint16_t *x, int64_t M, int64_t N, int dtype, int rule,

@@ -317,3 +317,119 @@ def test_dequantize_with_f32_intermediate_matches_reference_vectors(oracle, gold
         assert np.array_equal(oracle.f32_to_bf16_bits(got), z[key + ".deq_bf16"]), key
         differs += int(not np.array_equal(got.view(np.uint32), other.view(np.uint32)))
     assert differs >= 4  # the option matters on the IF4 / out-of-range MXFP4 cases
+
+
+def test_philox4x32_10_known_answers(oracle):
+    """The three published Random123 known-answer vectors for Philox4x32 with 10 rounds
+    (counter, key -> output): zeros, all ones, and the digits of pi."""
+    L = oracle.lib()
+    cases = (
+        ((0, 0, 0, 0), (0, 0), (0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8)),
+        ((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2, (0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD)),
+        ((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0),
+         (0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1)),
+    )
+    for ctr, key, want in cases:
+        c = np.array(ctr, dtype=np.uint32)
+        k = np.array(key, dtype=np.uint32)
+        out = np.zeros(4, dtype=np.uint32)
+        L.fos_oracle_philox4x32_10(c.ctypes.data, k.ctypes.data, out.ctypes.data)
+        assert tuple(int(v) for v in out) == want
+
+
+def test_if4_stochastic_rounding_known_answers(oracle):
+    """IF4 + MSE under the stochastic styles (the INT4 dither and the IF4 stochastic branch):
+    the reference's known answers 110 / 122 (unbiased) +- 5 % on randn 1024^2
+    (tests/test_quantize.py:321,360-372)."""
+    g = torch.Generator("cpu").manual_seed(0)
+    x = torch.randn(1024, 1024, generator=g).bfloat16()
+    xf = x.float().numpy()
+    for style, expect in (("stochastic", 110), ("stochastic_unbiased", 122)):
+        for seed in (1234, 99):
+            q = oracle.quantize(x, dtype="if4", scale_rule="mse", round_style=style, seed=seed)
+            deq = oracle.dequantize(q.values, q.scale_rows, q.amax, dtype="if4", scale_rule="mse", round_style=style)
+            deq = torch.from_numpy(deq).bfloat16().float().numpy()
+            dist = float(np.sqrt(((deq - xf) ** 2).sum()))
+            assert abs(dist - expect) / expect < 0.05, (style, seed, dist)
+        # both kinds of block occur, so the integer branch's dither is exercised
+        frac_int = float((q.scale_factors >= 128).mean())
+        assert 0.05 < frac_int < 0.95
+
+
+def _mac_tree_sum(lanes):
+    stage = [np.float32(v) for v in lanes]
+    while len(stage) > 1:
+        nxt = [np.float32(stage[i] + stage[i + 1]) for i in range(0, len(stage) - 1, 2)]
+        if len(stage) % 2:
+            nxt.append(stage[-1])
+        stage = nxt
+    return stage[0]
+
+
+@pytest.mark.parametrize("fmt", ["nvfp4", "if4"])
+def test_decode_and_scale_against_mac_known_answers(oracle, golden_dir, fmt):
+    """The reference's MAC test benches hold three dot products of K = 160 each for NVFP4 and
+    IF4 operands with their expected fp32 bit patterns (if4_mac/tb/nvfp4_mac_golden_ref.svh:1119-1121,
+    if4_mac/tb/if4_mac_golden_ref.svh; arithmetic of if4_mac/scripts/gen_golden_ref.py:164-209:
+    fp16 product of the two decoded values times the fp32 product of the two decoded scales,
+    one fp32 accumulator per lane, pairwise tree at the end).  Here the operands go through
+    the oracle's dequantize (code decode, E4M3 decode, IF4 integer blocks with bit 7 of the
+    scale byte) and the products are accumulated as the MAC does.  NVFP4 is bit-exact: value
+    x scale is exact in both formulations.  An IF4 integer block carries 6/7 in the decoded
+    value here and in the scale product there, so that file agrees to fp32 rounding only.
+    The MAC reads the scale byte 0x7F as 448 (gen_golden_ref.py:76-79), the float8_e4m3fn
+    cast never produces that byte: it is mapped to 0x7E before decoding."""
+    d = np.load(os.path.join(golden_dir, "if4_mac.npz"))
+    first, a, w = d[f"{fmt}.first"], d[f"{fmt}.a"], d[f"{fmt}.w"]
+    a_sf, w_sf = d[f"{fmt}.a_sf"].copy(), d[f"{fmt}.w_sf"].copy()
+    for sf in (a_sf, w_sf):
+        sf[(sf & 0x7F) == 0x7F] -= 1
+    n = first.size
+
+    def dequant(codes, sf):
+        # one 1x16 block per cycle: rows = cycles, 16 columns (packed low nibble first)
+        packed = (codes[:, 0::2] | (codes[:, 1::2] << 4)).astype(np.uint8)
+        div = 6.0 * 448.0
+        return oracle.dequantize(packed, sf.reshape(n, 1), div, dtype=fmt, scale_rule="static_6", f32_intermediate=True)
+
+    da, dw = dequant(a, a_sf), dequant(w, w_sf)
+    # amax == divisor, so the tensor scale is exactly 1 (the products below 2^12 * 2688 are exact)
+    got = []
+    acc = np.zeros(16, dtype=np.float32)
+    for i in range(n):
+        if first[i] and i:
+            got.append(_mac_tree_sum(acc))
+            acc = np.zeros(16, dtype=np.float32)
+        prod = (da[i].astype(np.float64) * dw[i].astype(np.float64)).astype(np.float32)
+        acc = (acc + prod).astype(np.float32)
+    got = np.array(got, dtype=np.float32)
+    want = d[f"{fmt}.expected"].view(np.float32)
+    assert got.size == 3
+    if fmt == "nvfp4":
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (got, want)
+    else:
+        assert np.allclose(got, want, rtol=2e-6, atol=0.0), (got, want)
+        assert int((d["if4.a_sf"] >= 128).sum()) > 5  # integer blocks are present
+
+
+def test_near_tie_fixture_holds_near_ties(oracle, golden_dir):
+    """tests/golden/near_ties.npz (written by make_near_ties.py): every stored block's two
+    selection errors differ, by at most 2e-4 relative, and at least a third of them by at most
+    2e-6 -- the inputs on which an approximate decision would go wrong."""
+    d = np.load(os.path.join(golden_dir, "near_ties.npz"))
+    cases = sorted(k[:-2] for k in d.files if k.endswith(".x"))
+    assert len(cases) == 7
+    for case in cases:
+        parts = case.split(".")
+        dtype, two_d, given = parts[0], parts[1] == "2d", len(parts) == 3
+        x, amax = d[case + ".x"], float(d[case + ".amax"][0])
+        e = oracle.selection_errors(x, dtype=dtype, block_scale_2d=two_d, amax=amax if given else None)
+        unit = 16 if two_d else 1
+        ea, eb = e[::unit, :, 0].astype(np.float64).ravel()[1:], e[::unit, :, 1].astype(np.float64).ravel()[1:]
+        live = np.maximum(ea, eb) > 0
+        assert live.sum() >= 40, case
+        rel = np.abs(ea - eb)[live] / np.maximum(ea, eb)[live]
+        assert (rel > 0).all() and (rel <= 2e-4).all(), case
+        assert (rel <= 2e-6).mean() > 0.25, case
+        if not given:
+            assert float(oracle.bf16_bits_to_f32(x).max()) == amax == 8.0

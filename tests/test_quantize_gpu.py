@@ -54,7 +54,12 @@ def test_matches_reference_vectors(path):
         assert np.array_equal(u8(q.values), d[k + ".values"]), k
         assert np.array_equal(u8(q.scale_factors).reshape(-1), d[k + ".sf"].reshape(-1)), k
         if k + ".deq_bf16" in d.files:
-            assert np.array_equal(bits16(fos.dequantize(q)), d[k + ".deq_bf16"]), k
+            want = d[k + ".deq_bf16"]
+            assert np.array_equal(bits16(fos.dequantize(q)), want), k
+            # the fused quantize -> dequantize kernel against the reference's own dequantized bits
+            r = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype=dt, scale_rule=rule, block_scale_2d=(dim == "2d"),
+                                                              pseudo_quantize=True))
+            assert r.shape == x.shape and np.array_equal(bits16(r), want[: x.shape[0], : x.shape[1]]), k + " (pseudo)"
 
 
 def test_fp32_and_fp16_inputs_match_reference_vectors(golden_dir):
@@ -186,6 +191,26 @@ def test_if4_mse_fast_path_inputs(oracle, two_d):
     given = float(np.float32(float(x.abs().max()) * 1.2345678))
     q = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype="if4", block_scale_2d=two_d, kwargs={"amax": torch.tensor(given, device="cuda")}))
     assert_same_quantization(q, oracle.quantize(x, dtype="if4", block_scale_2d=two_d, amax=given), "24-bit maximum")
+
+
+def test_near_ties_take_the_exact_decision(oracle, golden_dir):
+    """Blocks and tiles whose two candidate errors differ by a few units in the last place (found
+    by a CPU search, tests/golden/make_near_ties.py): the kernels' certified shortcut must hand
+    every one of them to the exact evaluation.  4/6 and IF4, 1-D and 2-D, tensor maximum from the
+    data and a caller-supplied 24-bit maximum; also under the fused pseudo-quantize epilogue."""
+    d = np.load(os.path.join(golden_dir, "near_ties.npz"))
+    for case in sorted(k[:-2] for k in d.files if k.endswith(".x")):
+        parts = case.split(".")
+        dtype, two_d, given = parts[0], parts[1] == "2d", len(parts) == 3
+        x = torch.from_numpy(d[case + ".x"].view(np.int16).copy()).view(torch.bfloat16)
+        amax = float(d[case + ".amax"][0])
+        kwargs = {"amax": torch.tensor(amax, device="cuda")} if given else {}
+        q = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype=dtype, scale_rule="mse", block_scale_2d=two_d, kwargs=kwargs))
+        ref = oracle.quantize(x, dtype=dtype, scale_rule="mse", block_scale_2d=two_d, amax=amax if given else None)
+        assert_same_quantization(q, ref, case)
+        if dtype == "nvfp4":
+            r = fos.quantize(x.cuda(), fos.QuantizationConfig(scale_rule="mse", block_scale_2d=two_d, pseudo_quantize=True, kwargs=kwargs))
+            assert torch.equal(r.view(torch.int16), fos.dequantize(q, dtype=torch.bfloat16).view(torch.int16)), case
 
 
 def test_negative_zero_inputs(oracle):
@@ -337,6 +362,11 @@ def test_stochastic_rounding_known_answers():
         q = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, round_style=style))
         dist = float(torch.dist(fos.dequantize(q).float(), x.float()))
         assert abs(dist - expect) / expect < 0.05, (rule, style, dist)
+    # IF4 + MSE: 110 / 122 (tests/test_quantize.py:321)
+    for style, expect in (("stochastic", 110), ("stochastic_unbiased", 122)):
+        q = fos.quantize(x, fos.QuantizationConfig(dtype="if4", scale_rule="mse", round_style=style))
+        dist = float(torch.dist(fos.dequantize(q).float(), x.float()))
+        assert abs(dist - expect) / expect < 0.05, ("if4", style, dist)
     cfg = fos.QuantizationConfig(scale_rule="static_6", round_style="stochastic")
     mean_err = torch.stack([(fos.dequantize(fos.quantize(x, cfg), torch.float32) - x.float()) for _ in range(4)]).mean()
     assert abs(float(mean_err)) < 1e-3
