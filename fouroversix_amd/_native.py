@@ -28,6 +28,7 @@ EXPORTS = (
     "fos_quantize_workspace_bytes",
     "fos_amax",
     "fos_quantize",
+    "fos_quantize_static",
     "fos_pseudo_quantize",
     "fos_transform",
     "fos_gemm_nvfp4",
@@ -74,6 +75,8 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, i32,
                                vp, vp, vp, i32, vp, sz, vp]
     L.fos_quantize.restype = i32
+    L.fos_quantize_static.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, i32, vp, vp, vp, i32, vp]
+    L.fos_quantize_static.restype = i32
     L.fos_pseudo_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i32, vp, sz, vp]
     L.fos_pseudo_quantize.restype = i32
     L.fos_transform.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, i64, vp, vp, sz, vp]

@@ -9,11 +9,18 @@
 // This file holds pass 1, the C entry points, and the pass-2 instantiations that use only
 // the operation-by-operation form (IF4, stochastic rounding); NVFP4 round-to-nearest is
 // instantiated in fos_quantize_fast.hip.
+#include <atomic>
 #include <cstdlib>
 
 #include "fos_quantize_kernel.h"
 
 namespace fos {
+
+// Pass-1 partials of fos_quantize_static: the one buffer the quantizer needs besides its
+// inputs and outputs, held by every GPU the library runs on until the process ends.  In
+// host code this name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kStaticScratchBytes = 2 * kMaxPartials * sizeof(uint32_t);
+static __device__ __align__(256) uint32_t scratch[2 * kMaxPartials];
 
 // ---------------------------------------------------------------------------------------
 // pass 1: per-workgroup max |x| as an integer max over the magnitude bits, plus a flag
@@ -408,4 +415,29 @@ extern "C" int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int6
     if (!out) return FOS_E_NULL_POINTER;
     return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, 0, 0, FOS_SF_LINEAR, nullptr, nullptr,
                          amax, amax_is_input, workspace, workspace_bytes, stream, static_cast<uint16_t *>(out), ldo);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+}  // namespace
+
+extern "C" int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                                   int dtype, int rule, int round_style, int block2d,
+                                   uint64_t seed, uint64_t offset, int sf_layout,
+                                   uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                                   fos_stream_t stream) {
+    if (rows <= 0 || cols <= 0) return FOS_E_BAD_SHAPE;
+    if (fos_quantize_workspace_bytes(rows, cols) > kStaticScratchBytes) return FOS_E_WORKSPACE;  // beyond the built-in scratch
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FOS_E_LAUNCH;
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // every GPU holds its own copy of the array at its own address
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return FOS_E_LAUNCH;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, seed, offset, sf_layout, codes, sf,
+                         amax, amax_is_input, ptr, kStaticScratchBytes, stream, nullptr, 0);
 }

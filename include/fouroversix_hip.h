@@ -2,9 +2,9 @@
  * fouroversix_hip.h -- C ABI of the gfx950 (MI355X) quantize / FP4-matmul library.
  *
  * Plain pointers and sizes only; every pointer except the error strings is DEVICE memory.
- * All entry points are asynchronous on the given HIP stream, never synchronise, and keep
- * no mutable global state, so they are safe to call from several host threads on
- * different streams.  Return value: 0 on success, a negative FOS_E_* code otherwise
+ * All entry points are asynchronous on the given HIP stream and never synchronise.  Apart
+ * from fos_quantize_static (which says so below) they keep no mutable state between calls,
+ * so they are safe to call from several host threads on different streams.  Return value: 0 on success, a negative FOS_E_* code otherwise
  * (nothing is launched when an argument check fails).
  *
  * Each function names the interface of the reference (mit-han-lab/fouroversix, paths
@@ -104,6 +104,24 @@ int fos_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t 
                  uint64_t seed, uint64_t offset, int sf_layout,
                  uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
                  void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * fos_quantize without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  The pass-1 partial maxima go to an 8 KiB array that the
+ * library holds in every GPU's memory for the life of the process; the call allocates and
+ * frees nothing.  The array's address is looked up on the first call on each device (with
+ * that device current), so make that first call outside a stream capture.  Every shape
+ * fos_quantize accepts fits (its workspace never exceeds the array); a shape that would
+ * not returns FOS_E_WORKSPACE.  All calls on one GPU share the array: calls that overlap
+ * in time on one GPU (different streams, concurrently replayed graphs) race on it and must
+ * be serialised by the caller.  Results are those of fos_quantize.
+ */
+int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                        int dtype, int rule, int round_style, int block2d,
+                        uint64_t seed, uint64_t offset, int sf_layout,
+                        uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                        fos_stream_t stream);
 
 /*
  * Pre-transform of the training-side quantize options: y = x^T (transpose != 0) and / or
