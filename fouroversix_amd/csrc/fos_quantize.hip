@@ -23,9 +23,8 @@ constexpr size_t kStaticScratchBytes = 2 * kMaxPartials * sizeof(uint32_t);
 static __device__ __align__(256) uint32_t scratch[2 * kMaxPartials];
 
 // ---------------------------------------------------------------------------------------
-// pass 1: per-workgroup max |x| as an integer max over the magnitude bits, plus a flag
-// telling whether any element is a negative zero (bit pattern 0x8000: the smallest signed
-// 16-bit integer, so a packed signed minimum finds it)
+// pass 1: per-workgroup max |x| as an integer max over the magnitude bits (the second
+// word of each partial pair is reserved and written as zero)
 // ---------------------------------------------------------------------------------------
 
 template <bool IS_BF16>
@@ -42,7 +41,7 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
     __shared__ uint32_t smem[4];
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
-    uint32_t m = 0, z = 0;
+    uint32_t m = 0;
     constexpr int U = 8;
     for (; i + (U - 1) * stride < n_vec; i += U * stride) {
         uint4 v[U];
@@ -54,7 +53,6 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
             m = pk_max_u16(m, v[u].y & 0x7fff7fffu);
             m = pk_max_u16(m, v[u].z & 0x7fff7fffu);
             m = pk_max_u16(m, v[u].w & 0x7fff7fffu);
-            z = pk_min_i16(pk_min_i16(z, v[u].x), pk_min_i16(v[u].y, pk_min_i16(v[u].z, v[u].w)));
         }
     }
     for (; i < n_vec; i += stride) {
@@ -63,14 +61,12 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
         m = pk_max_u16(m, v.y & 0x7fff7fffu);
         m = pk_max_u16(m, v.z & 0x7fff7fffu);
         m = pk_max_u16(m, v.w & 0x7fff7fffu);
-        z = pk_min_i16(pk_min_i16(z, v.x), pk_min_i16(v.y, pk_min_i16(v.z, v.w)));
     }
     uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
     mm = block_max_u32(mm, smem);
-    const uint32_t zz = block_max_u32(((z & 0xffffu) == 0x8000u || (z >> 16) == 0x8000u) ? 1u : 0u, smem);
     if (threadIdx.x == 0) {
         partials[2 * blockIdx.x] = mag16_to_f32_bits<IS_BF16>(mm);
-        partials[2 * blockIdx.x + 1] = zz;
+        partials[2 * blockIdx.x + 1] = 0u;
     }
 }
 
@@ -80,20 +76,18 @@ __global__ __launch_bounds__(kThreads) void amax_rows_kernel(const uint16_t *__r
                                                              int64_t cols, int64_t ld,
                                                              uint32_t *__restrict__ partials) {
     __shared__ uint32_t smem[4];
-    uint32_t m = 0, z = 0;
+    uint32_t m = 0;
     for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
         const uint16_t *row = x + r * ld;
         for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
-            const uint32_t h = row[c], v = h & 0x7fffu;
+            const uint32_t v = row[c] & 0x7fffu;
             m = m > v ? m : v;
-            z |= (h == 0x8000u) ? 1u : 0u;
         }
     }
     m = block_max_u32(m, smem);
-    z = block_max_u32(z, smem);
     if (threadIdx.x == 0) {
         partials[2 * blockIdx.x] = mag16_to_f32_bits<IS_BF16>(m);
-        partials[2 * blockIdx.x + 1] = z;
+        partials[2 * blockIdx.x + 1] = 0u;
     }
 }
 
@@ -102,11 +96,10 @@ __global__ __launch_bounds__(kThreads) void amax_flat_f32_kernel(const uint4 *__
                                                                  uint32_t *__restrict__ partials) {
     __shared__ uint32_t smem[4];
     const int64_t stride = (int64_t)gridDim.x * kThreads;
-    uint32_t m = 0, z = 0;
+    uint32_t m = 0;
     auto take = [&](uint32_t u) {
         const uint32_t v = u & 0x7fffffffu;
         m = m > v ? m : v;
-        z |= (u == 0x80000000u) ? 1u : 0u;
     };
     constexpr int U = 8;
     int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
@@ -122,10 +115,9 @@ __global__ __launch_bounds__(kThreads) void amax_flat_f32_kernel(const uint4 *__
         take(v.x), take(v.y), take(v.z), take(v.w);
     }
     m = block_max_u32(m, smem);
-    z = block_max_u32(z, smem);
     if (threadIdx.x == 0) {
         partials[2 * blockIdx.x] = m;
-        partials[2 * blockIdx.x + 1] = z;
+        partials[2 * blockIdx.x + 1] = 0u;
     }
 }
 
@@ -134,20 +126,18 @@ __global__ __launch_bounds__(kThreads) void amax_rows_f32_kernel(const uint32_t 
                                                                  int64_t cols, int64_t ld,
                                                                  uint32_t *__restrict__ partials) {
     __shared__ uint32_t smem[4];
-    uint32_t m = 0, z = 0;
+    uint32_t m = 0;
     for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
         const uint32_t *row = x + r * ld;
         for (int64_t c = threadIdx.x; c < cols; c += kThreads) {
-            const uint32_t u = row[c], v = u & 0x7fffffffu;  // magnitudes order like their bit patterns
+            const uint32_t v = row[c] & 0x7fffffffu;  // magnitudes order like their bit patterns
             m = m > v ? m : v;
-            z |= (u == 0x80000000u) ? 1u : 0u;
         }
     }
     m = block_max_u32(m, smem);
-    z = block_max_u32(z, smem);
     if (threadIdx.x == 0) {
         partials[2 * blockIdx.x] = m;
-        partials[2 * blockIdx.x + 1] = z;
+        partials[2 * blockIdx.x + 1] = 0u;
     }
 }
 

@@ -24,7 +24,7 @@ struct QuantParams {
     int64_t rows_p, cols_p;      // padded output extents
     uint8_t *codes;              // [rows_p, cols_p / 2]
     uint8_t *sf;                 // rows_p * cols_p / 16 bytes
-    const uint32_t *partials;    // pass-1 results, pairs {max|x| as f32 bits, 1 if a -0.0 was seen}
+    const uint32_t *partials;    // pass-1 results, pairs {max|x| as f32 bits, reserved}
     int n_partials;              // number of pairs; 0 = `partials` points at a caller-supplied f32 amax;
                                  // -1 = no pass 1 ran: pass 2 scans the (small, contiguous, aligned) input itself
     float *amax_out;             // written by workgroup 0 when not null
@@ -74,21 +74,17 @@ FOS_DEVICE uint32_t block_max_u32(uint32_t v, uint32_t *smem /* >= 4 words */) {
     return r;
 }
 
-// Tensor-wide results of pass 1, valid in every thread: bits of max|x| and whether the
-// input may contain a negative zero (unknown, hence assumed, for a caller-supplied amax).
-FOS_DEVICE void reduce_partials(const QuantParams &p, uint32_t *smem, uint32_t &amax_bits, bool &maybe_negzero) {
-    if (p.n_partials == 0) {
-        amax_bits = p.partials[0];
-        maybe_negzero = true;
-        return;
-    }
+// Tensor-wide result of pass 1, valid in every thread: the bits of max|x|.  (The second word
+// of each partial pair is reserved and ignored.)
+FOS_DEVICE uint32_t reduce_partials(const QuantParams &p, uint32_t *smem) {
+    if (p.n_partials == 0) return p.partials[0];
     if (p.n_partials < 0) {
         // small contiguous input: no pass 1 was launched and every workgroup scans the
         // whole tensor itself (rows * cols / 8 aligned 128-bit vectors, 128 KiB out of L2 at
         // most), which costs less than a launch and its dependency
         const uint4 *v4 = reinterpret_cast<const uint4 *>(p.x);
         const int n_vec = (int)((p.rows * p.cols) >> 3);
-        uint32_t m = 0, z = 0;
+        uint32_t m = 0;
         constexpr int U = 16;  // loads in flight per thread: the scan is latency-bound
         for (int base = 0; base < n_vec; base += U * kThreads) {
             uint4 v[U];
@@ -103,22 +99,17 @@ FOS_DEVICE void reduce_partials(const QuantParams &p, uint32_t *smem, uint32_t &
                 m = pk_max_u16(m, v[u].y & 0x7fff7fffu);
                 m = pk_max_u16(m, v[u].z & 0x7fff7fffu);
                 m = pk_max_u16(m, v[u].w & 0x7fff7fffu);
-                z = pk_min_i16(pk_min_i16(z, v[u].x), pk_min_i16(v[u].y, pk_min_i16(v[u].z, v[u].w)));
             }
         }
         const uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
-        amax_bits = block_max_u32(mm, smem) << 16;  // bf16 magnitude bits -> fp32 bits
-        maybe_negzero = block_max_u32(((z & 0xffffu) == 0x8000u || (z >> 16) == 0x8000u) ? 1u : 0u, smem) != 0;
-        return;
+        return block_max_u32(mm, smem) << 16;  // bf16 magnitude bits -> fp32 bits
     }
-    uint32_t m = 0, z = 0;
+    uint32_t m = 0;
     for (int i = threadIdx.x; i < p.n_partials; i += kThreads) {
-        const uint2 v = reinterpret_cast<const uint2 *>(p.partials)[i];
-        m = m > v.x ? m : v.x;
-        z |= v.y;
+        const uint32_t v = p.partials[2 * i];
+        m = m > v ? m : v;
     }
-    amax_bits = block_max_u32(m, smem);
-    maybe_negzero = block_max_u32(z, smem) != 0;
+    return block_max_u32(m, smem);
 }
 
 // ---------------------------------------------------------------------------------------

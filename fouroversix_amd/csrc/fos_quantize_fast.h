@@ -21,8 +21,8 @@
 //
 // A negative zero in the input must encode as +0 (the reference multiplies by sign(x),
 // and sign(-0) = 0) while a small negative value that rounds to zero keeps its sign; the
-// hardware convert keeps the sign in both cases, so when pass 1 saw a -0.0 anywhere the
-// block values are first canonicalised with x + 0.
+// hardware convert keeps the sign in both cases, so the scaled value is formed as
+// fma(x, inv, +0): the product of a non-zero x is unchanged and (-0) * inv + 0 is +0.
 #pragma once
 
 #include <type_traits>
@@ -35,7 +35,7 @@ struct FastLutEntry {
     float inv;       // 1 / (dec * s)                       (0 for s == 0)
     float d1;        // RN((s * amax) / errdiv)             factor for fq in {.5, 1, 2, 4}
     uint32_t delta;  // bits((s * amax) / 1024) - bits(d1)  added for fq in {1.5, 3, 6}
-    uint32_t pad;
+    float hh;        // d1 * d1: weight of this scale's sum of squares in the shortcut
 };
 
 // Entry for scale byte `s` (0..127); built with the reference's operations.
@@ -46,9 +46,12 @@ FOS_DEVICE FastLutEntry make_lut_entry(uint32_t s, const QuantConsts &k) {
     const float g = sf * k.amax;
     e.d1 = g / k.errdiv;
     e.delta = f2u((1.5f * g) / k.errdiv) - f2u(e.d1);  // 1.5 g is exact; with errdiv = 1536 this is g / 1024
-    e.pad = 0;
+    e.hh = e.d1 * e.d1;
     return e;
 }
+
+// Scaled value of one element: x * inv with the sign of a zero product dropped.
+FOS_DEVICE float scaled(float x, float inv) { return __builtin_fmaf(x, inv, 0.0f); }
 
 // x / y for a constant y with r = RN(1/y); equals IEEE division whenever the quotient is
 // a normal number.
@@ -104,11 +107,11 @@ template <bool TWO_D>
 FOS_DEVICE int shortcut_compare(float SA, float hA, float SB, float hB) {
     constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
     constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
-    const float EA = hA * SA, EB = hB * SB;
-    const float tA = hA * __builtin_fmaf(k1, SA, k0);
-    const float tB = hB * __builtin_fmaf(k1, SB, k0);
-    if (EB + tB < EA - tA) return 1;
-    if (EB - tB > EA + tA) return -1;
+    // |EB - EA| against tA + tB (the differences and sums round within a few 2^-24 of
+    // quantities that the tolerances exceed by 2^10)
+    const float D = __builtin_fmaf(hB, SB, -(hA * SA));
+    const float T = __builtin_fmaf(hA, __builtin_fmaf(k1, SA, k0), hB * __builtin_fmaf(k1, SB, k0));
+    if (fabsf(D) > T) return D < 0.0f ? 1 : -1;
     return 0;
 }
 
@@ -189,7 +192,7 @@ FOS_DEVICE uint32_t tie_violations(uint32_t a, uint32_t b) {
 // Exact selection of a block whose shortcut was inconclusive: the residuals of both
 // candidates from their packed codes, with the reference's rounding and order.
 template <int RULE, bool TWO_D>
-__device__ __attribute__((noinline)) bool exact_pick_b(Block16 blk, bool canon, uint32_t a0, uint32_t a1, uint32_t b0,
+__device__ __attribute__((noinline)) bool exact_pick_b(Block16 blk, uint32_t a0, uint32_t a1, uint32_t b0,
                                                        uint32_t b1, FastLutEntry A, FastLutEntry B) {
     uint32_t w[8];
 #pragma unroll
@@ -202,8 +205,7 @@ __device__ __attribute__((noinline)) bool exact_pick_b(Block16 blk, bool canon, 
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int idx = l + 8 * h;
-            float x = block_element(w, idx);
-            if (canon) x = x + 0.0f;
+            const float x = block_element(w, idx);  // the sign of a zero does not reach |d| or d * d
             const float dA = candidate_residual(e2m1_value((uint32_t)(ca >> (4 * idx)) & 0xfu), A, x);
             const float dB = candidate_residual(e2m1_value((uint32_t)(cb >> (4 * idx)) & 0xfu), B, x);
             e[0][h] = RULE == FOS_RULE_MSE ? dA * dA : fabsf(dA);
@@ -278,7 +280,7 @@ __device__ __attribute__((noinline)) BlockOut generic_block_sr(Block16 blk, Quan
 // One 1x16 block, NVFP4, any rule, round to nearest or (SR) a stochastic style; falls
 // back by itself.  `blkid` = row * (cols_p / 16) + block column keys the dither.
 template <int RULE, bool TWO_D, bool SR>
-FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
+FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq,
                                               bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
                                               uint64_t blkid) {
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
@@ -288,10 +290,6 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
         for (int i = 0; i < 8; ++i) {
             x[2 * i] = u2f(blk.w[i] << 16);
             x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
-        }
-        if (canon) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) x[i] = x[i] + 0.0f;
         }
         float bmax = 0.0f;
 #pragma unroll
@@ -322,7 +320,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 // rounded value may lie from the scaled one
                 float xa[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) xa[i] = x[i] * A.inv;
+                for (int i = 0; i < 16; ++i) xa[i] = scaled(x[i], A.inv);
                 const Philox4 pA = block_philox(seed, offset, blkid);
                 uint32_t a0, a1;
                 sr_pack16(xa, pA, a0, a1);
@@ -330,7 +328,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 const FastLutEntry B = lut[s4];
                 float xb[16];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) xb[i] = x[i] * B.inv;
+                for (int i = 0; i < 16; ++i) xb[i] = scaled(x[i], B.inv);
                 const Philox4 pB = second_candidate_words(pA);
                 uint32_t b0, b1;
                 sr_pack16(xb, pB, b0, b1);
@@ -352,7 +350,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                         SA = row16_sum_lane0(SA);
                         SB = row16_sum_lane0(SB);
                     }
-                    const int cmp = shortcut_compare<TWO_D>(SA, A.d1 * A.d1, SB, B.d1 * B.d1);
+                    const int cmp = shortcut_compare<TWO_D>(SA, A.hh, SB, B.hh);
                     certain = cmp != 0;
                     pickB = cmp > 0;
                 }
@@ -360,7 +358,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
                     if (TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                     if (tie) pickB = false;
-                    else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                    else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
                     else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // e.g. the unbiased style's divisor
                 }
                 return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
@@ -369,8 +367,8 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 uint32_t c0 = 0, c1 = 0;
                 static_for<0, 4>([&](auto jc) {
                     constexpr int j = decltype(jc)::value;
-                    c0 = pack_fp4<j>(c0, x[2 * j] * A.inv, x[2 * j + 1] * A.inv);
-                    c1 = pack_fp4<j>(c1, x[8 + 2 * j] * A.inv, x[9 + 2 * j] * A.inv);
+                    c0 = pack_fp4<j>(c0, scaled(x[2 * j], A.inv), scaled(x[2 * j + 1], A.inv));
+                    c1 = pack_fp4<j>(c1, scaled(x[8 + 2 * j], A.inv), scaled(x[9 + 2 * j], A.inv));
                 });
                 return BlockOut{c0, c1, s6};
             }
@@ -379,8 +377,8 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
             float SA = 0.0f, SB = 0.0f;
             static_for<0, 8>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                const float xa0 = x[2 * j] * A.inv, xa1 = x[2 * j + 1] * A.inv;
-                const float xb0 = x[2 * j] * B.inv, xb1 = x[2 * j + 1] * B.inv;
+                const float xa0 = scaled(x[2 * j], A.inv), xa1 = scaled(x[2 * j + 1], A.inv);
+                const float xb0 = scaled(x[2 * j], B.inv), xb1 = scaled(x[2 * j + 1], B.inv);
                 if (j < 4) {
                     a0 = pack_fp4<(j & 3)>(a0, xa0, xa1);
                     b0 = pack_fp4<(j & 3)>(b0, xb0, xb1);
@@ -404,7 +402,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     SA = row16_sum_lane0(SA);
                     SB = row16_sum_lane0(SB);
                 }
-                const int cmp = shortcut_compare<TWO_D>(SA, A.d1 * A.d1, SB, B.d1 * B.d1);
+                const int cmp = shortcut_compare<TWO_D>(SA, A.hh, SB, B.hh);
                 certain = cmp != 0;
                 pickB = cmp > 0;
             }
@@ -416,7 +414,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                 }
                 if (tie) pickB = false;
-                else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, canon, a0, a1, b0, b1, A, B);
+                else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
                 else return generic_block<RULE, TWO_D>(blk, k);
             }
             return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
@@ -445,7 +443,7 @@ __device__ __attribute__((noinline)) BlockOut generic_block_if4(Block16 blk, Qua
 }
 
 template <bool TWO_D>
-FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts &k, float enc, float rq, bool canon,
+FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts &k, float enc, float rq,
                                            bool in_range, const FastLutEntry *lut) {
     if (in_range) {
         float x[16];
@@ -453,10 +451,6 @@ FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts
         for (int i = 0; i < 8; ++i) {
             x[2 * i] = u2f(blk.w[i] << 16);
             x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
-        }
-        if (canon) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) x[i] = x[i] + 0.0f;
         }
         float bmax = 0.0f;
 #pragma unroll
@@ -471,7 +465,7 @@ FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts
             float SA = 0.0f, SB = 0.0f;
             static_for<0, 8>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
-                const float x0 = x[2 * j] * A.inv, x1 = x[2 * j + 1] * A.inv;
+                const float x0 = scaled(x[2 * j], A.inv), x1 = scaled(x[2 * j + 1], A.inv);
                 if (j < 4) a0 = pack_fp4<(j & 3)>(a0, x0, x1);
                 else a1 = pack_fp4<(j & 3)>(a1, x0, x1);
                 const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);

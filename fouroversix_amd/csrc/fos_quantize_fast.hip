@@ -45,9 +45,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     __shared__ uint32_t sf_tile[2][128];
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
-    uint32_t amax_bits;
-    bool maybe_negzero;
-    reduce_partials(p, red, amax_bits, maybe_negzero);
+    const uint32_t amax_bits = reduce_partials(p, red);
     QuantConsts k;
     k.amax = u2f(amax_bits);
     k.enc = p.c / k.amax;
@@ -74,7 +72,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         for (int h = 0; h < 2; ++h) {
             const int rr = h * 64 + wave * 16 + (lane & 15);
             const int64_t r = tile_y * 128 + rr;
-            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, SR>(t.b[h], k, enc_fast, rq, maybe_negzero, in_range, lut,
+            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, SR>(t.b[h], k, enc_fast, rq, in_range, lut,
                                                                           p.seed, p.offset, (uint64_t)(r * sf_cols + cb));
             if (PSEUDO) {
                 uint32_t w[8];
@@ -115,20 +113,46 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 }
 
 
-// 1x16 blocks, row-contiguous mapping: lane -> block column (lane & 15) of row (lane >> 4)
-// within the wavefront's 4 rows; workgroup tile 128 rows x 256 columns; workgroups stride
-// over the tiles so that the per-workgroup setup (tensor maximum, scale table) is paid
-// once for several tiles.  FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
+// Buffer resource (V#) over [base, base + bytes): raw 32-bit byte offsets, out-of-range
+// loads return zero.
+typedef __amdgpu_buffer_rsrc_t BufferRsrc;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+// 1x16 blocks, row-contiguous mapping.  Workgroup tile: 128 rows x 256 columns, walked in
+// eight steps; in a step a wavefront covers 4 rows x 16 blocks (lane -> block column lane & 15
+// of row lane >> 4), i.e. 512 contiguous bytes per row.  Wavefront w owns rows
+// 32 q + 8 w + 4 h + i (q = 0..3, h = 0..1: step g = 2 q + h; i = lane >> 4) of the tile: in the
+// 128x4 scale layout the scales of rows r, r + 32, r + 64, r + 96 share a 16-byte unit, so these
+// 32 rows' scales are 128 contiguous bytes of each of the tile's four scale tiles, which the
+// wavefront assembles in its own 512 bytes of LDS and writes itself -- the loop has no
+// workgroup barrier.  Workgroups stride over the tiles (the setup -- tensor maximum, scale
+// table -- is paid once) and the loads run three steps ahead, across tile boundaries.
+// Input, codes and the pseudo-quantize output go through buffer instructions: a
+// wave-uniform descriptor per tile, a per-lane 32-bit offset that is the same for every
+// tile, and a uniform offset per step, so the loop holds no 64-bit address arithmetic.  A
+// ragged tile's descriptor ends with the tensor's last row and lanes past the last column
+// get an offset beyond it: both read zeros, which is the padding the reference adds.
+// FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
+struct RowsTile {
+    BufferRsrc rx, rcodes, rout;
+    uint32_t x_off;      // this lane's offset into rx (beyond the descriptor for a lane past the last column)
+    int64_t row_base;    // first row of the tile
+    int64_t cb;          // this lane's block column in the tensor
+    uint32_t tile_y, tile_x;
+};
+
 template <int RULE, bool FULL, bool PSEUDO, bool SR>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
-    __shared__ uint32_t sf_stage[2][4 * 128];  // 4 scale tiles of 512 bytes, double-buffered
+    __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][128];  // per wavefront: 4 scale tiles x 128 bytes
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
-    uint32_t amax_bits;
-    bool maybe_negzero;
-    reduce_partials(p, red, amax_bits, maybe_negzero);
+    const uint32_t amax_bits = reduce_partials(p, red);
     QuantConsts k;
     k.amax = u2f(amax_bits);
     k.enc = p.c / k.amax;
@@ -145,77 +169,140 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t sf_cols = p.cols_p >> 4;
-    const int lb = lane & 15;                // block column inside the tile
-    const int rr0 = wave * 4 + (lane >> 4);  // row inside a 16-row step
+    const int lb = lane & 15;               // block column inside the tile
+    const int rl = wave * 8 + (lane >> 4);  // this lane's row in step 0
     const bool tiled = !PSEUDO && p.sf_layout == FOS_SF_TILED_128X4;
-    const int64_t row_pitch = p.ld, code_pitch = p.cols_p >> 1;
+    const int64_t code_pitch = p.cols_p >> 1;
     const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
-    int buf = 0;
+    // byte offsets inside a tile (the host checked that a tile spans less than 2^31 bytes);
+    // step g starts 32 (g >> 1) + 4 (g & 1) rows below step 0
+    const uint32_t x_lane = (uint32_t)(rl * p.ld + lb * 16) * 2u, x_row = (uint32_t)p.ld * 2u;
+    const uint32_t c_lane = (uint32_t)(rl * code_pitch + lb * 8), c_row = (uint32_t)code_pitch;
+    const uint32_t o_lane = PSEUDO ? (uint32_t)(rl * p.ldo + lb * 16) * 2u : 0u, o_row = PSEUDO ? (uint32_t)p.ldo * 2u : 0u;
+    auto step_row = [](int g) { return 32 * (g >> 1) + 4 * (g & 1); };
+    // scale byte of (q, h, i; block column lb) in the wavefront's staging area: 128 bytes per
+    // scale tile lb >> 2, unit 4 h + i, byte 4 q + (lb & 3)
+    uint8_t *stage = reinterpret_cast<uint8_t *>(sf_stage[wave]) + (lb >> 2) * 128 + (lane >> 4) * 16 + (lb & 3);
 
-    for (uint32_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x, buf ^= 1) {
-        const uint32_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - tile_y * (uint32_t)p.tiles_x;
-        const int64_t cb = (int64_t)tile_x * 16 + lb;  // block column in the tensor
-        const bool col_ok = FULL || cb < sf_cols;
-        const int64_t row0 = (int64_t)tile_y * 128 + rr0;
-        const uint16_t *src = p.x + row0 * row_pitch + cb * 16;
-        uint8_t *dst = p.codes + row0 * code_pitch + cb * 8;
-        uint8_t *stage = reinterpret_cast<uint8_t *>(sf_stage[buf]) + (lb >> 2) * 512 + (lb & 3);
-
-        auto load = [&](int g, Block16 &b) {
-            if (FULL || (col_ok && row0 + g * 16 < p.rows && cb * 16 < p.cols)) {
-                const uint4 *q = reinterpret_cast<const uint4 *>(src + (int64_t)g * 16 * row_pitch);
-                const uint4 lo = q[0], hi = q[1];
-                b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
-                b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) b.w[i] = 0;
+    auto open_tile = [&](uint32_t tile, bool valid) {
+        RowsTile t;
+        t.tile_y = tile / (uint32_t)p.tiles_x;
+        t.tile_x = tile - t.tile_y * (uint32_t)p.tiles_x;
+        t.row_base = (int64_t)t.tile_y * 128;
+        const int64_t col_base = (int64_t)t.tile_x * 256;
+        t.cb = (int64_t)t.tile_x * 16 + lb;
+        // input: everything from the tile's first element to the end of the tensor's last row
+        uint32_t x_bytes = valid ? 0xffffffffu : 0u;
+        if (!FULL && valid) {
+            const int64_t left = ((p.rows - t.row_base) * p.ld - col_base) * 2;
+            x_bytes = left <= 0 ? 0u : (left > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)left);
+        }
+        t.rx = make_rsrc(p.x + t.row_base * p.ld + col_base, x_bytes);
+        t.rcodes = make_rsrc(PSEUDO ? nullptr : p.codes + t.row_base * code_pitch + col_base / 2, 0xffffffffu);
+        t.rout = make_rsrc(PSEUDO ? p.pseudo_out + t.row_base * p.ldo + col_base : nullptr, 0xffffffffu);
+        t.x_off = (FULL || t.cb * 16 < p.cols) ? x_lane : 0x80000000u;
+        return t;
+    };
+    auto load = [&](const RowsTile &t, int g, Block16 &b) {
+        u32x4 lo, hi;
+        if (FULL) {
+            lo = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off, step_row(g) * x_row, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + 16u, step_row(g) * x_row, 0);
+        } else {
+            // the range check covers the per-lane offset only: keep the step inside it
+            lo = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + step_row(g) * x_row, 0, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + step_row(g) * x_row + 16u, 0, 0);
+        }
+        b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
+        b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
+    };
+    auto process = [&](const RowsTile &t, int g, const Block16 &b) {
+        if (!FULL && t.cb >= sf_cols) return;  // past the padded width
+        const int64_t row = t.row_base + step_row(g) + rl;
+        // a step that lies wholly in the row padding (decode-sized inputs: most steps) only
+        // writes its zero codes and scales
+        const bool padding_step = !FULL && t.row_base + step_row(g) + wave * 8 >= p.rows;
+        BlockOut o{0u, 0u, 0u};
+        if (!padding_step)
+            o = quantize_block_nvfp4_fast<RULE, false, SR>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                                                           (uint64_t)(row * sf_cols + t.cb));
+        if (PSEUDO) {
+            uint32_t w[8];
+            if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+            else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
+            if (FULL || (row < p.rows && t.cb * 16 < p.cols)) {
+                const u32x4 d0 = {w[0], w[1], w[2], w[3]}, d1 = {w[4], w[5], w[6], w[7]};
+                __builtin_amdgcn_raw_buffer_store_b128(d0, t.rout, o_lane, step_row(g) * o_row, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(d1, t.rout, o_lane + 16u, step_row(g) * o_row, 0);
             }
-        };
+            return;
+        }
+        const u32x2 c01 = {o.c0, o.c1};
+        __builtin_amdgcn_raw_buffer_store_b64(c01, t.rcodes, c_lane, step_row(g) * c_row, 0);
+        if (tiled) stage[(g & 1) * 64 + (g >> 1) * 4] = (uint8_t)o.s;
+        else p.sf[row * sf_cols + t.cb] = (uint8_t)o.s;
+    };
 
-        Block16 blk[8];
-        load(0, blk[0]);
-        load(1, blk[1]);
+    uint32_t tile = blockIdx.x;
+    RowsTile cur = open_tile(tile, tile < n_tiles);
+    Block16 ring[4];
+    __builtin_amdgcn_s_setprio(3);
+#ifdef FOS_TRACE
+    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime(), tr_c0 = __builtin_amdgcn_s_memtime();
+    uint64_t tr_tile[5] = {0, 0, 0, 0, 0};
+    int tr_n = 0;
+#endif
+    load(cur, 0, ring[0]);
+    load(cur, 1, ring[1]);
+    load(cur, 2, ring[2]);
+    while (tile < n_tiles) {
+        const uint32_t next = tile + gridDim.x;
+        const bool has_next = next < n_tiles;
+        const RowsTile nxt = open_tile(has_next ? next : tile, has_next);  // without a next tile: loads of nothing
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g + 2 < 8) load(g + 2, blk[g + 2]);
-            if (col_ok) {
-                const int rr = g * 16 + rr0;
-                // a 16-row step that lies wholly in the row padding (decode-sized inputs: seven of
-                // the eight steps) only writes its zero codes and scales
-                const bool padding_step = !FULL && (int64_t)tile_y * 128 + g * 16 >= p.rows;
-                BlockOut o{0u, 0u, 0u};
-                if (!padding_step)
-                    o = quantize_block_nvfp4_fast<RULE, false, SR>(blk[g], k, enc_fast, rq, maybe_negzero, in_range, lut, p.seed,
-                                                                   p.offset, (uint64_t)((row0 + g * 16) * sf_cols + cb));
-                if (PSEUDO) {
-                    uint32_t w[8];
-                    if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
-                    else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
-                    if (FULL || (row0 + g * 16 < p.rows && cb * 16 < p.cols)) {
-                        uint4 *d = reinterpret_cast<uint4 *>(p.pseudo_out + (row0 + g * 16) * p.ldo + cb * 16);
-                        d[0] = make_uint4(w[0], w[1], w[2], w[3]);
-                        d[1] = make_uint4(w[4], w[5], w[6], w[7]);
-                    }
-                    continue;
-                }
-                *reinterpret_cast<uint2 *>(dst + (int64_t)g * 16 * code_pitch) = make_uint2(o.c0, o.c1);
-                if (tiled) stage[(rr & 31) * 16 + (rr >> 5) * 4] = (uint8_t)o.s;
-                else p.sf[(row0 + g * 16) * sf_cols + cb] = (uint8_t)o.s;
+            // in its last tile a wavefront gives way, step by step, to those that are further behind
+            if (!has_next && (g & 1) == 0) {
+                if (g == 0) __builtin_amdgcn_s_setprio(3);
+                if (g == 2) __builtin_amdgcn_s_setprio(2);
+                if (g == 4) __builtin_amdgcn_s_setprio(1);
+                if (g == 6) __builtin_amdgcn_s_setprio(0);
             }
+            if (g + 3 < 8) load(cur, g + 3, ring[(g + 3) & 3]);
+            else load(nxt, g + 3 - 8, ring[(g + 3) & 3]);
+            process(cur, g, ring[g & 3]);
         }
         if (tiled) {
-            __syncthreads();
-            // 4 scale tiles x 512 bytes, contiguous in the output; 8 bytes per thread.  The
-            // other staging buffer is in use by the next tile, so one barrier per tile does.
-            const int t = threadIdx.x >> 6;
-            const int64_t group = (int64_t)tile_x * 4 + t;
-            if (FULL || group < (sf_cols >> 2)) {
-                uint2 *out = reinterpret_cast<uint2 *>(p.sf + ((int64_t)tile_y * (sf_cols >> 2) + group) * 512);
-                out[lane] = reinterpret_cast<const uint2 *>(sf_stage[buf])[threadIdx.x];
-            }
+            // the wavefront's own 4 x 128 bytes: written above by its lanes, read back here in
+            // output order (LDS operations of one wavefront complete in order)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int64_t group = (int64_t)cur.tile_x * 4 + (lane >> 4);
+            const uint2 v = reinterpret_cast<const uint2 *>(sf_stage[wave])[lane];
+            if (FULL || group < (sf_cols >> 2))
+                *reinterpret_cast<uint2 *>(p.sf + ((int64_t)cur.tile_y * (sf_cols >> 2) + group) * 512 + wave * 128 + (lane & 15) * 8) = v;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
+        cur = nxt;
+        tile = next;
+#ifdef FOS_TRACE
+        if (tr_n < 5) tr_tile[tr_n++] = __builtin_amdgcn_s_memrealtime();
+#endif
     }
+#ifdef FOS_TRACE
+    if (lane == 0) {
+        // trace record behind the scale bytes: {start, end (100 MHz ticks), shader cycles, tile ends...}
+        uint64_t *rec = reinterpret_cast<uint64_t *>(p.sf + p.rows_p * sf_cols) + (blockIdx.x * 4 + wave) * 8;
+        rec[0] = tr_t0;
+        rec[1] = __builtin_amdgcn_s_memrealtime();
+        rec[2] = __builtin_amdgcn_s_memtime() - tr_c0;
+        for (int i = 0; i < 3; ++i) rec[3 + i] = tr_tile[i];
+        rec[6] = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20) /* XCC_ID */;
+        rec[7] = __builtin_amdgcn_s_getreg((32 - 1) << 11 | 0 << 6 | 4) /* HW_ID */;
+    }
+#endif
 }
 
 template <int RULE, bool PSEUDO, bool SR>

@@ -23,9 +23,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
     __shared__ uint32_t sf_tile[T * 128];  // T tiles of 512 scale bytes
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[FAST ? 128 : 1];
 
-    uint32_t amax_bits;
-    bool maybe_negzero;
-    reduce_partials(p, red, amax_bits, maybe_negzero);
+    const uint32_t amax_bits = reduce_partials(p, red);
     QuantConsts k;
     k.amax = u2f(amax_bits);
     k.enc = p.c / k.amax;
@@ -106,8 +104,8 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
 #pragma unroll
             for (int i = 0; i < 8; ++i) blk.w[i] = w[it][i];
             BlockOut o;
-            if constexpr (DT == FOS_DTYPE_IF4) o = quantize_block_if4_mse<TWO_D>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut);
-            else o = quantize_block_nvfp4_fast<RULE, TWO_D, false>(blk, k, enc_fast, rq, maybe_negzero, in_range, lut, 0, 0, 0);
+            if constexpr (DT == FOS_DTYPE_IF4) o = quantize_block_if4_mse<TWO_D>(blk, k, enc_fast, rq, in_range, lut);
+            else o = quantize_block_nvfp4_fast<RULE, TWO_D, false>(blk, k, enc_fast, rq, in_range, lut, 0, 0, 0);
             codes[0] = o.c0;
             codes[1] = o.c1;
             sbyte = o.s;
