@@ -217,6 +217,28 @@ __device__ __attribute__((noinline)) bool exact_pick_b(Block16 blk, uint32_t a0,
     return finish_error<RULE, TWO_D>(totB) < finish_error<RULE, TWO_D>(totA);
 }
 
+// The same for a 1x16 block, unrolled in registers: no call and no scratch memory, so it can
+// sit in the streaming loop (a call there makes the wavefront wait for every load it has in
+// flight, and a few such waits were what the slowest wavefronts of a launch spent their time on).
+template <int RULE>
+FOS_DEVICE bool exact_pick_b_1d(const float *x, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, const FastLutEntry &A,
+                                const FastLutEntry &B) {
+    float eA[16], eB[16];
+    static_for<0, 8>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+        const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float dA = candidate_residual(fa[h], A, x[2 * j + h]);
+            const float dB = candidate_residual(fb[h], B, x[2 * j + h]);
+            eA[2 * j + h] = RULE == FOS_RULE_MSE ? dA * dA : fabsf(dA);
+            eB[2 * j + h] = RULE == FOS_RULE_MSE ? dB * dB : fabsf(dB);
+        }
+    });
+    return reduce_error<RULE, false>(eB) < reduce_error<RULE, false>(eA);
+}
+
 // Operation-by-operation form (sub-normal block scales, out-of-range tensors): the
 // arithmetic of quantize_block in fos_quantize_common.h, rolled.
 template <int RULE, bool TWO_D>
@@ -358,8 +380,10 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
                     if (TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                     if (tie) pickB = false;
-                    else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
-                    else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // e.g. the unbiased style's divisor
+                    else if (k.exact_ok) {
+                        if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
+                        else pickB = exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
+                    } else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // e.g. the unbiased style's divisor
                 }
                 return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
             }
@@ -414,8 +438,10 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                 }
                 if (tie) pickB = false;
-                else if (k.exact_ok) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
-                else return generic_block<RULE, TWO_D>(blk, k);
+                else if (k.exact_ok) {
+                    if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
+                    else pickB = exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
+                } else return generic_block<RULE, TWO_D>(blk, k);
             }
             return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
         }

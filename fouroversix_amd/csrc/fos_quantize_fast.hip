@@ -152,21 +152,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][128];  // per wavefront: 4 scale tiles x 128 bytes
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
-    const uint32_t amax_bits = reduce_partials(p, red);
-    QuantConsts k;
-    k.amax = u2f(amax_bits);
-    k.enc = p.c / k.amax;
-    k.dec = 1.0f / (p.c / k.amax);
-    k.qdiv = p.qdiv;
-    k.errdiv = p.errdiv;
-    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
-    if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
-    const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
-    const float enc_fast = in_range ? k.enc : 0.0f;
-    const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
-    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
-    __syncthreads();
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t sf_cols = p.cols_p >> 4;
     const int lb = lane & 15;               // block column inside the tile
@@ -216,6 +201,47 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
         b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
     };
+    // the first input loads do not depend on the tensor maximum: they go out before the setup below
+    uint32_t tile = blockIdx.x;
+    RowsTile cur = open_tile(tile, tile < n_tiles);
+    Block16 ring[4];
+#ifdef FOS_TRACE
+    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime(), tr_c0 = __builtin_amdgcn_s_memtime();
+    uint64_t tr_tile[5] = {0, 0, 0, 0, 0};
+    int tr_n = 0;
+#endif
+    load(cur, 0, ring[0]);
+    load(cur, 1, ring[1]);
+    load(cur, 2, ring[2]);
+
+    // pass-1 results behind them: one round trip to memory covers both
+    uint32_t pm[4] = {0u, 0u, 0u, 0u};
+    if (p.n_partials == 0) {
+        pm[0] = p.partials[0];
+    } else if (p.n_partials > 0) {
+#pragma unroll
+        for (int u = 0; u < kMaxPartials / kThreads; ++u)
+            if ((int)threadIdx.x + u * kThreads < p.n_partials) pm[u] = p.partials[2 * (threadIdx.x + u * kThreads)];
+    }
+    // setup: tensor maximum, constants, per-scale table
+    uint32_t amax_bits;
+    if (p.n_partials == 0) amax_bits = pm[0];
+    else if (p.n_partials > 0) amax_bits = block_max_u32(max(max(pm[0], pm[1]), max(pm[2], pm[3])), red);
+    else amax_bits = reduce_partials(p, red);  // small input: scan it here
+    QuantConsts k;
+    k.amax = u2f(amax_bits);
+    k.enc = p.c / k.amax;
+    k.dec = 1.0f / (p.c / k.amax);
+    k.qdiv = p.qdiv;
+    k.errdiv = p.errdiv;
+    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
+    const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
+    const float enc_fast = in_range ? k.enc : 0.0f;
+    const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
+    __syncthreads();
+
     auto process = [&](const RowsTile &t, int g, const Block16 &b) {
         if (!FULL && t.cb >= sf_cols) return;  // past the padded width
         const int64_t row = t.row_base + step_row(g) + rl;
@@ -232,8 +258,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
             if (FULL || (row < p.rows && t.cb * 16 < p.cols)) {
                 const u32x4 d0 = {w[0], w[1], w[2], w[3]}, d1 = {w[4], w[5], w[6], w[7]};
-                __builtin_amdgcn_raw_buffer_store_b128(d0, t.rout, o_lane, step_row(g) * o_row, 0);
-                __builtin_amdgcn_raw_buffer_store_b128(d1, t.rout, o_lane + 16u, step_row(g) * o_row, 0);
+                // (a 128-bit buffer store with a scalar offset register reads its data late: a VALU
+                // write to the data registers right behind it reached memory in tests, so the step goes
+                // into the per-lane offset)
+                const uint32_t o_off = o_lane + step_row(g) * o_row;
+                __builtin_amdgcn_raw_buffer_store_b128(d0, t.rout, o_off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(d1, t.rout, o_off + 16u, 0, 0);
             }
             return;
         }
@@ -243,18 +273,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         else p.sf[row * sf_cols + t.cb] = (uint8_t)o.s;
     };
 
-    uint32_t tile = blockIdx.x;
-    RowsTile cur = open_tile(tile, tile < n_tiles);
-    Block16 ring[4];
     __builtin_amdgcn_s_setprio(3);
-#ifdef FOS_TRACE
-    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime(), tr_c0 = __builtin_amdgcn_s_memtime();
-    uint64_t tr_tile[5] = {0, 0, 0, 0, 0};
-    int tr_n = 0;
-#endif
-    load(cur, 0, ring[0]);
-    load(cur, 1, ring[1]);
-    load(cur, 2, ring[2]);
     while (tile < n_tiles) {
         const uint32_t next = tile + gridDim.x;
         const bool has_next = next < n_tiles;
