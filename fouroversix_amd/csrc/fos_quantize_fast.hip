@@ -137,9 +137,17 @@ FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
 // ragged tile's descriptor ends with the tensor's last row and lanes past the last column
 // get an offset beyond it: both read zeros, which is the padding the reference adds.
 // FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
+// A wave-uniform 64-bit value, spelled so that the compiler keeps it in scalar registers (a
+// descriptor it believes to differ between lanes makes every buffer access a loop over lanes).
+FOS_DEVICE uint64_t uniform64(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+}
+
 struct RowsTile {
-    BufferRsrc rx, rcodes, rout;
-    uint32_t x_off;      // this lane's offset into rx (beyond the descriptor for a lane past the last column)
+    uint64_t x_base, codes_base, out_base;  // addresses of the tile's first input element / code byte / output element
+    uint32_t x_bytes;    // extent of the input descriptor
+    uint32_t x_off;      // this lane's offset into it (beyond the descriptor for a lane past the last column)
     int64_t row_base;    // first row of the tile
     int64_t cb;          // this lane's block column in the tensor
     uint32_t tile_y, tile_x;
@@ -182,21 +190,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const int64_t left = ((p.rows - t.row_base) * p.ld - col_base) * 2;
             x_bytes = left <= 0 ? 0u : (left > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)left);
         }
-        t.rx = make_rsrc(p.x + t.row_base * p.ld + col_base, x_bytes);
-        t.rcodes = make_rsrc(PSEUDO ? nullptr : p.codes + t.row_base * code_pitch + col_base / 2, 0xffffffffu);
-        t.rout = make_rsrc(PSEUDO ? p.pseudo_out + t.row_base * p.ldo + col_base : nullptr, 0xffffffffu);
+        t.x_bytes = __builtin_amdgcn_readfirstlane(x_bytes);
+        t.x_base = uniform64((uint64_t)(p.x + t.row_base * p.ld + col_base));
+        t.codes_base = PSEUDO ? 0 : uniform64((uint64_t)(p.codes + t.row_base * code_pitch + col_base / 2));
+        t.out_base = PSEUDO ? uniform64((uint64_t)(p.pseudo_out + t.row_base * p.ldo + col_base)) : 0;
         t.x_off = (FULL || t.cb * 16 < p.cols) ? x_lane : 0x80000000u;
         return t;
     };
     auto load = [&](const RowsTile &t, int g, Block16 &b) {
+        const BufferRsrc rx = make_rsrc(reinterpret_cast<const void *>(uniform64(t.x_base)), __builtin_amdgcn_readfirstlane(t.x_bytes));
         u32x4 lo, hi;
         if (FULL) {
-            lo = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off, step_row(g) * x_row, 0);
-            hi = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + 16u, step_row(g) * x_row, 0);
+            lo = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off, step_row(g) * x_row, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + 16u, step_row(g) * x_row, 0);
         } else {
             // the range check covers the per-lane offset only: keep the step inside it
-            lo = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + step_row(g) * x_row, 0, 0);
-            hi = __builtin_amdgcn_raw_buffer_load_b128(t.rx, t.x_off + step_row(g) * x_row + 16u, 0, 0);
+            lo = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + step_row(g) * x_row, 0, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + step_row(g) * x_row + 16u, 0, 0);
         }
         b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
         b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
@@ -262,13 +272,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 // write to the data registers right behind it reached memory in tests, so the step goes
                 // into the per-lane offset)
                 const uint32_t o_off = o_lane + step_row(g) * o_row;
-                __builtin_amdgcn_raw_buffer_store_b128(d0, t.rout, o_off, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b128(d1, t.rout, o_off + 16u, 0, 0);
+                const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
+                __builtin_amdgcn_raw_buffer_store_b128(d0, rout, o_off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(d1, rout, o_off + 16u, 0, 0);
             }
             return;
         }
         const u32x2 c01 = {o.c0, o.c1};
-        __builtin_amdgcn_raw_buffer_store_b64(c01, t.rcodes, c_lane, step_row(g) * c_row, 0);
+        const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
+        __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, step_row(g) * c_row, 0);
         if (tiled) stage[(g & 1) * 64 + (g >> 1) * 4] = (uint8_t)o.s;
         else p.sf[row * sf_cols + t.cb] = (uint8_t)o.s;
     };
