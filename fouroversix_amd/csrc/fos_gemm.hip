@@ -8,11 +8,17 @@
 // v_mfma_f32_32x32x16_f16 with FP32 accumulation; alpha is applied in the epilogue from
 // device memory (src/fouroversix/csrc/fp4_gemm.cu:143).
 //
-// Pipeline per workgroup (tile BM x BN x 64, BM = BN = threads / 2): every thread owns 32
-// codes of one A row and of one B row per K step.  Registers hold the packed data of step
-// k+2 (in flight from HBM) while step k+1 is dequantised into one LDS buffer and step k is
-// multiplied out of the other, so there is one barrier per K step and the VALU work of the
-// dequantisation issues in the shadow of the MFMAs.  The big tile (256 x 256, 8
+// Pipeline per workgroup (tile BM x BN x 64, BM = threads / 2): every thread owns 32 codes of
+// one A row per K step.  Registers hold the packed data of step k+2 (in flight from HBM) while
+// step k+1 is dequantised into one LDS buffer and step k is multiplied out of the other, so
+// there is one barrier per K step and the VALU work of the dequantisation issues in the shadow
+// of the MFMAs.  Only A goes through LDS: with both operands there, LDS traffic (fragment
+// reads plus staging writes) took as many cycles per K step as the MFMAs themselves -- a build
+// without the B fragment reads ran 13 % faster -- so each wavefront loads the packed rows of its
+// own B columns (two wavefronts share them: the second finds them in the vector cache) and
+// turns them into MFMA operands in registers.  Within a K step the contraction index is
+// permuted the same way for both operands: the 16-wide slice kk of lane half h covers
+// k = 32 h + 8 kk ... + 7, so that a lane's B codes are 16 contiguous bytes.  The big tile (256 x 256, 8
 // wavefronts of 128 x 64) keeps LDS reads at ~75 % of their bandwidth; a 128 x 128 tile
 // serves shapes that are not multiples of 256 or too small to fill the chip otherwise.
 // Workgroups are numbered so that the tiles resident on one XCD (blockIdx % 8) form a
@@ -80,10 +86,15 @@ FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
 
-// Packed operands of one K step as a thread holds them.
+// Packed operands of one K step as a thread holds them: the half row of A that it turns into
+// fp16 in LDS for the whole workgroup, and, per 32-row tile of its wavefront's B columns, the
+// 32 codes and 4 scale bytes it multiplies itself.
+template <int WN>
 struct Staged {
-    uint4 qa, qb;     // 32 codes of one A row / one B row
-    uint32_t sa, sb;  // the 4 scale bytes of that row's K step
+    uint4 qa;      // 32 codes of one A row
+    uint32_t sa;   // the 4 scale bytes of that row's K step
+    uint4 qb[WN];  // B row of tile j: codes 32 h ... 32 h + 31 of the step (h = lane >> 5)
+    uint32_t sb[WN];
 };
 
 // Output tile of workgroup `bid`: workgroups with equal bid % 8 share an XCD; give each
@@ -111,10 +122,9 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     constexpr bool OUT_BF16 = OUT == kOutBF16;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
-    static_assert(BM == kThreadsG / 2 && BN == kThreadsG / 2, "one thread per half row of each operand");
+    static_assert(BM == kThreadsG / 2, "one thread per half row of A");
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
-    _Float16 *lds_a[2] = {lds, lds + (BM + BN) * kPitch};
-    _Float16 *lds_b[2] = {lds + BM * kPitch, lds + (BM + BN) * kPitch + BM * kPitch};
+    _Float16 *lds_a[2] = {lds, lds + BM * kPitch};
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     int tile_m, tile_n;
@@ -133,34 +143,54 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)((BN >> 7) * sf_groups * 512));
     const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_half * 16);
     const uint32_t s_off = (uint32_t)((ld_row >> 7) * sf_groups * 512 + (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4);
+    // this lane's B rows: row (lane & 31) of tile j of the wavefront's columns, K half lane >> 5
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int lh = lane >> 5;
+    uint32_t qb_off[WN], sb_off[WN];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+        const int row = wn * WN * 32 + j * 32 + (lane & 31);
+        qb_off[j] = (uint32_t)(row * kbytes + lh * 16);
+        sb_off[j] = (uint32_t)((row >> 7) * sf_groups * 512 + (row & 31) * 16 + ((row & 127) >> 5) * 4);
+    }
     // this workgroup's share of the K steps (all of them unless the launch splits K)
     const int64_t ks0 = OUT == kOutPartial ? (int64_t)blockIdx.y * p.ksteps_per_split : 0;
     const int64_t ksteps_all = p.K / BK;
     const int64_t ksteps =
         OUT == kOutPartial ? (ksteps_all - ks0 < p.ksteps_per_split ? ksteps_all - ks0 : p.ksteps_per_split) : ksteps_all;
 
-    auto fetch = [&](int64_t ks, Staged &s) {
+    typedef Staged<WN> StagedT;
+    auto fetch = [&](int64_t ks, StagedT &s) {
         const uint32_t kq = (uint32_t)(ks0 + ks) * 32u, ksf = (uint32_t)(ks0 + ks) * 512u;
         s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
-        s.qb = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)q_off, (int)kq, 0));
         s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
-        s.sb = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)s_off, (int)ksf, 0);
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+            s.qb[j] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)qb_off[j], (int)kq, 0));
+            s.sb[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb, (int)sb_off[j], (int)ksf, 0);
+        }
     };
-    // quarter q (0..3) of the staged data -> 8 halfs of each operand in LDS buffer `buf`
-    auto stage_quarter = [&](const Staged &s, int buf, int q) {
+    // quarter q (0..3) of the staged A data -> 8 halfs in LDS buffer `buf`
+    auto stage_quarter = [&](const StagedT &s, int buf, int q) {
         const uint32_t wa = q == 0 ? s.qa.x : q == 1 ? s.qa.y : q == 2 ? s.qa.z : s.qa.w;
-        const uint32_t wb = q == 0 ? s.qb.x : q == 1 ? s.qb.y : q == 2 ? s.qb.z : s.qb.w;
-        // this thread's two block scales of each operand: bytes 2*ld_half, 2*ld_half + 1
-        const half2_t sa2 = e4m3x2_to_half2(s.sa >> (16 * ld_half)), sb2 = e4m3x2_to_half2(s.sb >> (16 * ld_half));
+        // this thread's two block scales: bytes 2*ld_half, 2*ld_half + 1
+        const half2_t sa2 = e4m3x2_to_half2(s.sa >> (16 * ld_half));
         const half2_t sa = (q >> 1) ? __builtin_shufflevector(sa2, sa2, 1, 1) : __builtin_shufflevector(sa2, sa2, 0, 0);
-        const half2_t sb = (q >> 1) ? __builtin_shufflevector(sb2, sb2, 1, 1) : __builtin_shufflevector(sb2, sb2, 0, 0);
         half8_t *da = reinterpret_cast<half8_t *>(lds_a[buf] + ld_row * kPitch + ld_half * 32);
-        half8_t *db = reinterpret_cast<half8_t *>(lds_b[buf] + ld_row * kPitch + ld_half * 32);
         da[q] = dequant8(wa, sa);
-        db[q] = dequant8(wb, sb);
+    };
+    // MFMA operands of slice kk from this lane's packed B rows: word kk of its 16 bytes, blocks
+    // 2 h + (kk >> 1) of the step
+    auto b_frags = [&](const StagedT &s, int kk, half8_t *fb) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+            const uint32_t wb = kk == 0 ? s.qb[j].x : kk == 1 ? s.qb[j].y : kk == 2 ? s.qb[j].z : s.qb[j].w;
+            const half2_t sb2 = e4m3x2_to_half2(s.sb[j] >> (16 * lh));
+            const half2_t sb = (kk >> 1) ? __builtin_shufflevector(sb2, sb2, 1, 1) : __builtin_shufflevector(sb2, sb2, 0, 0);
+            fb[j] = dequant8(wb, sb);
+        }
     };
 
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
     float16_t acc[WM][WN];
 #pragma unroll
     for (int i = 0; i < WM; ++i)
@@ -169,24 +199,24 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    auto read_frags = [&](int buf, int kk, half8_t *fa, half8_t *fb) {
-        const int kofs = kk * 16 + (lane >> 5) * 8;
+    auto read_frags = [&](int buf, int kk, half8_t *fa) {
+        const int kofs = lh * 32 + kk * 8;
 #pragma unroll
         for (int i = 0; i < WM; ++i)
             fa[i] = *reinterpret_cast<const half8_t *>(lds_a[buf] + (wm * WM * 32 + i * 32 + (lane & 31)) * kPitch + kofs);
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-            fb[j] = *reinterpret_cast<const half8_t *>(lds_b[buf] + (wn * WN * 32 + j * 32 + (lane & 31)) * kPitch + kofs);
     };
 
-    Staged st[2];
+    StagedT st[2];
+    StagedT bcur;                  // the step being multiplied: its B rows (st[] is refilled two steps ahead)
     half8_t fa[2][WM], fb[2][WN];  // MFMA fragments of the current and the next 16-wide K slice
     fetch(0, st[0]);
 #pragma unroll
     for (int q = 0; q < 4; ++q) stage_quarter(st[0], 0, q);
+    b_frags(st[0], 0, fb[0]);
+    bcur = st[0];
     if (ksteps > 1) fetch(1, st[1]);
     __syncthreads();
-    read_frags(0, 0, fa[0], fb[0]);
+    read_frags(0, 0, fa[0]);
 
     // Body of one K step: multiply out of buffer `buf` while staging `nxt` (step ks+1) into
     // the other buffer.  Inside a 16-wide K slice the order is: issue the LDS reads of the
@@ -198,14 +228,18 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     // The body is branch-free (the last step, which has nothing to stage, is a separate
     // instantiation; the prefetch index is clamped instead of guarded): waits are then
     // placed per register instead of conservatively at control-flow joins.
-    auto kstep = [&](auto have_next_c, int64_t ks, int buf, Staged &cur_regs, Staged &nxt) {
+    auto kstep = [&](auto have_next_c, int64_t ks, int buf, StagedT &cur_regs, StagedT &nxt) {
         constexpr bool have_next = decltype(have_next_c)::value;
-        // `cur_regs` (step ks) went into LDS during the previous step: refill them now,
-        // two steps ahead of their use, so HBM / L2 latency has a whole K step to hide in
+        // `cur_regs` (step ks): its A part went into LDS during the previous step and its B part
+        // was copied to `bcur` (before the first step, and at the end of the previous one); refill
+        // them now, two steps ahead of their use, so HBM / L2 latency has a whole K step to hide in
         if (have_next) fetch(ks + 2 < ksteps ? ks + 2 : ksteps - 1, cur_regs);
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
-            if (kk + 1 < BK / 16) read_frags(buf, kk + 1, fa[(kk + 1) & 1], fb[(kk + 1) & 1]);
+            if (kk + 1 < BK / 16) {
+                read_frags(buf, kk + 1, fa[(kk + 1) & 1]);
+                b_frags(bcur, kk + 1, fb[(kk + 1) & 1]);
+            }
             if (have_next) stage_quarter(nxt, buf ^ 1, kk);
             const bool at_barrier = have_next && kk + 1 == BK / 16;
             auto mfmas = [&](int i_begin, int i_end) {
@@ -223,9 +257,12 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
                 mfmas(0, WM / 2);
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
-                read_frags(buf ^ 1, 0, fa[0], fb[0]);
+                read_frags(buf ^ 1, 0, fa[0]);
                 __builtin_amdgcn_sched_barrier(0);
                 mfmas(WM / 2, WM);
+                // the next step's B rows become the current ones (fb[0] is free: slice 3 used fb[1])
+                bcur = nxt;
+                b_frags(bcur, 0, fb[0]);
             } else {
                 mfmas(0, WM);
             }
@@ -267,14 +304,22 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     }
     const float alpha = load_alpha(p);
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+    // A lane holds 4 consecutive n of row m = lane & 31: written as they are, a store
+    // instruction touches 32 rows with 16 bytes each, and the counters showed 2.2 bytes
+    // written to memory per byte of output.  Each wavefront therefore turns its 32-row tiles
+    // round in LDS (free after the last K step: 32 rows x WN * 64 bytes + 16 bytes of padding
+    // per wavefront) and stores whole rows: 16 bytes per lane, WN * 4 lanes per row.
+    constexpr int kRowBytes = WN * 64, kEpiPitch = kRowBytes + 16;
+    static_assert(2 * BM * kPitch * (int)sizeof(_Float16) >= WAVES_M * WAVES_N * 32 * kEpiPitch, "epilogue staging fits the A buffers");
+    __syncthreads();  // every wavefront is done reading the A buffers
+    uint8_t *epi = reinterpret_cast<uint8_t *>(lds) + wave * 32 * kEpiPitch;
+    constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerPass = 64 / kLanesPerRow;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
-        const int64_t m = m0 + wm * WM * 32 + i * 32 + (lane & 31);
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * (lane >> 5);
                 uint16_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -287,10 +332,23 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
                         o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
                     }
                 }
-                uint2 pk = make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
-                *reinterpret_cast<uint2 *>(D + m * p.ldd + n) = pk;
+                *reinterpret_cast<uint2 *>(epi + (lane & 31) * kEpiPitch + (j * 32 + 8 * g + 4 * (lane >> 5)) * 2) =
+                    make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
             }
         }
+        // (LDS operations of one wavefront complete in order: its own writes are visible to its reads)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < 32 / kRowsPerPass; ++t) {
+            const int row = t * kRowsPerPass + lane / kLanesPerRow, c16 = lane % kLanesPerRow;
+            const uint4 v = *reinterpret_cast<const uint4 *>(epi + row * kEpiPitch + c16 * 16);
+            const int64_t m = m0 + wm * WM * 32 + i * 32 + row;
+            *reinterpret_cast<uint4 *>(D + m * p.ldd + n0 + wn * WN * 32 + c16 * 8) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -847,7 +905,7 @@ template <int WAVES_M, int WAVES_N, int WM, int WN>
 static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
-    constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * kPitch * sizeof(_Float16);
+    constexpr size_t lds_bytes = 2 * (size_t)BM * kPitch * sizeof(_Float16);  // two buffers of A
     p.tiles_m = (int)(p.M / BM);
     p.tiles_n = (int)(p.N / BN);
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.splits);
@@ -1025,7 +1083,9 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
     GemmPlan g = plan_gemm(M, N, K);
-    if (M < 128 && g.kind != kPlanSkinny) return FOS_E_BAD_SHAPE;  // partial bands only through the weight-streaming kernel
+    if (M < 128 && g.kind != kPlanSkinny) return FOS_E_BAD_SHAPE;
+    // the tile kernels store whole rows of their output tiles, 16 bytes per lane
+    if (g.kind != kPlanSkinny && (((uintptr_t)D & 15) || (ldd % 8 != 0))) return FOS_E_BAD_ALIGNMENT;  // partial bands only through the weight-streaming kernel
     if (g.splits > 1 && !(workspace && !((uintptr_t)workspace & 15) &&
                           workspace_bytes >= (size_t)g.splits * (size_t)M * (size_t)N * sizeof(float))) {
         // no (or too small a) workspace: run unsplit

@@ -163,7 +163,8 @@ int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, i
  *   sfA, sfB  E4M3 bytes in the FOS_SF_TILED_128X4 layout of [M, K/16] / [N, K/16]
  *   alpha f32[1] on the device
  * N must be a multiple of 128 and K of 64, and M a multiple of 128 (the padded shapes that
- * fos_quantize produces).  M < 128 is also accepted when K is a multiple of 256: A then
+ * fos_quantize produces); D 16-byte aligned and ldd a multiple of 8 (8-byte aligned and a
+ * multiple of 4 suffice for M <= 128).  M < 128 is also accepted when K is a multiple of 256: A then
  * holds M rows, sfA the full 128-row band of the tiled layout, and only M rows of D are
  * written (decode-sized batches skip the work on the padding rows).
  *   workspace  optional (may be NULL): fos_gemm_workspace_bytes(M, N, K) bytes, 16-byte
