@@ -23,6 +23,7 @@ TORCH_TO_T = {torch.bfloat16: T_BF16, torch.float16: T_F16, torch.float32: T_F32
 EXPORTS = (
     "fos_version",
     "fos_error_string",
+    "fos_tuning_reload",
     "fos_padded_rows",
     "fos_padded_cols",
     "fos_quantize_workspace_bytes",
@@ -64,6 +65,8 @@ def lib() -> ctypes.CDLL:
     L.fos_version.restype = i32
     L.fos_error_string.argtypes = [i32]
     L.fos_error_string.restype = c.c_char_p
+    L.fos_tuning_reload.argtypes = []
+    L.fos_tuning_reload.restype = None
     L.fos_padded_rows.argtypes = [i64]
     L.fos_padded_rows.restype = i64
     L.fos_padded_cols.argtypes = [i64]

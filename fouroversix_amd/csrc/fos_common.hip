@@ -1,5 +1,36 @@
-// Version and error strings of the C ABI.
+// Version and error strings of the C ABI, and the tuning overrides.
+#include <cstdlib>
+#include <mutex>
+
+#include "fos_tuning.h"
 #include "fouroversix_hip.h"
+
+namespace fos {
+namespace {
+Tuning g_tuning;
+std::once_flag g_tuning_once;
+int env_int(const char *name) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : 0;
+}
+void load_tuning() {
+    g_tuning.gemm_tile = env_int("FOS_GEMM_TILE");
+    g_tuning.gemm_splitk = env_int("FOS_GEMM_SPLITK");
+    g_tuning.mx_tile = env_int("FOS_MX_TILE");
+    g_tuning.quant_grid = env_int("FOS_QUANT_GRID");
+    g_tuning.amax_grid = env_int("FOS_AMAX_GRID");
+}
+}  // namespace
+const Tuning &tuning() {
+    std::call_once(g_tuning_once, load_tuning);
+    return g_tuning;
+}
+}  // namespace fos
+
+extern "C" void fos_tuning_reload(void) {
+    (void)fos::tuning();
+    fos::load_tuning();
+}
 
 extern "C" int fos_version(void) { return 100; }
 

@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "fos_device.h"
+#include "fos_tuning.h"
 #include "fouroversix_hip.h"
 
 namespace fos {
@@ -978,14 +979,10 @@ struct GemmPlan {
     int wide;    // M > 32: workgroups of 64 rows of B and 64 rows of A, four wavefronts with two by two tiles each
 };
 constexpr int kTargetWorkgroups = 256;
-static int env_int(const char *name, int fallback) {
-    const char *e = getenv(name);
-    return e ? atoi(e) : fallback;
-}
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
     g.narrow = g.wide = 0;
-    const int tile = env_int("FOS_GEMM_TILE", 0);  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
+    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
     int64_t steps, tiles;
     if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32 || tile == 64)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
@@ -1027,7 +1024,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     const int64_t enough = g.kind == kPlanSkinny ? kTargetWorkgroups / 2 + 1 : kTargetWorkgroups / 2;
     int64_t want = tiles >= enough ? 1 : (kTargetWorkgroups + tiles - 1) / tiles;
     if (want > steps / min_steps) want = steps / min_steps;
-    want = env_int("FOS_GEMM_SPLITK", (int)want);  // tuning / tests
+    if (const int forced_splits = tuning().gemm_splitk) want = forced_splits;  // tuning / tests
     if (want > steps) want = steps;
     if (want > 32) want = 32;
     if (want < 1) want = 1;
@@ -1076,7 +1073,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 15) || ((uintptr_t)sfB & 15) ||
         ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
         return FOS_E_BAD_ALIGNMENT;
-    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 24)) return FOS_E_BAD_SHAPE;
+    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 22)) return FOS_E_BAD_SHAPE;  // a 256-row panel of packed codes stays below 2^31 bytes (32-bit buffer offsets)
     GemmParams p;
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
     p.amax_a = amax_a; p.amax_b = amax_b; p.inv_den = alpha ? 0.0f : (float)(1.0 / denominator);
@@ -1102,7 +1099,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);
             // FOS_GEMM_TILE = 16 / 32 forces / forbids it (tuning, tests)
             if (M <= 16) {
-                const int forced = env_int("FOS_GEMM_TILE", 0);
+                const int forced = tuning().gemm_tile;
                 if (forced == 16 || (forced != 32 && g.ksteps_per_split >= 16))
                     return g.narrow ? launch_decode<1>(p, out_type, s) : launch_decode<2>(p, out_type, s);
             }

@@ -20,6 +20,7 @@
 #include <cstdlib>
 
 #include "fos_quantize_fast.h"
+#include "fos_tuning.h"
 #include "fouroversix_hip.h"
 
 namespace fos {
@@ -751,14 +752,14 @@ extern "C" int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 15) || ((uintptr_t)sfB & 15) ||
         ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
         return FOS_E_BAD_ALIGNMENT;
-    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 24)) return FOS_E_BAD_SHAPE;
+    if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 22)) return FOS_E_BAD_SHAPE;  // a 256-row panel of packed codes stays below 2^31 bytes (32-bit buffer offsets)
     MxGemmParams p;
     p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
     bool big = (M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256;
     int forced = 0;
-    if (const char *e = getenv("FOS_MX_TILE")) forced = atoi(e);  // tuning / tests: 128 small tile, 256 register-staged big tile
+    forced = fos::tuning().mx_tile;  // tuning / tests: 128 small tile, 256 register-staged big tile
     big = big && forced != 128;
     if (big && forced != 256) return launch_gemm_mxfp4_dma(p, out_type, s);
     if (big) return launch_gemm_mxfp4<2, 4, 4, 2>(p, out_type, s);

@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "fos_quantize_kernel.h"
+#include "fos_tuning.h"
 
 namespace fos {
 
@@ -203,7 +204,7 @@ int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t l
         // one workgroup per compute unit reads fastest (128 MiB, inputs rotating through 512 MiB:
         // 21.6 us with 256 workgroups, 22.6 with 512, 26.9 with 1024 for the bare loads)
         int64_t cap = 256;
-        if (const char *e = getenv("FOS_AMAX_GRID")) cap = atoll(e) > 0 && atoll(e) <= kMaxPartials ? atoll(e) : cap;
+        if (const int forced = tuning().amax_grid) cap = forced > 0 && forced <= kMaxPartials ? forced : cap;
         n_partials = (int)(want > cap ? cap : (want < 1 ? 1 : want));
         hipLaunchKernelGGL((amax_flat_kernel<true>), dim3(n_partials), dim3(kThreads), 0, s, (const uint4 *)x, n_vec,
                            partials);

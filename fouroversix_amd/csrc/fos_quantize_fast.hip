@@ -14,6 +14,7 @@
 #include <cstdlib>
 
 #include "fos_quantize_kernel.h"
+#include "fos_tuning.h"
 
 namespace fos {
 
@@ -350,7 +351,7 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         // five resident workgroups per compute unit (256 CUs, <= 102 VGPRs); more tiles than
         // that are walked by the same workgroups.  FOS_QUANT_GRID overrides for tuning runs.
         int64_t grid = 1280;
-        if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
+        if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
         if (grid > n) grid = n;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
         if (full)
@@ -364,7 +365,7 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     // Persistent grid: a few workgroups per compute unit (256 CUs), fewer when the tensor
     // is small.  FOS_QUANT_GRID overrides the count for tuning runs.
     int64_t grid = 256 * 6;
-    if (const char *e = getenv("FOS_QUANT_GRID")) grid = atoll(e) > 0 ? atoll(e) : grid;
+    if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
     if (grid > n_tiles) grid = n_tiles;
     hipLaunchKernelGGL((quantize_nvfp4_tile_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }

@@ -1,0 +1,20 @@
+// Kernel-choice overrides for tuning runs and tests.  The FOS_* environment variables are
+// read once, when the first call needs them (and again on fos_tuning_reload()); the entry
+// points themselves only read these integers.  0 = no override.
+#pragma once
+
+#include <atomic>
+
+namespace fos {
+
+struct Tuning {
+    std::atomic<int> gemm_tile{0};    // FOS_GEMM_TILE
+    std::atomic<int> gemm_splitk{0};  // FOS_GEMM_SPLITK
+    std::atomic<int> mx_tile{0};      // FOS_MX_TILE
+    std::atomic<int> quant_grid{0};   // FOS_QUANT_GRID
+    std::atomic<int> amax_grid{0};    // FOS_AMAX_GRID
+};
+
+const Tuning &tuning();
+
+}  // namespace fos

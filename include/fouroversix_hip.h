@@ -51,6 +51,11 @@ int fos_version(void);
 /* Human-readable text for a return code (host pointer, static storage). */
 const char *fos_error_string(int code);
 
+/* Kernel-choice overrides for tuning runs and tests (FOS_GEMM_TILE, FOS_GEMM_SPLITK,
+ * FOS_MX_TILE, FOS_QUANT_GRID, FOS_AMAX_GRID) are read from the environment once, at the
+ * first call that needs them; this reads them again.  No counterpart in the reference. */
+void fos_tuning_reload(void);
+
 /* Rows / columns of the padded outputs: rows up to a multiple of 128, columns up to a
  * multiple of 64 (QuantizedTensor, src/fouroversix/quantize/quantized_tensor.py:65-78). */
 int64_t fos_padded_rows(int64_t rows);

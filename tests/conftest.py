@@ -25,3 +25,29 @@ def oracle():
 @pytest.fixture(scope="session")
 def golden_dir():
     return GOLDEN
+
+
+@pytest.fixture(autouse=True)
+def _tuning_follows_environment(monkeypatch):
+    """The library reads its FOS_* overrides once; tests that set them go through this hook,
+    and every test starts from the environment as it is."""
+    from fouroversix_amd import _native as nat
+
+    if not os.path.exists(nat.LIB_PATH):
+        yield
+        return
+    reload_tuning = nat.lib().fos_tuning_reload
+    reload_tuning()
+    set_env, del_env = monkeypatch.setenv, monkeypatch.delenv
+
+    def setenv(name, value, *a, **kw):
+        set_env(name, value, *a, **kw)
+        reload_tuning()
+
+    def delenv(name, *a, **kw):
+        del_env(name, *a, **kw)
+        reload_tuning()
+
+    monkeypatch.setattr(monkeypatch, "setenv", setenv, raising=False)
+    monkeypatch.setattr(monkeypatch, "delenv", delenv, raising=False)
+    yield
