@@ -68,10 +68,15 @@ def test_gemm_fp16_output_and_mixed_rules(oracle):
     assert float((got.float() - expect.float()).abs().max() / expect.float().abs().max()) <= MAX_REL
 
 
-@pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), (16, 4096, 4096), (128, 14336, 4096), (2048, 4096, 14336),
-                                           (128, 4096, 14336), (256, 384, 2368), (64, 14336, 4096), (96, 11008, 4096)])
+LLAMA_SHAPES = [(m, n, k) for m in (16, 128, 2048, 8192) for (n, k) in ((4096, 4096), (14336, 4096), (4096, 14336))]
+
+
+@pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), *LLAMA_SHAPES,
+                                           (16384, 4096, 4096), (16384, 1024, 4096),  # the decoder stack's token count, k/v projection
+                                           (256, 384, 2368), (64, 14336, 4096), (96, 11008, 4096)])
 def test_gemm_full_size_sampled(oracle, m, n, k):
-    """Headline and Llama-3-8B shapes: 192 sampled rows of each operand are multiplied by
+    """Headline shape, every Llama-3-8B linear shape (M in {16, 128, 2048, 8192}) and the
+    decoder stack's 16384-token shapes: 192 sampled rows of each operand are multiplied by
     the oracle (fp64 accumulation) and compared with the same entries of the GPU result."""
     a, b = make_input("randn", (m, k), 5), make_input("randn", (n, k), 6)
     cfg = fos.QuantizationConfig(scale_rule="mse")
