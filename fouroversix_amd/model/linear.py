@@ -133,16 +133,18 @@ class FourOverSixLinear(nn.Linear):
         if not config.keep_master_weights:
             wdt = config.weight_dtype
             pack = wdt.quantized_value_type.packing_factor
+            # (on the weight's device, so that a checkpoint of quantized buffers loads in place)
+            dev = module.weight.device
             self.register_buffer(
                 "quantized_weight_values",
-                torch.zeros(self.out_features, self.in_features // pack, dtype=torch.uint8),
+                torch.zeros(self.out_features, self.in_features // pack, dtype=torch.uint8, device=dev),
             )
             self.register_buffer(
                 "quantized_weight_scale_factors",
-                torch.zeros(self.out_features * self.in_features // wdt.block_size, dtype=wdt.scale_type.torch_dtype),
+                torch.zeros(self.out_features * self.in_features // wdt.block_size, dtype=wdt.scale_type.torch_dtype, device=dev),
             )
-            self.register_buffer("quantized_weight_amax", torch.zeros(1, dtype=torch.float32))
-            self.register_buffer("quantized_weight_metadata", torch.zeros(6, dtype=torch.int32))
+            self.register_buffer("quantized_weight_amax", torch.zeros(1, dtype=torch.float32, device=dev))
+            self.register_buffer("quantized_weight_metadata", torch.zeros(6, dtype=torch.int32, device=dev))
 
     @property
     def parameters_to_quantize(self) -> tuple[str, ...]:

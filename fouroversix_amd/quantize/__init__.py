@@ -1,6 +1,6 @@
 from .config import QuantizationConfig
 from .frontend import can_quantize, dequantize, quantize
-from .layout import from_blocked, to_blocked
+from .layout import from_blocked, get_rht_matrix, to_blocked
 from .quantized_tensor import QuantizedTensor
 
 __all__ = [
@@ -9,6 +9,7 @@ __all__ = [
     "can_quantize",
     "dequantize",
     "from_blocked",
+    "get_rht_matrix",
     "quantize",
     "to_blocked",
 ]

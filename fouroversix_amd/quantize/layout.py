@@ -38,3 +38,21 @@ def from_blocked(a: torch.Tensor, orig_shape: tuple[int, int]) -> torch.Tensor:
     raw = a.contiguous().view(torch.uint8) if a.element_size() == 1 else a.contiguous()
     out = raw.reshape(-1)[tiled_offsets(rows, cols, a.device)]
     return out.view(a.dtype) if a.element_size() == 1 else out
+
+
+# ---- random Hadamard transform matrix ------------------------------------------------------
+
+# The fixed sign vector of the reference's wgrad transform (src/fouroversix/quantize/utils.py:19-30).
+_RHT_SIGNS = (1, 1, 1, -1, 1, -1, -1, -1, -1, -1, -1, 1, -1, 1, -1, -1)
+
+
+def get_rht_matrix(*, with_random_sign_mask: bool = True, device: torch.device | str | int = "cuda") -> torch.Tensor:
+    """bf16 [16, 16]: ``diag(signs) @ H16 / 4`` with the Sylvester-ordered Hadamard matrix
+    ``H16[i, j] = (-1) ** popcount(i & j)`` -- the matrix ``x.reshape(-1, 16) @ M`` applies
+    (reference ``get_rht_matrix``, ``src/fouroversix/quantize/utils.py:68-85``; the kernels
+    apply the same transform as a butterfly, this is for callers that want the matrix)."""
+    idx = torch.arange(16)
+    parity = torch.tensor([[bin(int(i) & int(j)).count("1") & 1 for j in idx] for i in idx])
+    had = (1.0 - 2.0 * parity.float()) * 0.25
+    signs = torch.tensor(_RHT_SIGNS, dtype=torch.float32) if with_random_sign_mask else torch.ones(16)
+    return (signs.unsqueeze(1) * had).to(device=device, dtype=torch.bfloat16)

@@ -1,6 +1,7 @@
 """Host-side mirror of the reference interface: enums, configs, containers, frontends'
 argument handling (no GPU needed)."""
 
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -149,3 +150,24 @@ def test_quantize_of_meta_tensors_returns_padded_shapes():
     assert not q.scale_factors_are_in_blackwell_layout
     y = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True))
     assert y.device.type == "meta" and y.shape == x.shape and y.dtype == x.dtype
+
+
+def test_reference_import_name_and_rht_matrix(oracle):
+    """`import fouroversix` serves code written against the reference package (same public names,
+    sub-packages included), and get_rht_matrix is the matrix the reference's transform applies
+    (src/fouroversix/quantize/utils.py:68-85): diag(signs) H16 / 4, orthogonal."""
+    import fouroversix
+    import fouroversix_amd
+    from fouroversix import QuantizationConfig, dequantize, quantize, quantize_model, quantized_matmul  # noqa: F401
+    from fouroversix.model import FourOverSixLinear, ModuleQuantizationConfig  # noqa: F401
+    from fouroversix.quantize import QuantizedTensor, from_blocked, get_rht_matrix  # noqa: F401
+    from fouroversix.utils import DataType, ScaleRule  # noqa: F401
+
+    assert fouroversix.quantize is fouroversix_amd.quantize and QuantizationConfig is fouroversix_amd.QuantizationConfig
+    assert set(fouroversix.__all__) == set(fouroversix_amd.__all__)
+    m = get_rht_matrix(device="cpu")
+    assert m.dtype == torch.bfloat16 and m.shape == (16, 16)
+    assert np.array_equal(m.float().numpy(), oracle.rht_matrix())
+    assert torch.equal(m.float() @ m.float().T, torch.eye(16))
+    plain = get_rht_matrix(with_random_sign_mask=False, device="cpu")
+    assert torch.equal(plain[0].float(), torch.full((16,), 0.25)) and torch.equal(plain.float(), plain.float().T)

@@ -196,6 +196,40 @@ def test_linear_layer_forward(oracle):
     assert torch.equal(keep(x.cuda()), y)
 
 
+def test_quantized_checkpoint_round_trip():
+    """A quantized layer's state_dict -- the four `quantized_weight_*` buffers of the reference
+    (src/fouroversix/model/modules/linear.py:326-361,379-443) plus the bias -- saved, read back with
+    a loader that executes nothing, and loaded into a fresh module gives a bit-identical forward."""
+    import io
+
+    torch.manual_seed(2)
+    cfg = fos.ModuleQuantizationConfig(weight_scale_2d=True)
+    layer = fos.FourOverSixLinear(nn.Linear(512, 384, bias=True, dtype=torch.bfloat16).cuda(), cfg).quantize_weight_()
+    x = make_input("randn", (3, 40, 512), 37).cuda()
+    y = layer(x)
+    state = layer.state_dict()
+    assert set(state) == {"bias", "quantized_weight_values", "quantized_weight_scale_factors", "quantized_weight_amax",
+                          "quantized_weight_metadata"}
+    assert state["quantized_weight_values"].shape == (384, 256) and state["quantized_weight_values"].dtype == torch.uint8
+    assert state["quantized_weight_scale_factors"].dtype == torch.float8_e4m3fn
+    assert state["quantized_weight_metadata"].tolist() == [384, 512, 384, 512, 1, 1]
+    buf = io.BytesIO()
+    torch.save({k: v.cpu() for k, v in state.items()}, buf)
+    buf.seek(0)
+    loaded = torch.load(buf, weights_only=True)
+    fresh = fos.FourOverSixLinear(nn.Linear(512, 384, bias=True, dtype=torch.bfloat16).cuda(), cfg)
+    fresh.weight = None  # a checkpoint of quantized weights carries no high-precision weight
+    missing, unexpected = fresh.load_state_dict(loaded, strict=True)
+    assert not missing and not unexpected
+    assert torch.equal(fresh(x).view(torch.int16), y.view(torch.int16))
+    # ... and through quantize_model on a model, as a loader of quantized checkpoints would build it
+    model = nn.Sequential(nn.Linear(512, 384, bias=True, dtype=torch.bfloat16)).cuda()
+    fos.quantize_model(model, fos.ModelQuantizationConfig(weight_scale_2d=True))
+    model[0].weight = None
+    model.load_state_dict({"0." + k: v for k, v in loaded.items()})
+    assert torch.equal(model(x).view(torch.int16), y.view(torch.int16))
+
+
 def test_linear_layer_forward_in_fp16(oracle):
     """An fp16 model: fp16 activations and weights are quantized from their own values (the
     reference converts with `.float()`), fp16 output."""
