@@ -28,7 +28,25 @@ struct TransformParams {
     uint32_t *partials;      // pairs {max |y| as f32 bits, 1 if a -0.0 was written}
     int64_t n_units;         // tiles (transpose) or 16-element groups (rows)
     int tiles_x;
+    int vec;                 // x is 16-byte aligned with ld % 8 == 0: whole groups are read as two 128-bit loads
 };
+
+// The 16 elements x[r][c0 .. c0 + 15] as packed pairs, zero beyond the last column.
+FOS_DEVICE void load_group(const TransformParams &p, int64_t r, int64_t c0, uint32_t *w) {
+    if (p.vec && c0 + 16 <= p.cols) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
+        const uint4 lo = src[0], hi = src[1];
+        w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
+        w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
+        return;
+    }
+    const uint16_t *row = p.x + r * p.ld;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t a = c0 + 2 * j < p.cols ? row[c0 + 2 * j] : 0u, b = c0 + 2 * j + 1 < p.cols ? row[c0 + 2 * j + 1] : 0u;
+        w[j] = a | (b << 16);
+    }
+}
 
 typedef float float2_tt __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2_tt __attribute__((ext_vector_type(2)));
@@ -85,13 +103,12 @@ FOS_DEVICE void write_partials(uint32_t m, uint32_t z, uint32_t *partials) {
 
 // RHT without transposition: one thread per group of 16, grid-stride.
 __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParams p) {
-    const int64_t groups_per_row = p.cols >> 4;
+    const int64_t groups_per_row = (p.cols + 15) >> 4;  // a last, partial group is completed with zeros
     uint32_t m = 0, z = 0;
     for (int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x; g < p.n_units; g += (int64_t)gridDim.x * kThreads) {
         const int64_t r = g / groups_per_row, cb = g - r * groups_per_row;
-        const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + cb * 16);
-        const uint4 lo = src[0], hi = src[1];
-        uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        uint32_t w[8];
+        load_group(p, r, cb * 16, w);
         rht16(w);
         track(w, m, z);
         uint4 *dst = reinterpret_cast<uint4 *>(p.y + r * p.ldy + cb * 16);
@@ -102,8 +119,9 @@ __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParam
 }
 
 // Transposition (optionally followed by the RHT along the new rows) through a 64 x 64 LDS
-// tile: rows of x come in as 128-byte runs, rows of y leave as 128-byte runs.  rows and
-// cols are multiples of 16, so 16-element groups are either inside or outside the matrix.
+// tile: rows of x come in as 128-byte runs, rows of y leave as 128-byte runs.  Groups of 16
+// that reach past the last row / column are completed with zeros (y is written in whole groups:
+// its rows hold a multiple of 16 elements).
 template <bool RHT>
 __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformParams p) {
     constexpr int kPitchT = 66;  // halfs per LDS row: 33 dwords, odd, so a column walk changes bank every row
@@ -116,12 +134,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
         {
             const int row = t >> 2, chunk = t & 3;
             uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (r0 + row < p.rows && c0 + chunk * 16 < p.cols) {
-                const uint4 *src = reinterpret_cast<const uint4 *>(p.x + (r0 + row) * p.ld + c0 + chunk * 16);
-                const uint4 lo = src[0], hi = src[1];
-                w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
-                w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
-            }
+            if (r0 + row < p.rows && c0 + chunk * 16 < p.cols) load_group(p, r0 + row, c0 + chunk * 16, w);
             uint32_t *d = reinterpret_cast<uint32_t *>(tile + row * kPitchT + chunk * 16);
 #pragma unroll
             for (int j = 0; j < 8; ++j) d[j] = w[j];
@@ -168,12 +181,10 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if (x_type != FOS_T_BF16 || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
     const int64_t out_cols = transpose ? rows : cols;
-    if (ldy < out_cols) return FOS_E_BAD_SHAPE;
-    // whole 16-element groups in both orientations
-    if (cols % 16 != 0 || (transpose && rows % 16 != 0)) return FOS_E_UNSUPPORTED;
+    // y is written in whole 16-element groups
+    if (ldy < (out_cols + 15) / 16 * 16) return FOS_E_BAD_SHAPE;
     if (!workspace || workspace_bytes < fos_quantize_workspace_bytes(rows, cols)) return FOS_E_WORKSPACE;
-    if (((uintptr_t)x & 15) || ((uintptr_t)y & 15) || (ld % 8 != 0) || (ldy % 8 != 0) || ((uintptr_t)workspace & 7) ||
-        ((uintptr_t)amax & 3))
+    if (((uintptr_t)x & 1) || ((uintptr_t)y & 15) || (ldy % 8 != 0) || ((uintptr_t)workspace & 7) || ((uintptr_t)amax & 3))
         return FOS_E_BAD_ALIGNMENT;
     TransformParams p;
     p.x = static_cast<const uint16_t *>(x);
@@ -181,6 +192,7 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
     p.y = static_cast<uint16_t *>(y);
     p.ldy = ldy;
     p.partials = static_cast<uint32_t *>(workspace);
+    p.vec = (((uintptr_t)x & 15) == 0 && ld % 8 == 0) ? 1 : 0;
     hipStream_t s = (hipStream_t)stream;
     int64_t grid;
     constexpr int64_t kMaxGrid = 1024;  // pairs the workspace holds
@@ -192,7 +204,7 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
         else hipLaunchKernelGGL(transpose_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     } else {
         p.tiles_x = 0;
-        p.n_units = rows * (cols / 16);
+        p.n_units = rows * ((cols + 15) / 16);
         grid = (p.n_units + kThreads - 1) / kThreads;
         if (grid > kMaxGrid) grid = kMaxGrid;
         hipLaunchKernelGGL(rht_rows_kernel, dim3((unsigned)grid), dim3(kThreads), 0, s, p);

@@ -25,10 +25,10 @@ class QuantizationConfig:
     dtype           target format (``nvfp4`` or ``if4`` have kernels)
     kwargs          extra backend arguments: ``seed`` / ``offset`` of the dither stream
     pseudo_quantize return the quantize -> dequantize round trip as a high-precision tensor
-    rht             random Hadamard transform before quantizing (not implemented)
+    rht             random Hadamard transform of every 16 consecutive row elements before quantizing
     round_style     nearest / stochastic / stochastic_unbiased
     scale_rule      static_6, static_4, or the adaptive mse / mae / abs_max
-    transpose       quantize the transposed input (not implemented)
+    transpose       quantize the transposed input
     """
 
     backend: QuantizeBackend | None = None

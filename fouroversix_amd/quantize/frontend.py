@@ -110,7 +110,12 @@ def quantize(
         plain = QuantizationConfig(
             **{**config.__dict__, "transpose": False, "rht": False, "kwargs": {**config.kwargs, "amax": amax}}
         )
-        return quantize(y, plain)
+        q = quantize(y, plain)
+        # the logical shape is that of x (transposed); a ragged width that the Hadamard transform
+        # filled up to a multiple of 16 keeps its codes in the padding, as in the reference
+        # (src/fouroversix/quantize/pytorch/backend.py:57-79,110-121)
+        q.original_shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
+        return q
 
     if config.pseudo_quantize:
         # one fused kernel where the library has it, else the two-step round trip

@@ -162,10 +162,7 @@ def _pseudo_quantize_impl(x, dtype, selection_rule, round_style, is_2d, amax):
 
 def transform_unsupported_reason(x: torch.Tensor, transpose: bool, rht: bool) -> str | None:
     """Why the transpose / random-Hadamard pre-transform cannot run on ``x``, or None."""
-    rows, cols = x.shape
-    if cols % 16 != 0 or (transpose and rows % 16 != 0):
-        return "transpose / rht need dimensions that are multiples of 16"
-    return None
+    return None if x.dim() == 2 else "transpose / rht need a 2-D tensor"
 
 
 def _transform_impl(x, transpose, rht):
@@ -176,11 +173,15 @@ def _transform_impl(x, transpose, rht):
     reason = transform_unsupported_reason(x, transpose, rht)
     if reason is not None:
         raise RuntimeError(f"transform: {reason}")
-    if x.stride(-1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
+    if x.stride(-1) != 1:
         x = x.contiguous()
     rows, cols = x.shape
     dev = x.device
-    y = torch.empty((cols, rows) if transpose else (rows, cols), dtype=torch.bfloat16, device=dev)
+    out_rows, out_cols = (cols, rows) if transpose else (rows, cols)
+    # y is written in whole groups of 16 (zeros complete a ragged last group; with rht that group
+    # then holds values in all 16 places, so the padded width is what gets quantized)
+    width = -(-out_cols // 16) * 16
+    y = torch.empty((out_rows, width), dtype=torch.bfloat16, device=dev)
     amax = torch.empty(1, dtype=torch.float32, device=dev)
     with _on_device(dev):
         stream = nat.current_stream(dev)
@@ -190,7 +191,7 @@ def _transform_impl(x, transpose, rht):
             y.data_ptr(), y.stride(0), amax.data_ptr(), workspace.data_ptr(), workspace.numel(), stream,
         )
     nat.check(rc, "fouroversix::transform")
-    return y, amax
+    return (y if rht or width == out_cols else y[:, :out_cols]), amax
 
 
 def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):

@@ -136,9 +136,13 @@ int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, i
  * for the `x.T` / `x.reshape(-1, 16) @ had` / `abs().max()` steps of the reference
  * quantizer (src/fouroversix/quantize/pytorch/reference.py:567-578,
  * quantize/utils.py:19-85; CUDA: csrc/include/hadamard_transform.h:16-37).  Follow it with
- * fos_quantize(y, ..., amax, amax_is_input = 1).  x and y 16-byte aligned, ld and ldy
- * multiples of 8, cols (and rows when transposing) multiples of 16; same workspace as
- * fos_quantize.
+ * fos_quantize(y, ..., amax, amax_is_input = 1).  y is written in whole groups of 16: it is
+ * 16-byte aligned and ldy a multiple of 8 that holds the output width rounded up to 16; a
+ * group that reaches past the input's last row / column is completed with zeros (the
+ * reference's zero padding, src/fouroversix/quantize/pytorch/backend.py:57-79), so with rht
+ * the last group of a ragged width carries values in all 16 places.  x is read with 128-bit
+ * loads when it is 16-byte aligned and ld a multiple of 8, element by element otherwise.
+ * Same workspace as fos_quantize.
  */
 int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
                   int transpose, int rht, void *y, int64_t ldy, float *amax,

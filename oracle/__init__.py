@@ -185,12 +185,16 @@ def transform(xb: np.ndarray, *, transpose=False, rht=False) -> np.ndarray:
     """bf16 bits of the tensor the reference quantizes when ``transpose`` / ``rht`` are set
     (src/fouroversix/quantize/pytorch/reference.py:567-571): ``x.T``, then every group of 16
     consecutive elements of a row times the RHT matrix as a bf16 matmul, i.e. exact
-    products, fp32 accumulation (here in the order i = 0..15), one rounding to bf16."""
+    products, fp32 accumulation (here in the order i = 0..15), one rounding to bf16.  A ragged
+    width is first completed with zeros (the reference pads to its block multiples before the
+    transform, src/fouroversix/quantize/pytorch/backend.py:57-79), so with ``rht`` the result
+    is a multiple of 16 wide."""
     xb = np.asarray(xb, dtype=np.uint16)
     if transpose:
         xb = np.ascontiguousarray(xb.T)
     if rht:
-        assert xb.shape[1] % 16 == 0
+        if xb.shape[1] % 16:
+            xb = np.pad(xb, ((0, 0), (0, 16 - xb.shape[1] % 16)))
         g = bf16_bits_to_f32(xb).reshape(-1, 16)
         h = rht_matrix()
         acc = np.zeros_like(g)

@@ -134,6 +134,35 @@ def write_transform_vectors() -> None:
     print("wrote transform", len(out))
 
 
+def write_ragged_transpose_vectors(quantize, QuantizationConfig) -> None:  # noqa: N803
+    """`transpose=True` on shapes that are not multiples of (128, 64), through the reference's
+    PyTorch backend wrapper (quantize/pytorch/backend.py:57-79): it sizes the zero padding from
+    the transposed shape but applies it to the tensor before transposing.  Shapes whose padded,
+    transposed extent is not block-aligned make the reference raise; that is recorded too
+    (`<name>.raised` = 1, no outputs)."""
+    out: dict[str, np.ndarray] = {}
+    for name, shape, seed in [("16x80", (16, 80), 41), ("80x144", (80, 144), 42), ("48x112", (48, 112), 43),
+                              ("100x80", (100, 80), 44), ("16x64", (16, 64), 45), ("200x72", (200, 72), 46)]:
+        x = make_input("randn", shape, seed)
+        out[f"{name}.x"] = bits(x)
+        for rule, two_d in (("mse", False), ("static_6", True)):
+            key = f"{name}.{rule}.{'2d' if two_d else '1d'}"
+            try:
+                q = quantize(x.clone(), QuantizationConfig(backend="pytorch", scale_rule=rule, block_scale_2d=two_d, transpose=True))
+                out[key + ".values"] = u8(q.values)
+                out[key + ".sf"] = u8(q.scale_factors)
+                out[key + ".amax"] = np.array([float(q.amax)], dtype=np.float32)
+                out[key + ".padded"] = np.array(q.padded_shape)
+                out[key + ".shape"] = np.array(q.original_shape)
+                out[key + ".raised"] = np.array([0])
+                print(key, "ok", tuple(q.values.shape), q.original_shape, q.padded_shape)
+            except Exception as e:  # noqa: BLE001
+                out[key + ".raised"] = np.array([1])
+                print(key, "raised", type(e).__name__, str(e)[:100])
+    np.savez_compressed(os.path.join(HERE, "ragged_transpose.npz"), **out)
+    print("wrote ragged_transpose", len(out))
+
+
 def write_mxfp4_vectors(quantize, dequantize, quantized_matmul, QuantizationConfig) -> None:  # noqa: N803
     """MXFP4 (E2M1 codes, E8M0 scale per 1x32 block; quantize/pytorch/reference.py:149-181)
     through the reference's PyTorch backend: quantize, dequantize and matmul."""
@@ -233,12 +262,16 @@ def main() -> None:
     ap.add_argument("--time", action="store_true", help="also time the reference CPU path")
     ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
     ap.add_argument("--only-mxfp4", action="store_true", help="write only mxfp4.npz")
+    ap.add_argument("--only-ragged-transpose", action="store_true", help="write only ragged_transpose.npz")
     args = ap.parse_args()
 
     fos = import_reference()
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_ragged_transpose_vectors(quantize, QuantizationConfig)
+    if args.only_ragged_transpose:
+        return
     write_input_dtype_vectors(quantize, QuantizationConfig)
     if args.only_input_dtypes:
         return

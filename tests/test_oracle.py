@@ -106,6 +106,31 @@ def test_transform_options_match_reference_vectors(oracle, golden_dir):
     assert n == 27
 
 
+def test_ragged_transpose_matches_reference_vectors(oracle, golden_dir):
+    """transpose=True on shapes outside the block multiples: where the reference's backend gets
+    through (its padding is sized from the transposed shape but applied before the transpose,
+    src/fouroversix/quantize/pytorch/backend.py:57-79, which fits only some shapes) the result
+    is that of transposing first and completing with zeros; the fixture also records the
+    shapes on which it raised."""
+    d = np.load(os.path.join(golden_dir, "ragged_transpose.npz"))
+    ok = raised = 0
+    for key in d.files:
+        if not key.endswith(".raised"):
+            continue
+        base = key[: -len(".raised")]
+        name, rule, dim = base.split(".")
+        if int(d[key][0]):
+            raised += 1
+            continue
+        q = oracle.quantize(d[f"{name}.x"], scale_rule=rule, block_scale_2d=(dim == "2d"), transpose=True)
+        assert np.array_equal(q.values, d[base + ".values"]), base
+        assert np.array_equal(q.scale_factors, d[base + ".sf"].reshape(-1)), base
+        assert q.amax == d[base + ".amax"][0], base
+        assert tuple(q.padded_shape) == tuple(d[base + ".padded"]) and tuple(q.original_shape) == tuple(d[base + ".shape"])
+        ok += 1
+    assert (ok, raised) == (6, 6)
+
+
 def test_dequantize_matches_reference_vectors(oracle, golden_dir):
     for name in ("randn_256x128", "ragged_100x80", "tiny_blocks_128x128"):
         d = np.load(os.path.join(golden_dir, f"quantize_{name}.npz"))

@@ -567,7 +567,46 @@ def test_transform_properties_full_size():
     assert torch.equal(tt, x)
     th, _ = ops.transform(x, True, True)
     assert torch.equal(th, ops.transform(t, False, True)[0])
-    with pytest.raises(ValueError, match="multiples of 16"):
-        fos.quantize(x[:, :200], fos.QuantizationConfig(rht=True))
-    with pytest.raises(ValueError, match="multiples of 16"):
-        fos.quantize(x[:100], fos.QuantizationConfig(transpose=True))
+
+
+@pytest.mark.parametrize("name", ["16x80", "48x112", "200x72"])
+@pytest.mark.parametrize("rule,two_d", [("mse", False), ("static_6", True)])
+def test_ragged_transpose_matches_the_reference(golden_dir, name, rule, two_d):
+    """Shapes the reference's own backend gets through with transpose=True although neither side
+    is a multiple of its block sizes (vectors written by tests/golden/make_golden.py
+    --only-ragged-transpose): same codes, scales, amax and shapes."""
+    g = np.load(os.path.join(golden_dir, "ragged_transpose.npz"))
+    key = f"{name}.{rule}.{'2d' if two_d else '1d'}"
+    assert int(g[f"{key}.raised"][0]) == 0
+    x = torch.from_numpy(g[f"{name}.x"].view(np.int16)).view(torch.bfloat16).cuda()
+    q = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, block_scale_2d=two_d, transpose=True))
+    assert tuple(q.original_shape) == tuple(int(v) for v in g[f"{key}.shape"])
+    assert tuple(q.padded_shape) == tuple(int(v) for v in g[f"{key}.padded"])
+    assert float(q.amax) == float(g[f"{key}.amax"][0])
+    assert np.array_equal(u8(q.values), g[f"{key}.values"])
+    assert np.array_equal(u8(q.scale_factors).reshape(-1), g[f"{key}.sf"].reshape(-1))
+
+
+@pytest.mark.parametrize("shape", [(16, 64), (80, 144), (100, 80), (37, 50), (130, 200), (1000, 72)])
+@pytest.mark.parametrize("transpose,rht", [(True, False), (False, True), (True, True)])
+def test_ragged_transform_matches_oracle(oracle, shape, transpose, rht):
+    """Shapes that are not multiples of 16 (several of which the reference's backend refuses when
+    transposing): the result is that of quantizing the transposed, zero-completed tensor."""
+    x = make_input("randn", shape, 11)
+    for rule, two_d in (("mse", False), ("static_6", True)):
+        q = hip_quantize(x, scale_rule=rule, block_scale_2d=two_d, transpose=transpose, rht=rht)
+        ref = oracle.quantize(bits16(x), scale_rule=rule, block_scale_2d=two_d, transpose=transpose, rht=rht)
+        assert tuple(q.original_shape) == ((shape[1], shape[0]) if transpose else shape)
+        assert_same_quantization(q, ref, f"{shape} {rule} transpose={transpose} rht={rht}")
+
+
+def test_transform_reads_unaligned_rows():
+    """x whose rows start at odd element offsets takes the element-wise loads."""
+    from fouroversix_amd.quantize import ops
+
+    base = make_input("randn", (256, 264), 5).cuda()
+    x = base[:, 3:259]
+    t, amax = ops.transform(x, True, False)
+    assert torch.equal(t, x.T) and float(amax) == float(x.abs().max())
+    h, _ = ops.transform(x, False, True)
+    assert torch.equal(h, ops.transform(x.contiguous(), False, True)[0])
