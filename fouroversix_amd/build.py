@@ -20,7 +20,7 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libfouroversix_hip.so")
 OBJ_DIR = os.path.join(CSRC, "build")
 
-SOURCES = ["fos_common.hip", "fos_quantize.hip", "fos_quantize_fast.hip", "fos_gemm.hip", "fos_dequantize.hip", "fos_transform.hip", "fos_mxfp4.hip"]
+SOURCES = ["fos_common.hip", "fos_quantize.hip", "fos_quantize_fast.hip", "fos_quantize_tiles.hip", "fos_gemm.hip", "fos_dequantize.hip", "fos_transform.hip", "fos_mxfp4.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -82,8 +82,8 @@ FOS_DEVICE float candidate_residual(float fq, const FastLutEntry &e, float x) {
 //     |E_k - h_k^2 S~_k| <= h_k^2 * u * (330 sqrt(S_k) + 40 S_k)        (16 elements)
 // (5 roundings from amax to x*inv: 33u absolute on the scaled value; 7u on the reference's
 // residual; 16u relative on either sum; 256-element tiles multiply the two coefficients by
-// 4 and 16).  The kernel uses 2^-14 (sqrt(n/16) (1 + S) / 2 + (n/16) S) >= three times that
-// (sqrt(S) <= (1 + S) / 2) as the tolerance: when the two intervals do not overlap the comparison E_4 < E_6 is
+// 4 and 16).  The kernel uses 2^-14 ((1 + S) / 2 + S) for a block and 2^-14 (2 (1 + S) + 2 S) for a
+// tile, both >= three times that (sqrt(S) <= (1 + S) / 2), as the tolerance: when the two intervals do not overlap the comparison E_4 < E_6 is
 // decided by the shortcut, otherwise (a few blocks in 10^4 on real data; every block of a
 // tensor whose candidates tie exactly) the exact evaluation runs.
 
@@ -102,11 +102,11 @@ FOS_DEVICE float row16_sum_lane0(float v) {
 // scaled-domain sums (S already summed over the tile when TWO_D): returns +1 when the
 // second is surely smaller, -1 when it is surely not smaller (the first wins, also on a
 // tie), 0 when the two tolerance intervals overlap.
-// Tolerance 2^-14 (c1 sqrt(S) + c2 S) with sqrt(S) <= (1 + S) / 2.
+// Tolerance h (k0 + k1 S) per candidate.
 template <bool TWO_D>
 FOS_DEVICE int shortcut_compare(float SA, float hA, float SB, float hB) {
     constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
-    constexpr float k1 = (TWO_D ? 16.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
+    constexpr float k1 = (TWO_D ? 2.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
     // |EB - EA| against tA + tB (the differences and sums round within a few 2^-24 of
     // quantities that the tolerances exceed by 2^10)
     const float D = __builtin_fmaf(hB, SB, -(hA * SA));

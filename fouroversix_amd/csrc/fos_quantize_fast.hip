@@ -13,6 +13,7 @@
 //    workgroups walk over 128 x 64 tiles with the next tile prefetched.
 #include <cstdlib>
 
+#include "fos_buffer.h"
 #include "fos_quantize_kernel.h"
 #include "fos_tuning.h"
 
@@ -114,15 +115,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 }
 
 
-// Buffer resource (V#) over [base, base + bytes): raw 32-bit byte offsets, out-of-range
-// loads return zero.
-typedef __amdgpu_buffer_rsrc_t BufferRsrc;
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
-}
-
 // 1x16 blocks, row-contiguous mapping.  Workgroup tile: 128 rows x 256 columns, walked in
 // eight steps; in a step a wavefront covers 4 rows x 16 blocks (lane -> block column lane & 15
 // of row lane >> 4), i.e. 512 contiguous bytes per row.  Wavefront w owns rows
@@ -138,13 +130,6 @@ FOS_DEVICE BufferRsrc make_rsrc(const void *base, uint32_t bytes) {
 // ragged tile's descriptor ends with the tensor's last row and lanes past the last column
 // get an offset beyond it: both read zeros, which is the padding the reference adds.
 // FULL: rows % 128 == 0 and cols % 256 == 0, no bounds checks.
-// A wave-uniform 64-bit value, spelled so that the compiler keeps it in scalar registers (a
-// descriptor it believes to differ between lanes makes every buffer access a loop over lanes).
-FOS_DEVICE uint64_t uniform64(uint64_t v) {
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return ((uint64_t)hi << 32) | lo;
-}
-
 struct RowsTile {
     uint64_t x_base, codes_base, out_base;  // addresses of the tile's first input element / code byte / output element
     uint32_t x_bytes;    // extent of the input descriptor
@@ -337,6 +322,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 #endif
 }
 
+// 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): round to nearest, static and MSE rules.
+template <int RULE, bool PSEUDO>
+void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s);
+
 template <int RULE, bool PSEUDO, bool SR>
 static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     if (!aligned) {
@@ -348,9 +337,11 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     if (!two_d) {
         p.tiles_x = (int)((p.cols_p + 255) / 256);
         const int64_t n = (p.rows_p / 128) * p.tiles_x;
-        // five resident workgroups per compute unit (256 CUs, <= 102 VGPRs); more tiles than
-        // that are walked by the same workgroups.  FOS_QUANT_GRID overrides for tuning runs.
-        int64_t grid = 1280;
+        // three workgroups per compute unit (256 CUs), each walking several tiles: measured at
+        // 8192 x 8192 with the 4/6-MSE rule, 768 workgroups take 31.6 us where 1024 take 33.2 and the
+        // 1280 that fit (<= 102 VGPRs) 35.5 -- the setup is paid fewer times and the wavefronts stay
+        // in their streaming loop longer.  FOS_QUANT_GRID overrides for tuning runs.
+        int64_t grid = 768;
         if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
         if (grid > n) grid = n;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
@@ -358,6 +349,10 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        return;
+    }
+    if constexpr (!SR && (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_MSE)) {
+        launch_quantize_nvfp4_tiles<RULE, PSEUDO>(p, s);
         return;
     }
     p.tiles_x = (int)(p.cols_p / 64);

@@ -502,6 +502,10 @@ def test_pseudo_quantize_full_size():
     r = fos.quantize(x, cfg)
     e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(scale_rule="mse")), dtype=x.dtype)
     assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+    # 16x16 tiles: a few hundred of the 262144 take the undecided-tile path under the fused epilogue
+    r = fos.quantize(x, fos.QuantizationConfig(scale_rule="mse", block_scale_2d=True, pseudo_quantize=True))
+    e = fos.dequantize(fos.quantize(x, fos.QuantizationConfig(scale_rule="mse", block_scale_2d=True)), dtype=x.dtype)
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
     del e
     s6 = fos.QuantizationConfig(scale_rule="static_6", pseudo_quantize=True)
     once = fos.quantize(x, s6)
