@@ -19,6 +19,7 @@ void load_tuning() {
     g_tuning.mx_tile = env_int("FOS_MX_TILE");
     g_tuning.quant_grid = env_int("FOS_QUANT_GRID");
     g_tuning.amax_grid = env_int("FOS_AMAX_GRID");
+    g_tuning.quant_map = env_int("FOS_QUANT_MAP");
 }
 }  // namespace
 const Tuning &tuning() {

@@ -31,10 +31,33 @@ struct QuantParams {
     uint64_t seed, offset;
     int sf_layout;
     int tiles_x;                 // workgroup tiles along the columns
+    int tile_map = 0;            // TileMap: which tile the n-th unit of work is
     float c, qdiv, errdiv;       // f32(qmax*smax*adj), f32(qmax*adj), selection divisor
     uint16_t *pseudo_out;        // fused quantize -> dequantize: bf16 [rows, cols] output instead of codes / sf
     int64_t ldo;                 // its leading dimension
 };
+
+// Order in which the streaming kernels walk their tiles.  Workgroups are dealt to the eight
+// XCDs (each with its own L2) round-robin, so unit n runs on XCD n % 8.
+enum TileMap {
+    kMapRowMajor = 0,  // unit n = tile n, row-major: an XCD sees every eighth tile of each tile row
+    kMapBands = 1,     // XCD k walks the contiguous band of tiles [k n/8, (k+1) n/8) (needs n % 8 == 0)
+    kMapColMajor = 2,  // unit n = tile n, column-major
+    kMapBandsCol = 3,  // bands of the column-major order
+    kMapSplitHalves = 4,  // (16x16-tile kernel, with the above) a workgroup's two 256-column halves lie 2048 columns apart
+};
+
+FOS_DEVICE void map_tile(uint32_t unit, uint32_t n_tiles, uint32_t tiles_x, int map, uint32_t &tile_y, uint32_t &tile_x) {
+    if ((map & 1) && n_tiles % 8 == 0) unit = (unit & 7u) * (n_tiles >> 3) + (unit >> 3);
+    if (map & 2) {
+        const uint32_t tiles_y = n_tiles / tiles_x;
+        tile_x = unit / tiles_y;
+        tile_y = unit - tile_x * tiles_y;
+    } else {
+        tile_y = unit / tiles_x;
+        tile_x = unit - tile_y * tiles_x;
+    }
+}
 
 // ---- workgroup reductions ------------------------------------------------------------
 

@@ -165,8 +165,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
     auto open_tile = [&](uint32_t tile, bool valid) {
         RowsTile t;
-        t.tile_y = tile / (uint32_t)p.tiles_x;
-        t.tile_x = tile - t.tile_y * (uint32_t)p.tiles_x;
+        map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map, t.tile_y, t.tile_x);
         t.row_base = (int64_t)t.tile_y * 128;
         const int64_t col_base = (int64_t)t.tile_x * 256;
         t.cb = (int64_t)t.tile_x * 16 + lb;
@@ -197,7 +196,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         b.w[0] = lo.x; b.w[1] = lo.y; b.w[2] = lo.z; b.w[3] = lo.w;
         b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
     };
-    // the first input loads do not depend on the tensor maximum: they go out before the setup below
+    // pass-1 results first, the first input loads (which do not depend on them) right behind: loads
+    // return in order, so the setup below does not wait for the input
+    uint32_t pm[4] = {0u, 0u, 0u, 0u};
+    if (p.n_partials == 0) {
+        pm[0] = p.partials[0];
+    } else if (p.n_partials > 0) {
+#pragma unroll
+        for (int u = 0; u < kMaxPartials / kThreads; ++u)
+            if ((int)threadIdx.x + u * kThreads < p.n_partials) pm[u] = p.partials[2 * (threadIdx.x + u * kThreads)];
+    }
     uint32_t tile = blockIdx.x;
     RowsTile cur = open_tile(tile, tile < n_tiles);
     Block16 ring[4];
@@ -210,15 +218,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     load(cur, 1, ring[1]);
     load(cur, 2, ring[2]);
 
-    // pass-1 results behind them: one round trip to memory covers both
-    uint32_t pm[4] = {0u, 0u, 0u, 0u};
-    if (p.n_partials == 0) {
-        pm[0] = p.partials[0];
-    } else if (p.n_partials > 0) {
-#pragma unroll
-        for (int u = 0; u < kMaxPartials / kThreads; ++u)
-            if ((int)threadIdx.x + u * kThreads < p.n_partials) pm[u] = p.partials[2 * (threadIdx.x + u * kThreads)];
-    }
     // setup: tensor maximum, constants, per-scale table
     uint32_t amax_bits;
     if (p.n_partials == 0) amax_bits = pm[0];
@@ -344,6 +343,8 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         int64_t grid = 768;
         if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
         if (grid > n) grid = n;
+        p.tile_map = kMapRowMajor;
+        if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
         if (full)
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);

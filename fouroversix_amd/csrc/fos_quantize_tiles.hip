@@ -2,7 +2,7 @@
 // static_4 and 4/6-MSE, on the row-contiguous lane mapping of the 1x16 kernel: a wavefront
 // touches 4 rows x 512 contiguous bytes per step.
 //
-// Workgroup tile: 128 rows x 512 columns.  Wavefront w covers the 256 columns of half w >> 1 and
+// Workgroup tile: 128 rows x two windows of 256 columns.  Wavefront w covers window w >> 1 and
 // the 16-row bands of parity w & 1: rows 32 q + 16 (w & 1) + 4 s + i for group q = 0..3, step
 // s = 0..3 and i = lane >> 4; lane & 15 is the block column.  A lane therefore holds, per group,
 // the four 1x16 blocks of rows i, 4 + i, 8 + i, 12 + i of ONE 16x16 tile, and the tile's other
@@ -130,9 +130,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
     auto open_tile = [&](uint32_t tile, bool valid) {
         TilesPos t;
-        const uint32_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - tile_y * (uint32_t)p.tiles_x;
+        uint32_t tile_y, tile_x;
+        map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map, tile_y, tile_x);
         t.row0 = (int32_t)(tile_y * 128u) + 16 * par;
-        const int64_t col0 = (int64_t)tile_x * 512 + 256 * half;
+        // The two 256-column windows of a workgroup lie eight windows apart inside each complete run
+        // of sixteen (kMapSplitHalves; side by side otherwise and in what is left of a row): with
+        // row-major units an XCD then reads every eighth 512-byte window of a row, the pattern of the
+        // 1x16 kernel.  Measured at 8192 x 8192, 4/6-MSE: 37.8 us against 45.9 with the windows side
+        // by side and 39.2 with one band of tiles per XCD.
+        int64_t col0 = (int64_t)tile_x * 512 + 256 * half;
+        if ((p.tile_map & kMapSplitHalves) && tile_x < 8u * (uint32_t)(p.cols_p >> 12))
+            col0 = (int64_t)((tile_x >> 3) * 16 + (tile_x & 7u) + 8u * half) * 256;
         t.cb = (int32_t)(col0 >> 4) + lb;
         uint32_t x_bytes = valid ? 0xffffffffu : 0u;
         if (!FULL && valid) {
@@ -164,18 +172,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         b.w[4] = hi.x; b.w[5] = hi.y; b.w[6] = hi.z; b.w[7] = hi.w;
     };
 
-    // the first group's loads do not depend on the tensor maximum: they go out before the setup
-    uint32_t tile = blockIdx.x;
-    TilesPos cur = open_tile(tile, tile < n_tiles);
-    // Blocks 0 and 1 of a group alternate between two register sets (the next group's are loaded
-    // while this one is processed); blocks 2 and 3 have one set, consumed first and refilled at once
-    // with the next group's, half a group ahead of their use.
-    Block16 lo_a[2], lo_b[2], hi[2];
-    load(cur, 0, lo_a[0]);
-    load(cur, 4, lo_a[1]);
-    load(cur, 8, hi[0]);
-    load(cur, 12, hi[1]);
-
+    // pass-1 results first, the first group's loads (which do not depend on them) right behind:
+    // loads return in order, so the setup below does not wait for the group
     uint32_t pm[4] = {0u, 0u, 0u, 0u};
     if (p.n_partials == 0) {
         pm[0] = p.partials[0];
@@ -184,6 +182,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         for (int u = 0; u < kMaxPartials / kThreads; ++u)
             if ((int)threadIdx.x + u * kThreads < p.n_partials) pm[u] = p.partials[2 * (threadIdx.x + u * kThreads)];
     }
+    uint32_t tile = blockIdx.x;
+    TilesPos cur = open_tile(tile, tile < n_tiles);
+    // One register set holds a group; each block's registers are refilled with the next group's as
+    // soon as the block has been consumed.  (More loads in flight do not help: with a second set,
+    // or with three wavefronts per SIMD and deeper queues, the launch took as long or longer --
+    // wavefronts whose first loads were served late then finished late.)
+    Block16 blk[4];
+#ifdef FOS_TRACE
+    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime();
+    uint64_t tr_g[6] = {0, 0, 0, 0, 0, 0};
+    int tr_n = 0;
+#endif
+#pragma unroll
+    for (int s = 0; s < 4; ++s) load(cur, 4 * s, blk[s]);
+
     uint32_t amax_bits;
     if (p.n_partials == 0) amax_bits = pm[0];
     else if (p.n_partials > 0) amax_bits = block_max_u32(max(max(pm[0], pm[1]), max(pm[2], pm[3])), red);
@@ -205,6 +218,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
     __syncthreads();
 
+#ifdef FOS_TRACE
+    tr_g[tr_n++] = __builtin_amdgcn_s_memrealtime();  // setup done
+#endif
     // one quantised block (row `rstep` rows below the share's first, + li) to memory
     auto emit = [&](const TilesPos &t, uint32_t rstep, uint32_t c0, uint32_t c1, uint32_t sbyte, bool pred) {
         const int32_t row = t.row0 + (int32_t)rstep + li;
@@ -333,11 +349,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     };
 
     // one group: four blocks per lane in, codes (or dequantised values) out; returns the scale byte
-    auto process = [&](const TilesPos &t, uint32_t q, const Block16 (&lo)[2], Block16 (&lo_next)[2], const TilesPos &nt,
-                       uint32_t nq) -> uint32_t {
-        load(nt, 32 * nq, lo_next[0]);
-        load(nt, 32 * nq + 4, lo_next[1]);
-        auto blk = [&](int s) -> const Block16 & { return s < 2 ? lo[s] : hi[s - 2]; };
+    auto process = [&](const TilesPos &t, uint32_t q, const TilesPos &nt, uint32_t nq) -> uint32_t {
         const int32_t grow = t.row0 + 32 * (int32_t)q;  // first row of the group (wave-uniform)
         uint32_t oc[4][2] = {{0, 0}, {0, 0}, {0, 0}, {0, 0}}, os = 0;
         bool need_slow = false;
@@ -351,7 +363,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    bmax = fmaxf(fmaxf(fabsf(u2f(blk(s).w[j] << 16)), fabsf(u2f(blk(s).w[j]))), bmax);
+                    bmax = fmaxf(fmaxf(fabsf(u2f(blk[s].w[j] << 16)), fabsf(u2f(blk[s].w[j]))), bmax);
             bmax = tile_max(u2f(f2u(bmax) & 0xffff0000u));
             const float s_hp6 = div_const(bmax, k.qdiv, rq) * enc_fast;
             const float s_hp4 = s_hp6 * 1.5f;
@@ -366,12 +378,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const bool fast_ok = s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f);
             uint32_t cB[4][2];
             float SA = 0.0f, SB = 0.0f;
-            block_candidates<MSE>(hi[0], A.inv, B.inv, oc[2][0], oc[2][1], cB[2][0], cB[2][1], SA, SB);
-            block_candidates<MSE>(hi[1], A.inv, B.inv, oc[3][0], oc[3][1], cB[3][0], cB[3][1], SA, SB);
-            load(nt, 32 * nq + 8, hi[0]);
-            load(nt, 32 * nq + 12, hi[1]);
-            block_candidates<MSE>(lo[0], A.inv, B.inv, oc[0][0], oc[0][1], cB[0][0], cB[0][1], SA, SB);
-            block_candidates<MSE>(lo[1], A.inv, B.inv, oc[1][0], oc[1][1], cB[1][0], cB[1][1], SA, SB);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                block_candidates<MSE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
+                load(nt, 32 * nq + 4 * s, blk[s]);
+            }
             int cmp = -1;
             if (MSE) {
                 SA = tile_sum(SA);
@@ -404,8 +415,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 }
             }
         } else {
-            load(nt, 32 * nq + 8, hi[0]);
-            load(nt, 32 * nq + 12, hi[1]);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) load(nt, 32 * nq + 4 * s, blk[s]);
             need_slow = !padding && (FULL || t.cb < (int32_t)sf_cols);  // (not beyond the padded width)
         }
 #pragma unroll
@@ -427,9 +438,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         const TilesPos nxt = open_tile(has_next ? next : tile, has_next);  // without a next tile: loads of nothing
         uint32_t sw = 0;  // the lane's scale bytes of the four groups
 #pragma nounroll
-        for (uint32_t q = 0; q < 4; q += 2) {
-            sw |= process(cur, q, lo_a, lo_b, cur, q + 1) << (8 * q);
-            sw |= process(cur, q + 1, lo_b, lo_a, q == 0 ? cur : nxt, q == 0 ? 2u : 0u) << (8 * q + 8);
+        for (uint32_t q = 0; q < 4; ++q) {
+            sw |= process(cur, q, q == 3 ? nxt : cur, q == 3 ? 0u : q + 1) << (8 * q);
+#ifdef FOS_TRACE
+            if (tr_n < 6) tr_g[tr_n++] = __builtin_amdgcn_s_memrealtime();
+#endif
         }
         if (tiled) {
             // 16-byte unit of rows r, r + 32, r + 64, r + 96 and block columns 4 g .. 4 g + 3: word q =
@@ -446,6 +459,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         cur = nxt;
         tile = next;
     }
+#ifdef FOS_TRACE
+    if (lane == 0) {
+        // trace record behind the scale bytes: {start, end (100 MHz ticks), setup done, group ends...}
+        uint64_t *rec = reinterpret_cast<uint64_t *>(p.sf + p.rows_p * sf_cols) + (blockIdx.x * 4 + wave) * 8;
+        rec[0] = tr_t0;
+        rec[1] = __builtin_amdgcn_s_memrealtime();
+        for (int i = 0; i < 6; ++i) rec[2 + i] = tr_g[i];
+    }
+#endif
 }
 
 }  // namespace
@@ -460,6 +482,8 @@ void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s) {
     int64_t grid = 768;
     if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
     if (grid > n) grid = n;
+    p.tile_map = kMapSplitHalves;
+    if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
     const bool full = p.rows % 128 == 0 && p.cols % 512 == 0;
     if (full)
         hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
