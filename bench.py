@@ -105,6 +105,20 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
             x = fos.quantized_matmul(gate, layer["down"], input_config=acfg)
         return x
 
+    def step_amax():
+        # variant of step_shared: every GEMM records max|output|, so only x0 is reduced by a pass of its own
+        x = x0
+        for layer in weights:
+            qx = fos.quantize(x, acfg)
+            q = fos.quantized_matmul(qx, layer["q"], emit_amax=True)
+            fos.quantized_matmul(qx, layer["k"])
+            fos.quantized_matmul(qx, layer["v"])
+            qh = fos.quantize(fos.quantized_matmul(q, layer["o"], input_config=acfg, emit_amax=True), acfg)
+            gate = fos.quantized_matmul(qh, layer["gate"], emit_amax=True)
+            fos.quantized_matmul(qh, layer["up"])
+            x = fos.quantized_matmul(gate, layer["down"], input_config=acfg, emit_amax=True)
+        return x
+
     def timed(fn):
         for _ in range(warmup):
             fn()
@@ -117,6 +131,7 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
 
     sec = timed(step)
     sec_shared = timed(step_shared)
+    sec_amax = timed(step_amax)
     flops = 2.0 * tokens * sum(n * k for _, n, k in shapes) * layers
     return {
         "workload": f"{layers} layers x (q,k,v,o,gate,up,down) quantize+GEMM, {tokens} tokens, hidden {hidden}, "
@@ -125,6 +140,7 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
         "tokens_per_s": round(tokens / sec, 1),
         "TFLOP/s": round(flops / sec / 1e12, 1),
         "shared_activation_quantize": {"ms_per_step": round(sec_shared * 1e3, 3), "tokens_per_s": round(tokens / sec_shared, 1)},
+        "shared_and_gemm_recorded_amax": {"ms_per_step": round(sec_amax * 1e3, 3), "tokens_per_s": round(tokens / sec_amax, 1)},
     }
 
 

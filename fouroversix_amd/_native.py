@@ -34,6 +34,7 @@ EXPORTS = (
     "fos_transform",
     "fos_gemm_nvfp4",
     "fos_gemm_nvfp4_amax",
+    "fos_gemm_nvfp4_amax_out",
     "fos_gemm_mxfp4",
     "fos_gemm_alpha",
     "fos_padded_cols_for",
@@ -88,6 +89,8 @@ def lib() -> ctypes.CDLL:
     L.fos_gemm_nvfp4.restype = i32
     L.fos_gemm_nvfp4_amax.argtypes = [vp, vp, vp, vp, vp, vp, dbl, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4_amax.restype = i32
+    L.fos_gemm_nvfp4_amax_out.argtypes = [vp, vp, vp, vp, vp, vp, dbl, i64, i64, i64, vp, i32, i64, vp, vp, ctypes.c_size_t, vp]
+    L.fos_gemm_nvfp4_amax_out.restype = i32
     L.fos_gemm_alpha.argtypes = [vp, vp, dbl, vp, vp]
     L.fos_gemm_alpha.restype = i32
     L.fos_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp]

@@ -47,6 +47,7 @@ struct GemmParams {
     const float *amax_a, *amax_b;
     float inv_den;
     void *D;
+    float *d_amax;             // optional: max|D| as stored is folded into d_amax[0] (unsigned atomic max on the bits)
     int64_t M, N, K, ldd;
     int tiles_m, tiles_n;
     // split-K: workgroup (tile, blockIdx.y) contracts K steps [y * ksteps_per_split, ...) and
@@ -59,6 +60,26 @@ struct GemmParams {
 // arithmetic of gemm_alpha_kernel (product, then times the fp32 reciprocal of the divisor).
 FOS_DEVICE float load_alpha(const GemmParams &p) {
     return p.alpha ? *p.alpha : (*p.amax_a * *p.amax_b) * p.inv_den;
+}
+
+// max|D| for the caller that quantizes D next: `vmax` is the largest |alpha * acc| this lane
+// stored (0 for a lane that stored nothing).  Rounding to the output type is monotonic, so
+// the rounded maximum is the maximum of the rounded values.  One vector atomic per wavefront
+// on the unsigned image of the value (non-negative floats order like their bits); every lane
+// of the wavefront must call it.
+template <bool OUT_BF16>
+FOS_DEVICE void fold_amax(float *d_amax, float vmax) {
+    float r;
+    if (OUT_BF16) {
+        uint32_t u = f2u(vmax);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        r = u2f(u & 0xffff0000u);
+    } else {
+        r = (float)(_Float16)vmax;
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) r = fmaxf(r, __shfl_xor(r, off));
+    if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned int *>(d_amax), f2u(r));
 }
 
 // The two E4M3 bytes in the low 16 bits of `w` -> fp16 pair {s0, s1} (one hardware
@@ -315,6 +336,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     __syncthreads();  // every wavefront is done reading the A buffers
     uint8_t *epi = reinterpret_cast<uint8_t *>(lds) + wave * 32 * kEpiPitch;
     constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerPass = 64 / kLanesPerRow;
+    float vmax = 0.0f;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
@@ -325,6 +347,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float v = alpha * acc[i][j][4 * g + e];
+                    vmax = fmaxf(vmax, fabsf(v));
                     if (OUT_BF16) {
                         uint32_t u = f2u(v);
                         u += 0x7fffu + ((u >> 16) & 1u);
@@ -351,6 +374,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
+    if (p.d_amax) fold_amax<OUT_BF16>(p.d_amax, vmax);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -667,8 +691,10 @@ __global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1
     constexpr int kGroups = R == 2 ? 1 : R / 4;
     float *P = OUT == kOutPartial ? p.partials + (int64_t)blockIdx.y * p.M * p.N : nullptr;
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+    float vmax = 0.0f;
     auto to16 = [&](float v) -> uint32_t {
         v *= alpha;
+        vmax = fmaxf(vmax, fabsf(v));
         if (OUT == kOutBF16) {
             uint32_t u = f2u(v);
             u += 0x7fffu + ((u >> 16) & 1u);
@@ -694,6 +720,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1
                     make_uint2(to16(mine[4 * c]) | (to16(mine[4 * c + 1]) << 16), to16(mine[4 * c + 2]) | (to16(mine[4 * c + 3]) << 16));
         }
     }
+    if (OUT != kOutPartial && p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, vmax);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -840,24 +867,29 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
         }
         __syncthreads();
     }
-    if (wave != 0 || c >= p.M) return;
+    if (wave != 0) return;
+    const bool row_ok = c < p.M;  // rows beyond M are padding of the band and are not written
 
     const int64_t n_out = NB == 2 ? n128 + 64 * (g >> 1) + r0 + 4 * (g & 1)  // column of acc[0][0]; acc[1] is 32 further
                                   : n128 + 32 * g + r0;
     if (OUT == kOutPartial) {
         float *P = p.partials + (int64_t)blockIdx.y * p.M * p.N;
+        if (row_ok) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-            *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n_out + 32 * b) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+            for (int b = 0; b < NB; ++b)
+                *reinterpret_cast<float4 *>(P + (int64_t)c * p.N + n_out + 32 * b) = make_float4(acc[b][0], acc[b][1], acc[b][2], acc[b][3]);
+        }
         return;
     }
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
+    float vmax = 0.0f;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         uint16_t o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const float v = alpha * acc[b][e];
+            if (row_ok) vmax = fmaxf(vmax, fabsf(v));
             if (OUT == kOutBF16) {
                 uint32_t u = f2u(v);
                 u += 0x7fffu + ((u >> 16) & 1u);
@@ -866,17 +898,20 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
                 o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
             }
         }
-        *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n_out + 32 * b) =
-            make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+        if (row_ok)
+            *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n_out + 32 * b) =
+                make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
     }
+    if (p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, vmax);
 }
 
 // D = alpha * (sum of the split-K partial tiles, in split order), 4 consecutive n per thread.
 template <bool OUT_BF16>
 __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
     const int64_t quads = p.M * (p.N >> 2);
-    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (t >= quads) return;
+    const int64_t t_raw = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool mine = t_raw < quads;
+    const int64_t t = mine ? t_raw : 0;  // (idle lanes redo quad 0 and store nothing: every lane reaches fold_amax)
     const int64_t m = t / (p.N >> 2), n = (t - m * (p.N >> 2)) << 2;
     const float4 *P = reinterpret_cast<const float4 *>(p.partials + m * p.N + n);
     const int64_t stride = (p.M * p.N) >> 2;
@@ -898,8 +933,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
             o[e] = __builtin_bit_cast(uint16_t, (_Float16)v[e]);
         }
     }
-    *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.D) + m * p.ldd + n) =
-        make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+    if (mine)
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.D) + m * p.ldd + n) =
+            make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+    if (p.d_amax) {
+        const float vmax = mine ? fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))) : 0.0f;
+        fold_amax<OUT_BF16>(p.d_amax, vmax);
+    }
 }
 
 template <int WAVES_M, int WAVES_N, int WM, int WN>
@@ -1062,9 +1102,10 @@ extern "C" size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
                            const float *alpha, const float *amax_a, const float *amax_b, double denominator,
-                           int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd,
+                           int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, float *d_amax,
                            void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!A || !B || !sfA || !sfB || !D) return FOS_E_NULL_POINTER;
+    if ((uintptr_t)d_amax & 3) return FOS_E_BAD_ALIGNMENT;
     if (!alpha && (!amax_a || !amax_b)) return FOS_E_NULL_POINTER;
     if (!alpha && (((uintptr_t)amax_a & 3) || ((uintptr_t)amax_b & 3))) return FOS_E_BAD_ALIGNMENT;
     if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || N % 128 != 0 || K % 64 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
@@ -1075,7 +1116,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
         return FOS_E_BAD_ALIGNMENT;
     if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 22)) return FOS_E_BAD_SHAPE;  // a 256-row panel of packed codes stays below 2^31 bytes (32-bit buffer offsets)
     GemmParams p;
-    p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D;
+    p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D; p.d_amax = d_amax;
     p.amax_a = amax_a; p.amax_b = amax_b; p.inv_den = alpha ? 0.0f : (float)(1.0 / denominator);
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
@@ -1115,7 +1156,7 @@ extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
                               void *D, int out_type, int64_t ldd,
                               void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!alpha) return FOS_E_NULL_POINTER;
-    return gemm_nvfp4_impl(A, B, sfA, sfB, alpha, nullptr, nullptr, 1.0, M, N, K, D, out_type, ldd, workspace,
+    return gemm_nvfp4_impl(A, B, sfA, sfB, alpha, nullptr, nullptr, 1.0, M, N, K, D, out_type, ldd, nullptr, workspace,
                            workspace_bytes, stream);
 }
 
@@ -1125,6 +1166,16 @@ extern "C" int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uin
                                    void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!amax_a || !amax_b) return FOS_E_NULL_POINTER;
     if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
-    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, workspace,
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, nullptr, workspace,
+                           workspace_bytes, stream);
+}
+
+extern "C" int fos_gemm_nvfp4_amax_out(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                                       const float *amax_a, const float *amax_b, double denominator,
+                                       int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, float *d_amax,
+                                       void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!amax_a || !amax_b || !d_amax) return FOS_E_NULL_POINTER;
+    if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, d_amax, workspace,
                            workspace_bytes, stream);
 }

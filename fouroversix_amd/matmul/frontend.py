@@ -16,7 +16,7 @@ import torch
 
 from fouroversix_amd.quantize import QuantizationConfig, QuantizedTensor, quantize
 from fouroversix_amd.quantize import ops
-from fouroversix_amd.quantize.frontend import dequantize, dequantize_divisor
+from fouroversix_amd.quantize.frontend import attach_known_amax, dequantize, dequantize_divisor
 from fouroversix_amd.utils import NATIVE_FORMAT_IDS, DataType, MatmulBackend
 
 
@@ -85,7 +85,12 @@ def quantized_matmul(
     out_dtype: DataType = DataType.bfloat16,
     **kwargs: dict[str, Any],
 ) -> torch.Tensor:
-    """FP4 matrix product ``input @ other.T`` -> ``[M, N]`` tensor of ``out_dtype``."""
+    """FP4 matrix product ``input @ other.T`` -> ``[M, N]`` tensor of ``out_dtype``.
+
+    ``emit_amax=True`` (no counterpart in the reference) lets the NVFP4 GEMM record max|out| while
+    it stores it and attaches it to the result (``known_amax``), so that a following
+    ``quantize(out)`` skips its own reduction pass over the tensor."""
+    emit_amax = bool(kwargs.pop("emit_amax", False))
     del kwargs
     if isinstance(input, torch.Tensor):
         input = quantize(input, QuantizationConfig() if input_config is None else input_config)
@@ -136,10 +141,17 @@ def quantized_matmul(
     ):
         # the kernel forms alpha from the two maxima itself (same arithmetic, one launch less)
         den = dequantize_divisor(input) * dequantize_divisor(other)
+        d_amax = torch.zeros(1, dtype=torch.float32, device=a_values.device) if emit_amax else None
         out = ops.gemm_nvfp4_from_amax(
             a_values, other.values, input.scale_factors, other.scale_factors, a_amax, b_amax, den,
-            torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16,
+            torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16, d_amax,
         )
+        out_shape = (input.original_shape[0], other.original_shape[0])
+        if tuple(out.shape) != out_shape:
+            out = out[: out_shape[0], : out_shape[1]]  # (the padding is zeros: same maximum)
+        if d_amax is not None:
+            attach_known_amax(out, d_amax)
+        return out
     else:
         alpha = gemm_alpha(input, other)
         gemm = (

@@ -21,6 +21,7 @@ import torch.nn as nn
 
 from fouroversix_amd.matmul import quantized_matmul
 from fouroversix_amd.quantize import QuantizedTensor, dequantize, quantize
+from fouroversix_amd.quantize.frontend import attach_known_amax, known_amax
 from fouroversix_amd.utils import DataType
 
 from .config import ModuleQuantizationConfig
@@ -44,13 +45,23 @@ def fp4_linear(
             out = torch.matmul(quantize(flat, config.get_activation_config()), weight.T)
             out = out.reshape(*input.shape[:-1], weight.shape[0])
         else:
-            out = quantized_matmul(
+            # (a maximum recorded on `input` by the layer that produced it survives the flattening:
+            # a view shares the version counter)
+            amax_in = known_amax(input)
+            if amax_in is not None and flat is not input:
+                attach_known_amax(flat, amax_in)
+            out2d = quantized_matmul(
                 flat,
                 weight,
                 backend=config.matmul_backend,
                 input_config=config.get_activation_config(),
                 out_dtype=config.output_dtype,
-            ).reshape(*input.shape[:-1], weight.original_shape[0])
+                emit_amax=config.emit_output_amax and bias is None,
+            )
+            out = out2d.reshape(*input.shape[:-1], weight.original_shape[0])
+            amax_out = known_amax(out2d)
+            if amax_out is not None and out is not out2d:
+                attach_known_amax(out, amax_out)
     if bias is not None:
         out = out + bias
     return out

@@ -74,6 +74,26 @@ def _quantize_meta(x: torch.Tensor, config: QuantizationConfig) -> QuantizedTens
     )
 
 
+# max|x| that a producer already has (the FP4 GEMM can record it while storing its output): kept
+# as an attribute of the tensor object together with the tensor's version counter, so that an
+# in-place write, or any operation that returns a new tensor, drops it.
+_KNOWN_AMAX = "_fos_known_amax"
+
+
+def attach_known_amax(x: torch.Tensor, amax: torch.Tensor) -> torch.Tensor:
+    """Record ``amax`` (device f32[1] = max|x|) on ``x`` for a later ``quantize(x)``."""
+    setattr(x, _KNOWN_AMAX, (amax, x._version))
+    return x
+
+
+def known_amax(x: torch.Tensor) -> torch.Tensor | None:
+    """The maximum recorded by ``attach_known_amax`` if ``x`` has not been written since."""
+    tag = getattr(x, _KNOWN_AMAX, None)
+    if tag is None or tag[1] != x._version or tag[0].device != x.device:
+        return None
+    return tag[0]
+
+
 def quantize(
     x: torch.Tensor,
     config: QuantizationConfig | None = None,
@@ -123,7 +143,7 @@ def quantize(
         fmt, style = NATIVE_FORMAT_IDS[config.dtype.value], config.round_style.native_id
         if ops.pseudo_quantize_is_fused(x, fmt, style):
             return ops.pseudo_quantize(
-                x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax")
+                x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax", known_amax(x))
             )
         plain = QuantizationConfig(**{**config.__dict__, "pseudo_quantize": False})
         return dequantize(quantize(x, plain), dtype=x.dtype)
@@ -146,7 +166,7 @@ def quantize(
         seed,
         offset,
         nat.SF_LINEAR if linear else nat.SF_TILED,
-        None if config.dtype == DataType.mxfp4 else config.kwargs.get("amax"),  # mxfp4 has no tensor scale
+        None if config.dtype == DataType.mxfp4 else config.kwargs.get("amax", known_amax(x)),  # mxfp4 has no tensor scale
     )
     return QuantizedTensor(
         values,

@@ -209,9 +209,10 @@ def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selec
     return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, amax)
 
 
-def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None):
+def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None, d_amax=None):
     """``amax`` = (amax_a, amax_b, denominator) forms the output scale inside the kernel
-    (``alpha`` is then ignored and may be None)."""
+    (``alpha`` is then ignored and may be None); with it, ``d_amax`` (device f32[1], zero or an
+    earlier maximum) receives max|out|."""
     scale_tensors = (("alpha", alpha),) if amax is None else (("amax_a", amax[0]), ("amax_b", amax[1]))
     for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), *scale_tensors):
         nat.require_gpu_tensor(t, name)
@@ -250,6 +251,10 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None):
                 ws.data_ptr() if ws is not None else None, ws_bytes, nat.current_stream(a.device))
         if amax is None:
             rc = L.fos_gemm_nvfp4(a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(), alpha.data_ptr(), *tail)
+        elif d_amax is not None:
+            nat.require_gpu_tensor(d_amax, "d_amax")
+            rc = L.fos_gemm_nvfp4_amax_out(a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(),
+                                           amax[0].data_ptr(), amax[1].data_ptr(), float(amax[2]), *tail[:6], d_amax.data_ptr(), *tail[6:])
         else:
             rc = L.fos_gemm_nvfp4_amax(a.data_ptr(), b.data_ptr(), a_sf.data_ptr(), b_sf.data_ptr(),
                                        amax[0].data_ptr(), amax[1].data_ptr(), float(amax[2]), *tail)
@@ -421,10 +426,11 @@ def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
-def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype):
+def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax=None):
     """The NVFP4 GEMM with the output scale ``(amax_a * amax_b) * f32(1 / denominator)`` formed
-    in the kernel (``fos_gemm_nvfp4_amax``): one launch less than alpha + GEMM, same result."""
-    return _gemm_impl(a, b, a_sf, b_sf, None, out_dtype, amax=(amax_a, amax_b, denominator))
+    in the kernel (``fos_gemm_nvfp4_amax``): one launch less than alpha + GEMM, same result.
+    ``d_amax`` (device f32[1] holding 0) additionally receives max|out|."""
+    return _gemm_impl(a, b, a_sf, b_sf, None, out_dtype, amax=(amax_a, amax_b, denominator), d_amax=d_amax)
 
 
 def gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):

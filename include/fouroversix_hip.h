@@ -198,6 +198,20 @@ int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, 
                         void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * fos_gemm_nvfp4_amax that also folds max|D| -- of the values as stored, in the output type --
+ * into d_amax[0] (device f32[1]): every wavefront does an unsigned atomic max on the value's
+ * bits, so the caller sets d_amax[0] to 0 before the call (or leaves an earlier maximum there to
+ * extend it).  The next layer's activation quantization can then take d_amax as its
+ * `amax` input (amax_is_input = 1) and skip its own pass over D.  No counterpart in the
+ * reference, whose quantize op always reduces its input
+ * (src/fouroversix/quantize/pytorch/reference.py:573-600).
+ */
+int fos_gemm_nvfp4_amax_out(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                            const float *amax_a, const float *amax_b, double denominator,
+                            int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, float *d_amax,
+                            void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * alpha[0] = (amax_a[0] * amax_b[0]) * f32(1 / denominator), in fp32 on the device: the
  * GEMM's output scale as src/fouroversix/matmul/cutlass/backend.py:86-98 forms it on a GPU
  * (torch divides a tensor by a host scalar through the reciprocal, taken in double and

@@ -386,3 +386,67 @@ def test_linear_backward_on_the_fp4_gemm():
         layer.weight.grad = None
         layer(x).backward(g)
         assert rel(x.grad.reshape(-1, k), rx) < 0.25 and rel(layer.weight.grad, rw) < 0.25
+
+
+# ---- max|output| recorded by the GEMM -------------------------------------------------------
+
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float16"])
+@pytest.mark.parametrize(("m", "n", "k"), [(256, 256, 512), (1024, 4096, 1024), (8, 4096, 4096), (16, 1024, 8192), (48, 384, 1024),
+                                           (100, 384, 1024), (128, 1024, 4096), (128, 14336, 4096), (2048, 256, 192)])
+def test_gemm_records_the_output_maximum(m, n, k, out_dtype):
+    """Every kernel of the plan (tiles, the two weight-streaming kernels, the split-K reduction)
+    folds max|out| into the caller's word: equal to the maximum of what was stored, and the output
+    itself unchanged."""
+    a, b = make_input("randn", (m, k), 51).cuda(), make_input("weight", (n, k), 52).cuda()
+    qa, qb = fos.quantize(a), fos.quantize(b, fos.QuantizationConfig(block_scale_2d=True))
+    plain = fos.quantized_matmul(qa, qb, out_dtype=out_dtype)
+    out = fos.quantized_matmul(qa, qb, out_dtype=out_dtype, emit_amax=True)
+    assert torch.equal(out, plain)
+    amax = fos.quantize.__globals__["known_amax"](out)
+    assert amax is not None and amax.dtype == torch.float32
+    assert float(amax) == float(out.float().abs().max())
+
+
+def test_known_amax_follows_the_tensor():
+    """quantize() uses a recorded maximum exactly as long as the tensor is the one that was
+    measured: same result as measuring again; an in-place write or a new tensor drops it."""
+    from fouroversix_amd.quantize import attach_known_amax, known_amax
+
+    a, b = make_input("randn", (512, 1024), 53).cuda(), make_input("weight", (768, 1024), 54).cuda()
+    out = fos.quantized_matmul(a, b, emit_amax=True)
+    assert known_amax(out) is not None
+    q1, q2 = fos.quantize(out), fos.quantize(out.clone())
+    assert torch.equal(q1.values, q2.values) and torch.equal(q1.scale_factors.view(torch.uint8), q2.scale_factors.view(torch.uint8))
+    assert float(q1.amax) == float(q2.amax)
+    # a wrong recorded value would be used (that is the contract) ...
+    wrong = out.clone()
+    attach_known_amax(wrong, torch.full((1,), 2.0 * float(out.abs().max()), device="cuda"))
+    assert float(fos.quantize(wrong).amax) == 2.0 * float(out.float().abs().max())
+    # ... until the tensor is written
+    wrong.mul_(1.0)
+    assert known_amax(wrong) is None and float(fos.quantize(wrong).amax) == float(q2.amax)
+    assert known_amax(out * 1) is None and known_amax(out[:, :64]) is None
+
+
+def test_linear_layers_hand_the_maximum_on():
+    """emit_output_amax: a stack of layers gives bit-identical outputs with and without it."""
+    from fouroversix_amd.model import FourOverSixLinear, ModuleQuantizationConfig
+    from fouroversix_amd.quantize import known_amax
+
+    torch.manual_seed(3)
+    dims = [(1024, 512), (512, 768), (768, 256)]
+    mods = [nn.Linear(i, o, bias=False, device="cuda", dtype=torch.bfloat16) for i, o in dims]
+    x = make_input("randn", (4, 96, 1024), 55).cuda()
+    outs = []
+    for emit in (False, True):
+        cfg = ModuleQuantizationConfig(weight_scale_2d=True, emit_output_amax=emit)
+        y = x
+        for m in mods:
+            layer = FourOverSixLinear(nn.Linear(m.in_features, m.out_features, bias=False, device="cuda", dtype=torch.bfloat16), cfg)
+            layer.weight = nn.Parameter(m.weight.data.clone())
+            layer.quantize_weight_()
+            with torch.no_grad():
+                y = layer(y)
+            assert (known_amax(y) is not None) == emit
+        outs.append(y)
+    assert torch.equal(outs[0], outs[1])
