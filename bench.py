@@ -283,36 +283,33 @@ def main() -> int:
     stream = nat.current_stream(dev)
     counter = [0]
 
+    # each kernel's average launch duration: HIP events on the launch stream around K back-to-back
+    # launches of that kernel alone (an event between two different kernels would add the idle time
+    # of its own packet to both), inputs rotating, every buffer's maximum computed beforehand
+    amaxes = torch.zeros(n_buf, dtype=torch.float32, device=dev)
+
     def run_amax():
-        x = xs[counter[0] % n_buf]
-        nat.check(L.fos_amax(x.data_ptr(), 0, rows, cols, cols, amax.data_ptr(), ws.data_ptr(), ws_bytes, stream), "amax")
+        i = counter[0] % n_buf
+        counter[0] += 1
+        nat.check(L.fos_amax(xs[i].data_ptr(), 0, rows, cols, cols, amaxes[i:].data_ptr(), ws.data_ptr(), ws_bytes, stream), "amax")
 
     def run_quant_only():
-        x = xs[counter[0] % n_buf]
+        i = counter[0] % n_buf
         counter[0] += 1
-        nat.check(L.fos_quantize(x.data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(),
-                                 sf.data_ptr(), amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")
+        nat.check(L.fos_quantize(xs[i].data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(),
+                                 sf.data_ptr(), amaxes[i:].data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")
 
-    def run_both():
+    for _ in range(max(W, n_buf)):
         run_amax()
-        run_quant_only()
-
     for _ in range(W):
-        run_both()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3 * K)]
-    for i in range(K):
-        ev[3 * i].record()
-        run_amax()
-        ev[3 * i + 1].record()
         run_quant_only()
-        ev[3 * i + 2].record()
-    torch.cuda.synchronize()
-    amax_ms = sum(ev[3 * i].elapsed_time(ev[3 * i + 1]) for i in range(K)) / K
-    quant_ms = sum(ev[3 * i + 1].elapsed_time(ev[3 * i + 2]) for i in range(K)) / K
+    amax_ms = event_ms(run_amax, K)
+    quant_ms = event_ms(run_quant_only, K)
     counter[0] = 0
-    same_buffer_ms = event_ms(lambda: (run_amax(), nat.check(L.fos_quantize(
-        xs[0].data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(), sf.data_ptr(),
-        amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")), K)
+    same_buffer_ms = event_ms(lambda: (
+        nat.check(L.fos_amax(xs[0].data_ptr(), 0, rows, cols, cols, amax.data_ptr(), ws.data_ptr(), ws_bytes, stream), "amax"),
+        nat.check(L.fos_quantize(xs[0].data_ptr(), 0, rows, cols, cols, 0, 3, 0, 0, 0, 0, 1, codes.data_ptr(), sf.data_ptr(),
+                                 amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")), K)
     q_achieved = algo_bytes / (quant_ms * 1e-3) / 1e9
     roofline = {
         "kernel": "fos::quantize_nvfp4_rows_kernel<3, true, false, false> (pass 2: scale, 4/6 select, pack)",

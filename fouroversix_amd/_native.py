@@ -112,7 +112,10 @@ def check(code: int, what: str) -> None:
 
 
 def current_stream(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Handle of torch's current stream on ``device`` (the raw query: building a
+    ``torch.cuda.Stream`` object for it costs several microseconds per call)."""
+    index = device.index
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
 
 
 def require_gpu_tensor(t: torch.Tensor, name: str) -> None:

@@ -64,9 +64,9 @@ FOS_DEVICE float load_alpha(const GemmParams &p) {
 
 // max|D| for the caller that quantizes D next: `vmax` is the largest |alpha * acc| this lane
 // stored (0 for a lane that stored nothing).  Rounding to the output type is monotonic, so
-// the rounded maximum is the maximum of the rounded values.  One vector atomic per wavefront
-// on the unsigned image of the value (non-negative floats order like their bits); every lane
-// of the wavefront must call it.
+// the rounded maximum is the maximum of the rounded values.  At most one vector atomic per
+// wavefront on the unsigned image of the value (non-negative floats order like their bits);
+// every lane of the wavefront must call it.
 template <bool OUT_BF16>
 FOS_DEVICE void fold_amax(float *d_amax, float vmax) {
     float r;
@@ -79,7 +79,12 @@ FOS_DEVICE void fold_amax(float *d_amax, float vmax) {
     }
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) r = fmaxf(r, __shfl_xor(r, off));
-    if ((threadIdx.x & 63) == 0) atomicMax(reinterpret_cast<unsigned int *>(d_amax), f2u(r));
+    // (the atomics of a launch all go to one address and are served one after the other: a
+    // wavefront first looks whether its value would change anything -- only the first few do)
+    if ((threadIdx.x & 63) == 0) {
+        unsigned int *word = reinterpret_cast<unsigned int *>(d_amax);
+        if (f2u(r) > __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(word, f2u(r));
+    }
 }
 
 // The two E4M3 bytes in the low 16 bits of `w` -> fp16 pair {s0, s1} (one hardware

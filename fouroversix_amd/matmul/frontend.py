@@ -50,6 +50,24 @@ def _dequantize_form_applies(input: QuantizedTensor, other: QuantizedTensor, out
     )
 
 
+def _members_fit(q: QuantizedTensor, values: torch.Tensor) -> bool:
+    """The cheap form of the op's argument checks for the members of a QuantizedTensor: packed
+    codes and E4M3 scales of the padded shape (or its first rows), contiguous, on the GPU."""
+    rows_p, cols_p = q.padded_shape
+    sf = q.scale_factors
+    return (
+        values.dtype == torch.uint8
+        and values.dim() == 2
+        and values.shape[1] * 2 == cols_p
+        and (values.shape[0] == rows_p or (values.shape[0] < 128 == rows_p and cols_p % 256 == 0))
+        and values.is_contiguous()
+        and sf.dtype == torch.float8_e4m3fn
+        and sf.numel() * 16 == rows_p * cols_p
+        and sf.is_contiguous()
+        and sf.device == values.device
+    )
+
+
 _UNIT_ALPHA: dict = {}
 
 
@@ -93,9 +111,9 @@ def quantized_matmul(
     emit_amax = bool(kwargs.pop("emit_amax", False))
     del kwargs
     if isinstance(input, torch.Tensor):
-        input = quantize(input, QuantizationConfig() if input_config is None else input_config)
+        input = quantize(input, input_config)
     if isinstance(other, torch.Tensor):
-        other = quantize(other, QuantizationConfig() if other_config is None else other_config)
+        other = quantize(other, other_config)
     if isinstance(out_dtype, str):
         out_dtype = DataType(out_dtype)
 
@@ -145,6 +163,7 @@ def quantized_matmul(
         out = ops.gemm_nvfp4_from_amax(
             a_values, other.values, input.scale_factors, other.scale_factors, a_amax, b_amax, den,
             torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16, d_amax,
+            checked=_members_fit(input, a_values) and _members_fit(other, other.values),
         )
         out_shape = (input.original_shape[0], other.original_shape[0])
         if tuple(out.shape) != out_shape:

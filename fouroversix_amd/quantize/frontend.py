@@ -10,6 +10,9 @@ multiples, NVFP4 scales in the 128x4-tile layout, IF4 scales row-major, 0-dim fp
 
 from __future__ import annotations
 
+import functools
+import warnings
+
 import torch
 
 from fouroversix_amd import _native as nat
@@ -20,6 +23,7 @@ from .config import QuantizationConfig
 from .quantized_tensor import QuantizedTensor
 
 _LINEAR_SCALE_FORMATS = {DataType.if4, DataType.nvint4}
+_DEFAULT_CONFIG = QuantizationConfig()
 
 
 def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | None:
@@ -106,7 +110,7 @@ def quantize(
     ``amax`` (a tensor) to skip the tensor-wide maximum pass.
     """
     if config is None:
-        config = QuantizationConfig()
+        config = _DEFAULT_CONFIG  # (read only)
 
     if x.device.type == "meta" and x.dim() == 2:
         return _quantize_meta(x, config)
@@ -149,6 +153,13 @@ def quantize(
         return dequantize(quantize(x, plain), dtype=x.dtype)
 
     if config.round_style.is_stochastic and "seed" not in config.kwargs:
+        if x.is_cuda and torch.cuda.is_current_stream_capturing():
+            # the seed is a launch argument: a graph replays the one drawn now, every time
+            warnings.warn(
+                "stochastic rounding captured into a graph without kwargs['seed'] / kwargs['offset']: every replay "
+                "will round with the same random bits",
+                stacklevel=2,
+            )
         seed = int(torch.randint(0, 2**62, (1,)).item())
     else:
         seed = int(config.kwargs.get("seed", config.kwargs.get("rbits", 0)))
@@ -176,17 +187,23 @@ def quantize(
         tuple(x.shape),
         config.scale_rule,
         config.round_style,
+        (values.shape[0], values.shape[1] * config.dtype.quantized_value_type.packing_factor),  # as the kernel padded it
         scale_factors_are_in_blackwell_layout=not linear,
+    )
+
+
+@functools.lru_cache(maxsize=None)
+def _divisor(dtype: DataType, scale_rule, round_style) -> float:
+    return (
+        dtype.quantized_value_type.get_maximum_value(scale_rule)
+        * dtype.scale_type.get_maximum_value(scale_rule)
+        * round_style.adjustment_factor
     )
 
 
 def dequantize_divisor(tensor: QuantizedTensor) -> float:
     """qmax * smax * adjustment of the tensor's scale rule and rounding style."""
-    return (
-        tensor.dtype.quantized_value_type.get_maximum_value(tensor.scale_rule)
-        * tensor.dtype.scale_type.get_maximum_value(tensor.scale_rule)
-        * tensor.round_style.adjustment_factor
-    )
+    return _divisor(tensor.dtype, tensor.scale_rule, tensor.round_style)
 
 
 def dequantize(

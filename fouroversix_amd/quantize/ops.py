@@ -12,6 +12,8 @@ current stream.
 
 from __future__ import annotations
 
+import contextlib
+
 import torch
 
 from fouroversix_amd import _native as nat
@@ -46,38 +48,41 @@ def _padded(rows: int, cols: int, dtype: int = 0) -> tuple[int, int]:
 
 
 # Pass-1 workspace (8 KiB), one per (device, stream): calls on one stream are ordered, so
-# they can share it; calls on different streams must not.
+# they can share it; calls on different streams must not.  While a stream is being captured
+# into a graph the workspace comes from the allocator instead (the graph's private pool keeps
+# it for the graph's lifetime; a cached one would be shared by every graph captured on that
+# stream and pinned after they are gone).
 _WORKSPACES: dict[tuple[int, int], torch.Tensor] = {}
 _WS_BYTES = 0
 
 
 def _workspace(dev: torch.device, stream: int) -> torch.Tensor:
     global _WS_BYTES
+    if _WS_BYTES == 0:
+        _WS_BYTES = int(nat.lib().fos_quantize_workspace_bytes(1, 1))
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(_WS_BYTES, dtype=torch.uint8, device=dev)
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream)
     ws = _WORKSPACES.get(key)
     if ws is None:
-        if _WS_BYTES == 0:
-            _WS_BYTES = int(nat.lib().fos_quantize_workspace_bytes(1, 1))
         ws = torch.empty(_WS_BYTES, dtype=torch.uint8, device=dev)
         _WORKSPACES[key] = ws
     return ws
 
 
-class _on_device:
+_SAME_DEVICE = contextlib.nullcontext()
+
+
+def _on_device(dev: torch.device):
     """`with torch.cuda.device(dev)` only when `dev` is not already current."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(dev)
 
-    def __init__(self, dev: torch.device) -> None:
-        self.ctx = None
-        if dev.index is not None and dev.index != torch.cuda.current_device():
-            self.ctx = torch.cuda.device(dev)
 
-    def __enter__(self) -> None:
-        if self.ctx is not None:
-            self.ctx.__enter__()
-
-    def __exit__(self, *exc) -> None:
-        if self.ctx is not None:
-            self.ctx.__exit__(*exc)
+# split-K workspace size per GEMM shape (the library plans the shape once for the size and once
+# for the launch; the size never changes)
+_GEMM_WS_BYTES: dict[tuple[int, int, int], int] = {}
 
 
 def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
@@ -209,10 +214,16 @@ def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selec
     return _quantize_impl(x, 0, selection_rule, 0 if is_rtn else 1, is_2d, seed, 0, nat.SF_TILED, amax)
 
 
-def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None, d_amax=None):
+def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None, d_amax=None, checked=False):
     """``amax`` = (amax_a, amax_b, denominator) forms the output scale inside the kernel
     (``alpha`` is then ignored and may be None); with it, ``d_amax`` (device f32[1], zero or an
-    earlier maximum) receives max|out|."""
+    earlier maximum) receives max|out|.  ``checked``: the operands are the members of two
+    QuantizedTensors on one GPU (the frontend has looked): only the shapes are compared."""
+    if checked:
+        m, ka, n = a.shape[0], a.shape[1] * 2, b.shape[0]
+        if b.shape[1] * 2 != ka:
+            raise RuntimeError(f"Inner dims mismatch: {ka} vs {b.shape[1] * 2}")
+        return _gemm_launch(a, b, a_sf, b_sf, alpha, out_dtype, amax, d_amax, m, n, ka)
     scale_tensors = (("alpha", alpha),) if amax is None else (("amax_a", amax[0]), ("amax_b", amax[1]))
     for name, t in (("A", a), ("B", b), ("A_sf", a_sf), ("B_sf", b_sf), *scale_tensors):
         nat.require_gpu_tensor(t, name)
@@ -240,9 +251,15 @@ def _gemm_impl(a, b, a_sf, b_sf, alpha, out_dtype, amax=None, d_amax=None):
         raise RuntimeError("A with fewer than 128 rows needs K to be a multiple of 256")
     if b_sf.numel() * 16 != n * kb:
         raise RuntimeError("B_sf size mismatch")
+    return _gemm_launch(a, b, a_sf, b_sf, alpha, out_dtype, amax, d_amax, m, n, ka)
+
+
+def _gemm_launch(a, b, a_sf, b_sf, alpha, out_dtype, amax, d_amax, m, n, ka):
     out = torch.empty(m, n, dtype=out_dtype, device=a.device)
     L = nat.lib()
-    ws_bytes = int(L.fos_gemm_workspace_bytes(m, n, ka))
+    ws_bytes = _GEMM_WS_BYTES.get((m, n, ka))
+    if ws_bytes is None:
+        ws_bytes = _GEMM_WS_BYTES[(m, n, ka)] = int(L.fos_gemm_workspace_bytes(m, n, ka))
     with _on_device(a.device):
         # split-K partial tiles of small-M shapes; from torch's caching allocator, which
         # keeps the block tied to the current stream
@@ -426,11 +443,11 @@ def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
-def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax=None):
+def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax=None, checked=False):
     """The NVFP4 GEMM with the output scale ``(amax_a * amax_b) * f32(1 / denominator)`` formed
     in the kernel (``fos_gemm_nvfp4_amax``): one launch less than alpha + GEMM, same result.
     ``d_amax`` (device f32[1] holding 0) additionally receives max|out|."""
-    return _gemm_impl(a, b, a_sf, b_sf, None, out_dtype, amax=(amax_a, amax_b, denominator), d_amax=d_amax)
+    return _gemm_impl(a, b, a_sf, b_sf, None, out_dtype, amax=(amax_a, amax_b, denominator), d_amax=d_amax, checked=checked)
 
 
 def gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha, out_dtype=torch.bfloat16):

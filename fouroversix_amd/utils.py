@@ -221,17 +221,26 @@ def _scale_type(self: "DataType") -> ScaleType | None:
     return f.scale if f else None
 
 
-def _rules(self: "DataType") -> set[ScaleRule]:
+_RULES_CACHE: dict = {}
+
+
+def _rules(self: "DataType") -> frozenset[ScaleRule]:
+    cached = _RULES_CACHE.get(self)
+    if cached is not None:
+        return cached
     f = _fmt(self)
     if f is None:
-        return set()
-    if f.rules == "all":
-        return set(ScaleRule)
-    if f.rules == "static":
-        return {r for r in ScaleRule if r.is_static}
-    if f.rules == "adaptive":
-        return {r for r in ScaleRule if not r.is_static}
-    return {ScaleRule.static_6}
+        rules = frozenset()
+    elif f.rules == "all":
+        rules = frozenset(ScaleRule)
+    elif f.rules == "static":
+        rules = frozenset(r for r in ScaleRule if r.is_static)
+    elif f.rules == "adaptive":
+        rules = frozenset(r for r in ScaleRule if not r.is_static)
+    else:
+        rules = frozenset({ScaleRule.static_6})
+    _RULES_CACHE[self] = rules
+    return rules
 
 
 def _torch_dtype(self: "DataType") -> torch.dtype | None:
