@@ -47,16 +47,24 @@ enum TileMap {
     kMapSplitHalves = 4,  // (16x16-tile kernel, with the above) a workgroup's two 256-column halves lie 2048 columns apart
 };
 
-FOS_DEVICE void map_tile(uint32_t unit, uint32_t n_tiles, uint32_t tiles_x, int map, uint32_t &tile_y, uint32_t &tile_x) {
+struct TileYX {
+    uint32_t y, x;
+};
+
+// (returned by value: results handed back through references to members of a struct went
+// through a stack slot, which gave the kernels a private segment)
+FOS_DEVICE TileYX map_tile(uint32_t unit, uint32_t n_tiles, uint32_t tiles_x, int map) {
     if ((map & 1) && n_tiles % 8 == 0) unit = (unit & 7u) * (n_tiles >> 3) + (unit >> 3);
+    TileYX t;
     if (map & 2) {
         const uint32_t tiles_y = n_tiles / tiles_x;
-        tile_x = unit / tiles_y;
-        tile_y = unit - tile_x * tiles_y;
+        t.x = unit / tiles_y;
+        t.y = unit - t.x * tiles_y;
     } else {
-        tile_y = unit / tiles_x;
-        tile_x = unit - tile_y * tiles_x;
+        t.y = unit / tiles_x;
+        t.x = unit - t.y * tiles_x;
     }
+    return t;
 }
 
 // ---- workgroup reductions ------------------------------------------------------------

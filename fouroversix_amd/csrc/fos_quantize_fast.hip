@@ -140,7 +140,10 @@ struct RowsTile {
 };
 
 template <int RULE, bool FULL, bool PSEUDO, bool SR>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_rows_kernel(
+// (the stochastic instantiations hold two sets of scaled values and the Philox state: with 128
+// registers they spilled -- 30 MB of scratch traffic per launch at 8192 x 8192 -- and the launch
+// grid of three workgroups per compute unit leaves 168)
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3 : 4))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
     __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][128];  // per wavefront: 4 scale tiles x 128 bytes
@@ -165,7 +168,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
     auto open_tile = [&](uint32_t tile, bool valid) {
         RowsTile t;
-        map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map, t.tile_y, t.tile_x);
+        const TileYX yx = map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map);
+        t.tile_y = yx.y;
+        t.tile_x = yx.x;
         t.row_base = (int64_t)t.tile_y * 128;
         const int64_t col_base = (int64_t)t.tile_x * 256;
         t.cb = (int64_t)t.tile_x * 16 + lb;

@@ -130,8 +130,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
     auto open_tile = [&](uint32_t tile, bool valid) {
         TilesPos t;
-        uint32_t tile_y, tile_x;
-        map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map, tile_y, tile_x);
+        const TileYX yx = map_tile(tile, n_tiles, (uint32_t)p.tiles_x, p.tile_map);
+        const uint32_t tile_y = yx.y, tile_x = yx.x;
         t.row0 = (int32_t)(tile_y * 128u) + 16 * par;
         // The two 256-column windows of a workgroup lie eight windows apart inside each complete run
         // of sixteen (kMapSplitHalves; side by side otherwise and in what is left of a row): with
