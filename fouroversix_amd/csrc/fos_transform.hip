@@ -3,15 +3,18 @@
 // with the tensor maximum of y -- the steps the reference performs before it scales
 // (src/fouroversix/quantize/pytorch/reference.py:567-578; sign vector and matrix
 // src/fouroversix/quantize/utils.py:19-85; CUDA form src/fouroversix/csrc/include/
-// hadamard_transform.h:16-37).  The result is a plain bf16 matrix that fos_quantize then
-// reads with `amax_is_input`, so the whole option costs one extra write and read of x.
+// hadamard_transform.h:16-37).  The result is a plain matrix of the input's type (bf16 or
+// fp16) that fos_quantize then reads with `amax_is_input`, so the whole option costs one extra
+// write and read of x.
 //
 // RHT arithmetic: the reference multiplies bf16 [.., 16] by the bf16 matrix
 // diag(signs) * H16 / 4 with fp32 accumulation and one rounding to bf16.  All products are
 // exact, so the sum is evaluated here as a fast Walsh-Hadamard butterfly in fp32 (64 adds
 // instead of 256 multiply-adds) and scaled by 1/4 at the end; the two orders of summation
 // agree unless the fp32 partial sums themselves round, i.e. unless a group spans more
-// than ~12 binades, and then only when the last fp32 bit decides a bf16 rounding.
+// than ~12 binades, and then only when the last fp32 bit decides a bf16 rounding.  fp16 input:
+// the reference casts the matrix to the input's type (`had.to(x.dtype)`: +-1/4 is exact) and the
+// product is an fp16 matmul -- the same sum, rounded once to fp16.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -55,13 +58,21 @@ typedef __bf16 bf16x2_tt __attribute__((ext_vector_type(2)));
 constexpr uint32_t kRhtNegMask = (1u << 3) | (1u << 5) | (1u << 6) | (1u << 7) | (1u << 8) | (1u << 9) | (1u << 10) |
                                  (1u << 12) | (1u << 14) | (1u << 15);
 
-// w[0..7]: 16 bf16 (element 2j in the low half of w[j]) -> RHT -> 16 bf16, same packing.
+// w[0..7]: 16 bf16 / fp16 (element 2j in the low half of w[j]) -> RHT -> 16 of the same type, same packing.
+template <bool F16>
 FOS_DEVICE void rht16(uint32_t *w) {
     float v[16];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        v[2 * j] = u2f((w[j] << 16) ^ (((kRhtNegMask >> (2 * j)) & 1u) << 31));
-        v[2 * j + 1] = u2f((w[j] & 0xffff0000u) ^ (((kRhtNegMask >> (2 * j + 1)) & 1u) << 31));
+        if (F16) {
+            // the sign bit of the 16-bit pattern is flipped before the conversion
+            const uint32_t flipped = w[j] ^ (((kRhtNegMask >> (2 * j)) & 1u) << 15) ^ (((kRhtNegMask >> (2 * j + 1)) & 1u) << 31);
+            v[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(flipped & 0xffffu));
+            v[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(flipped >> 16));
+        } else {
+            v[2 * j] = u2f((w[j] << 16) ^ (((kRhtNegMask >> (2 * j)) & 1u) << 31));
+            v[2 * j + 1] = u2f((w[j] & 0xffff0000u) ^ (((kRhtNegMask >> (2 * j + 1)) & 1u) << 31));
+        }
     }
 #pragma unroll
     for (int len = 1; len < 16; len <<= 1) {
@@ -78,7 +89,10 @@ FOS_DEVICE void rht16(uint32_t *w) {
     for (int j = 0; j < 8; ++j) {
         // + 0.0f: a dot product accumulated from +0 never yields -0
         const float2_tt q = {v[2 * j] * 0.25f + 0.0f, v[2 * j + 1] * 0.25f + 0.0f};
-        w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_tt));
+        if (F16)
+            w[j] = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)q.x) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)q.y) << 16);
+        else
+            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_tt));
     }
 }
 
@@ -90,18 +104,21 @@ FOS_DEVICE void track(const uint32_t *w, uint32_t &m, uint32_t &z) {
     }
 }
 
+// (magnitudes of either 16-bit type order like their bit patterns)
+template <bool F16>
 FOS_DEVICE void write_partials(uint32_t m, uint32_t z, uint32_t *partials) {
     __shared__ uint32_t smem[4];
     uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
     mm = block_max_u32(mm, smem);
     const uint32_t zz = block_max_u32(((z & 0xffffu) == 0x8000u || (z >> 16) == 0x8000u) ? 1u : 0u, smem);
     if (threadIdx.x == 0) {
-        partials[2 * blockIdx.x] = mm << 16;
+        partials[2 * blockIdx.x] = F16 ? f2u((float)__builtin_bit_cast(_Float16, (uint16_t)mm)) : mm << 16;
         partials[2 * blockIdx.x + 1] = zz;
     }
 }
 
 // RHT without transposition: one thread per group of 16, grid-stride.
+template <bool F16>
 __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParams p) {
     const int64_t groups_per_row = (p.cols + 15) >> 4;  // a last, partial group is completed with zeros
     uint32_t m = 0, z = 0;
@@ -109,20 +126,20 @@ __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParam
         const int64_t r = g / groups_per_row, cb = g - r * groups_per_row;
         uint32_t w[8];
         load_group(p, r, cb * 16, w);
-        rht16(w);
+        rht16<F16>(w);
         track(w, m, z);
         uint4 *dst = reinterpret_cast<uint4 *>(p.y + r * p.ldy + cb * 16);
         dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
         dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
     }
-    write_partials(m, z, p.partials);
+    write_partials<F16>(m, z, p.partials);
 }
 
 // Transposition (optionally followed by the RHT along the new rows) through a 64 x 64 LDS
 // tile: rows of x come in as 128-byte runs, rows of y leave as 128-byte runs.  Groups of 16
 // that reach past the last row / column are completed with zeros (y is written in whole groups:
 // its rows hold a multiple of 16 elements).
-template <bool RHT>
+template <bool RHT, bool F16>
 __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformParams p) {
     constexpr int kPitchT = 66;  // halfs per LDS row: 33 dwords, odd, so a column walk changes bank every row
     __shared__ uint16_t tile[64 * kPitchT];
@@ -149,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
                     const uint32_t a = tile[(rb * 16 + 2 * j) * kPitchT + c], b = tile[(rb * 16 + 2 * j + 1) * kPitchT + c];
                     w[j] = a | (b << 16);
                 }
-                if (RHT) rht16(w);
+                if (RHT) rht16<F16>(w);
                 track(w, m, z);
                 uint4 *dst = reinterpret_cast<uint4 *>(p.y + (c0 + c) * p.ldy + r0 + rb * 16);
                 dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
@@ -158,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
         }
         __syncthreads();
     }
-    write_partials(m, z, p.partials);
+    write_partials<F16>(m, z, p.partials);
 }
 
 __global__ __launch_bounds__(kThreads) void transform_amax_kernel(const uint32_t *__restrict__ partials, int n,
@@ -179,7 +196,8 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
                              void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!x || !y || !amax) return FOS_E_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
-    if (x_type != FOS_T_BF16 || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
+    if ((x_type != FOS_T_BF16 && x_type != FOS_T_F16) || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
+    const bool f16 = x_type == FOS_T_F16;
     const int64_t out_cols = transpose ? rows : cols;
     // y is written in whole 16-element groups
     if (ldy < (out_cols + 15) / 16 * 16) return FOS_E_BAD_SHAPE;
@@ -200,14 +218,17 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
         p.tiles_x = (int)((cols + 63) / 64);
         p.n_units = ((rows + 63) / 64) * p.tiles_x;
         grid = p.n_units < kMaxGrid ? p.n_units : kMaxGrid;
-        if (rht) hipLaunchKernelGGL(transpose_kernel<true>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
-        else hipLaunchKernelGGL(transpose_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        if (rht && f16) hipLaunchKernelGGL((transpose_kernel<true, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else if (rht) hipLaunchKernelGGL((transpose_kernel<true, false>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else if (f16) hipLaunchKernelGGL((transpose_kernel<false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL((transpose_kernel<false, false>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     } else {
         p.tiles_x = 0;
         p.n_units = rows * ((cols + 15) / 16);
         grid = (p.n_units + kThreads - 1) / kThreads;
         if (grid > kMaxGrid) grid = kMaxGrid;
-        hipLaunchKernelGGL(rht_rows_kernel, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        if (f16) hipLaunchKernelGGL(rht_rows_kernel<true>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL(rht_rows_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     }
     hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s, p.partials, (int)grid, amax);
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;

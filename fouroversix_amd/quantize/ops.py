@@ -172,8 +172,8 @@ def transform_unsupported_reason(x: torch.Tensor, transpose: bool, rht: bool) ->
 
 def _transform_impl(x, transpose, rht):
     """``(y, amax)``: y = RHT(x^T) as the reference forms it before scaling, amax = max|y|."""
-    if x.dim() != 2 or x.dtype != torch.bfloat16:
-        raise RuntimeError("transform: x must be a 2-D bfloat16 tensor")
+    if x.dim() != 2 or x.dtype not in (torch.bfloat16, torch.float16):
+        raise RuntimeError("transform: x must be a 2-D bfloat16 or float16 tensor")
     nat.require_gpu_tensor(x, "x")
     reason = transform_unsupported_reason(x, transpose, rht)
     if reason is not None:
@@ -186,13 +186,13 @@ def _transform_impl(x, transpose, rht):
     # y is written in whole groups of 16 (zeros complete a ragged last group; with rht that group
     # then holds values in all 16 places, so the padded width is what gets quantized)
     width = -(-out_cols // 16) * 16
-    y = torch.empty((out_rows, width), dtype=torch.bfloat16, device=dev)
+    y = torch.empty((out_rows, width), dtype=x.dtype, device=dev)
     amax = torch.empty(1, dtype=torch.float32, device=dev)
     with _on_device(dev):
         stream = nat.current_stream(dev)
         workspace = _workspace(dev, stream)
         rc = nat.lib().fos_transform(
-            x.data_ptr(), nat.T_BF16, rows, cols, x.stride(0), int(transpose), int(rht),
+            x.data_ptr(), nat.TORCH_TO_T[x.dtype], rows, cols, x.stride(0), int(transpose), int(rht),
             y.data_ptr(), y.stride(0), amax.data_ptr(), workspace.data_ptr(), workspace.numel(), stream,
         )
     nat.check(rc, "fouroversix::transform")
@@ -205,8 +205,8 @@ def _quantize_ref_schema(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selec
     if not 0 <= selection_rule <= 4:
         raise RuntimeError(f"Invalid selection_rule: {selection_rule}")
     # the reference's native op takes fp16 and bf16 (csrc/quantize/fp4_quant.cu:134-136)
-    if x.dtype not in (torch.float16, torch.bfloat16) or (x.dtype != torch.bfloat16 and (is_rht or is_transpose)):
-        raise RuntimeError(f"quantize: x must be bfloat16 (or float16 without rht / transpose), got {x.dtype}")
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"quantize: x must be bfloat16 or float16, got {x.dtype}")
     seed = 0 if rbits < 0 else rbits
     amax = None
     if is_rht or is_transpose:

@@ -131,8 +131,9 @@ int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, i
 /*
  * Pre-transform of the training-side quantize options: y = x^T (transpose != 0) and / or
  * the 16-point random Hadamard transform of every group of 16 consecutive row elements
- * (rht != 0; fixed sign vector), written as a row-major bf16 matrix y ([cols, rows] when
- * transposed, else [rows, cols]; leading dimension ldy), and amax[0] = max |y|.  Stands in
+ * (rht != 0; fixed sign vector), written as a row-major matrix y of x's type (x_type
+ * FOS_T_BF16 or FOS_T_F16; [cols, rows] when transposed, else [rows, cols]; leading dimension
+ * ldy), and amax[0] = max |y|.  Stands in
  * for the `x.T` / `x.reshape(-1, 16) @ had` / `abs().max()` steps of the reference
  * quantizer (src/fouroversix/quantize/pytorch/reference.py:567-578,
  * quantize/utils.py:19-85; CUDA: csrc/include/hadamard_transform.h:16-37).  Follow it with

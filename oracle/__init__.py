@@ -181,26 +181,28 @@ def f32_to_bf16_bits(f: np.ndarray) -> np.ndarray:
     return ((u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
 
 
-def transform(xb: np.ndarray, *, transpose=False, rht=False) -> np.ndarray:
-    """bf16 bits of the tensor the reference quantizes when ``transpose`` / ``rht`` are set
-    (src/fouroversix/quantize/pytorch/reference.py:567-571): ``x.T``, then every group of 16
-    consecutive elements of a row times the RHT matrix as a bf16 matmul, i.e. exact
-    products, fp32 accumulation (here in the order i = 0..15), one rounding to bf16.  A ragged
-    width is first completed with zeros (the reference pads to its block multiples before the
-    transform, src/fouroversix/quantize/pytorch/backend.py:57-79), so with ``rht`` the result
-    is a multiple of 16 wide."""
+def transform(xb: np.ndarray, *, transpose=False, rht=False, x_type=0) -> np.ndarray:
+    """Bit patterns (bf16, or fp16 when ``x_type`` is 1) of the tensor the reference quantizes when
+    ``transpose`` / ``rht`` are set (src/fouroversix/quantize/pytorch/reference.py:567-571): ``x.T``,
+    then every group of 16 consecutive elements of a row times the RHT matrix cast to the input's
+    type, as a matmul of that type, i.e. exact products, fp32 accumulation (here in the order
+    i = 0..15), one rounding to the input's type.  A ragged width is first completed with zeros
+    (the reference pads to its block multiples before the transform,
+    src/fouroversix/quantize/pytorch/backend.py:57-79), so with ``rht`` the result is a multiple
+    of 16 wide."""
     xb = np.asarray(xb, dtype=np.uint16)
     if transpose:
         xb = np.ascontiguousarray(xb.T)
     if rht:
         if xb.shape[1] % 16:
             xb = np.pad(xb, ((0, 0), (0, 16 - xb.shape[1] % 16)))
-        g = bf16_bits_to_f32(xb).reshape(-1, 16)
+        g = (xb.view(np.float16).astype(np.float32) if x_type == 1 else bf16_bits_to_f32(xb)).reshape(-1, 16)
         h = rht_matrix()
         acc = np.zeros_like(g)
         for i in range(16):
             acc = acc + g[:, i:i + 1] * h[i][None, :]
-        xb = f32_to_bf16_bits(acc).reshape(xb.shape)
+        out = acc.astype(np.float16).view(np.uint16) if x_type == 1 else f32_to_bf16_bits(acc)
+        xb = out.reshape(xb.shape)
     return xb
 
 
@@ -210,8 +212,8 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
     xb, x_type = input_bits(x)
     assert xb.ndim == 2
     if transpose or rht:
-        assert x_type == 0, "transpose / rht: bf16 input only"
-        xb = transform(xb, transpose=transpose, rht=rht)
+        assert x_type in (0, 1), "transpose / rht: bf16 or fp16 input"
+        xb = transform(xb, transpose=transpose, rht=rht, x_type=x_type)
     orig = tuple(int(v) for v in xb.shape)
     xp = np.ascontiguousarray(pad_bits(xb))
     mp, np_ = xp.shape

@@ -134,6 +134,38 @@ def write_transform_vectors() -> None:
     print("wrote transform", len(out))
 
 
+def write_fp16_transform_vectors() -> None:
+    """The same options on fp16 tensors (values with 11 significant bits): the reference casts the
+    Hadamard matrix to the input's type and multiplies in that type
+    (quantize/pytorch/reference.py:570-571), then quantizes the fp16 result."""
+    from fouroversix.quantize.pytorch.reference import quantize as ref_quantize  # noqa: PLC0415
+    from fouroversix.quantize.utils import get_rht_matrix  # noqa: PLC0415
+    from fouroversix.utils import DataType, RoundStyle, ScaleRule  # noqa: PLC0415
+
+    had = get_rht_matrix(device="cpu")
+    out: dict[str, np.ndarray] = {}
+    for name, shape, seed, scale in [("randn_256x128", (256, 128), 61, 1.0), ("wide_128x256", (128, 256), 62, 40.0)]:
+        g = torch.Generator("cpu").manual_seed(seed)
+        x = (torch.randn(*shape, generator=g) * scale).half()
+        out[f"{name}.x"] = x.contiguous().view(torch.int16).numpy().view(np.uint16)
+        for transpose in (False, True):
+            for rht in (False, True):
+                if not transpose and not rht:
+                    continue
+                for rule, two_d in (("mse", False), ("static_6", True)):
+                    v, sf, amax = ref_quantize(
+                        x.clone(), had=had if rht else None, fp4_format=DataType.nvfp4,
+                        round_style=RoundStyle.nearest, scale_rule=ScaleRule(rule), block_scale_2d=two_d,
+                        transpose=transpose, use_blackwell_scale_layout=True,
+                    )
+                    key = f"{name}.t{int(transpose)}.h{int(rht)}.{rule}.{'2d' if two_d else '1d'}"
+                    out[key + ".values"] = u8(v)
+                    out[key + ".sf"] = u8(sf)
+                    out[key + ".amax"] = np.array([float(amax)], dtype=np.float32)
+    np.savez_compressed(os.path.join(HERE, "transform_fp16.npz"), **out)
+    print("wrote transform_fp16", len(out))
+
+
 def write_ragged_transpose_vectors(quantize, QuantizationConfig) -> None:  # noqa: N803
     """`transpose=True` on shapes that are not multiples of (128, 64), through the reference's
     PyTorch backend wrapper (quantize/pytorch/backend.py:57-79): it sizes the zero padding from
@@ -263,12 +295,16 @@ def main() -> None:
     ap.add_argument("--only-transform", action="store_true", help="write only transform.npz")
     ap.add_argument("--only-mxfp4", action="store_true", help="write only mxfp4.npz")
     ap.add_argument("--only-ragged-transpose", action="store_true", help="write only ragged_transpose.npz")
+    ap.add_argument("--only-transform-fp16", action="store_true", help="write only transform_fp16.npz")
     args = ap.parse_args()
 
     fos = import_reference()
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_fp16_transform_vectors()
+    if args.only_transform_fp16:
+        return
     write_ragged_transpose_vectors(quantize, QuantizationConfig)
     if args.only_ragged_transpose:
         return

@@ -106,6 +106,25 @@ def test_transform_options_match_reference_vectors(oracle, golden_dir):
     assert n == 27
 
 
+def test_fp16_transform_matches_reference_vectors(oracle, golden_dir):
+    """transpose / random-Hadamard on fp16 tensors: the reference multiplies by the matrix cast to
+    fp16 (quantize/pytorch/reference.py:570-571); vectors written by the reference function on CPU."""
+    d = np.load(os.path.join(golden_dir, "transform_fp16.npz"))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        base = key[: -len(".values")]
+        name, t, hh, rule, dim = base.split(".")
+        x = d[f"{name}.x"].view(np.float16)
+        q = oracle.quantize(x, scale_rule=rule, block_scale_2d=(dim == "2d"), transpose=(t == "t1"), rht=(hh == "h1"))
+        assert np.array_equal(q.values, d[base + ".values"]), base
+        assert np.array_equal(q.scale_factors, d[base + ".sf"].reshape(-1)), base
+        assert q.amax == d[base + ".amax"][0], base
+        n += 1
+    assert n == 12
+
+
 def test_ragged_transpose_matches_reference_vectors(oracle, golden_dir):
     """transpose=True on shapes outside the block multiples: where the reference's backend gets
     through (its padding is sized from the transposed shape but applied before the transpose,

@@ -123,9 +123,14 @@ def test_fp32_and_fp16_inputs_other_paths(oracle):
         assert torch.equal(out, fos.dequantize(q, dtype=t))
         q2 = fos.quantize(xt, fos.QuantizationConfig(kwargs={"amax": q.amax}))
         assert torch.equal(q2.values, q.values)
-        for bad in (dict(dtype="mxfp4", scale_rule="static_6"), dict(rht=True), dict(transpose=True)):
-            with pytest.raises(ValueError, match="bfloat16 input only"):
-                fos.quantize(xt, fos.QuantizationConfig(**bad))
+        with pytest.raises(ValueError, match="bfloat16 input only"):
+            fos.quantize(xt, fos.QuantizationConfig(dtype="mxfp4", scale_rule="static_6"))
+        for option in (dict(rht=True), dict(transpose=True)):
+            if t == torch.float32:
+                with pytest.raises(ValueError, match="bfloat16 or float16 input"):
+                    fos.quantize(xt, fos.QuantizationConfig(**option))
+            else:
+                assert fos.quantize(xt, fos.QuantizationConfig(**option)).original_shape == (128, 128)
     with pytest.raises(ValueError, match="bfloat16, float16 or float32"):
         fos.quantize(x.double().cuda())
 
@@ -602,6 +607,34 @@ def test_ragged_transform_matches_oracle(oracle, shape, transpose, rht):
         ref = oracle.quantize(bits16(x), scale_rule=rule, block_scale_2d=two_d, transpose=transpose, rht=rht)
         assert tuple(q.original_shape) == ((shape[1], shape[0]) if transpose else shape)
         assert_same_quantization(q, ref, f"{shape} {rule} transpose={transpose} rht={rht}")
+
+
+def test_fp16_transform_matches_reference_vectors_and_oracle(oracle, golden_dir):
+    """transpose / rht on fp16 tensors: the reference's vectors, then larger and ragged shapes
+    against the oracle."""
+    d = np.load(os.path.join(golden_dir, "transform_fp16.npz"))
+    n = 0
+    for key in d.files:
+        if not key.endswith(".values"):
+            continue
+        base = key[: -len(".values")]
+        name, t, hh, rule, dim = base.split(".")
+        x = torch.from_numpy(d[f"{name}.x"].view(np.float16).copy()).cuda()
+        q = fos.quantize(x, fos.QuantizationConfig(scale_rule=rule, block_scale_2d=(dim == "2d"), transpose=(t == "t1"), rht=(hh == "h1")))
+        assert np.array_equal(u8(q.values), d[base + ".values"]), base
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), d[base + ".sf"].reshape(-1)), base
+        assert float(q.amax) == float(d[base + ".amax"][0]), base
+        n += 1
+    assert n == 12
+    g = torch.Generator("cpu").manual_seed(9)
+    for shape in ((1024, 2048), (100, 200), (37, 50)):
+        x = (torch.randn(*shape, generator=g) * 3).half()
+        for transpose, rht in ((True, False), (False, True), (True, True)):
+            q = hip_quantize(x, transpose=transpose, rht=rht)
+            ref = oracle.quantize(x, transpose=transpose, rht=rht)
+            assert_same_quantization(q, ref, f"fp16 {shape} transpose={transpose} rht={rht}")
+    with pytest.raises(ValueError, match="float32"):
+        fos.quantize(torch.randn(64, 64, device="cuda"), fos.QuantizationConfig(rht=True))
 
 
 def test_transform_reads_unaligned_rows():
