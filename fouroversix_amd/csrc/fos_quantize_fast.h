@@ -98,21 +98,50 @@ FOS_DEVICE float row16_sum_lane0(float v) {
     return __shfl(v, lane & 48);
 }
 
-// Certified comparison of two candidates' errors h_a^2 S_a and h_b^2 S_b from their
-// scaled-domain sums (S already summed over the tile when TWO_D): returns +1 when the
-// second is surely smaller, -1 when it is surely not smaller (the first wins, also on a
-// tie), 0 when the two tolerance intervals overlap.
-// Tolerance h (k0 + k1 S) per candidate.
-template <bool TWO_D>
-FOS_DEVICE int shortcut_compare(float SA, float hA, float SB, float hB) {
-    constexpr float k0 = (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f;
-    constexpr float k1 = (TWO_D ? 2.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f;
+// Certified comparison of two candidates' errors from their scaled-domain reductions (S already
+// reduced over the tile when TWO_D): returns +1 when the second is surely smaller, -1 when it is
+// surely not smaller (the first wins, also on a tie), 0 when the two tolerance intervals overlap.
+// The weight w of a candidate is d1^2 (MSE) or d1 (MAE, abs-max); tolerance w (k0 + k1 S) each:
+//  * MSE: as derived above;
+//  * MAE, E = h sum |fq - x / h|: the 40u per element add up, 16 * 40u = 640u (256 * 40u for a
+//    tile), and the two summations and the products round with <= 40u S (520u S): three times
+//    that is below 2^-14 (2 + S / 8) resp. 2^-14 (32 + 2 S);
+//  * abs-max, E = h max |fq - x / h|: 40u and one rounding of the product, three times that is
+//    below 2^-17 whatever the block size.
+template <int RULE, bool TWO_D>
+FOS_DEVICE int shortcut_compare(float SA, float wA, float SB, float wB) {
+    constexpr float k0 = RULE == FOS_RULE_MSE ? (TWO_D ? 4.0f : 1.0f) * 0.5f * 0x1p-14f
+                         : RULE == FOS_RULE_MAE ? (TWO_D ? 32.0f : 2.0f) * 0x1p-14f
+                                                : 0x1p-17f;
+    constexpr float k1 = RULE == FOS_RULE_MSE ? (TWO_D ? 2.0f + 2.0f : 1.0f + 0.5f) * 0x1p-14f
+                         : RULE == FOS_RULE_MAE ? (TWO_D ? 2.0f : 0.125f) * 0x1p-14f
+                                                : 0.0f;
     // |EB - EA| against tA + tB (the differences and sums round within a few 2^-24 of
     // quantities that the tolerances exceed by 2^10)
-    const float D = __builtin_fmaf(hB, SB, -(hA * SA));
-    const float T = __builtin_fmaf(hA, __builtin_fmaf(k1, SA, k0), hB * __builtin_fmaf(k1, SB, k0));
+    const float D = __builtin_fmaf(wB, SB, -(wA * SA));
+    const float T = __builtin_fmaf(wA, __builtin_fmaf(k1, SA, k0), wB * __builtin_fmaf(k1, SB, k0));
     if (fabsf(D) > T) return D < 0.0f ? 1 : -1;
     return 0;
+}
+
+// One element pair's rounding residuals into the running reduction of a rule.
+template <int RULE>
+FOS_DEVICE void accumulate_scaled(float r0, float r1, float &S) {
+    if (RULE == FOS_RULE_MSE) {
+        S = __builtin_fmaf(r0, r0, S);
+        S = __builtin_fmaf(r1, r1, S);
+    } else if (RULE == FOS_RULE_MAE) {
+        S = S + fabsf(r0);
+        S = S + fabsf(r1);
+    } else {
+        S = fmaxf(fmaxf(fabsf(r0), fabsf(r1)), S);
+    }
+}
+
+// Weight of a candidate's scaled-domain reduction in its error.
+template <int RULE>
+FOS_DEVICE float shortcut_weight(const FastLutEntry &e) {
+    return RULE == FOS_RULE_MSE ? e.hh : e.d1;
 }
 
 // The two rare paths are real function calls (arguments and results by value, in
@@ -306,6 +335,11 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                                               bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
                                               uint64_t blkid) {
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
+    // the certified shortcut: MSE, and MAE for 1x16 blocks.  (Abs-max has one too, but 3 % of the
+    // blocks of N(0,1) data tie exactly under that rule -- the largest residual belongs to an
+    // element that both candidates represent by the same value -- so nearly every wavefront step
+    // ran the exact evaluation anyway and the shortcut only added to it: 55 us against 47.)
+    constexpr bool SHORTCUT = RULE == FOS_RULE_MSE || (RULE == FOS_RULE_MAE && !TWO_D);
     if (in_range) {
         float x[16];
 #pragma unroll
@@ -355,24 +389,20 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 uint32_t b0, b1;
                 sr_pack16(xb, pB, b0, b1);
                 bool pickB = false, certain = false;
-                if (RULE == FOS_RULE_MSE) {
+                if (SHORTCUT) {
                     float SA = 0.0f, SB = 0.0f;
                     static_for<0, 8>([&](auto jc) {
                         constexpr int j = decltype(jc)::value;
                         const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
                         const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
-                        const float ra0 = fa.x - xa[2 * j], ra1 = fa.y - xa[2 * j + 1];
-                        const float rb0 = fb.x - xb[2 * j], rb1 = fb.y - xb[2 * j + 1];
-                        SA = __builtin_fmaf(ra0, ra0, SA);
-                        SA = __builtin_fmaf(ra1, ra1, SA);
-                        SB = __builtin_fmaf(rb0, rb0, SB);
-                        SB = __builtin_fmaf(rb1, rb1, SB);
+                        accumulate_scaled<RULE>(fa.x - xa[2 * j], fa.y - xa[2 * j + 1], SA);
+                        accumulate_scaled<RULE>(fb.x - xb[2 * j], fb.y - xb[2 * j + 1], SB);
                     });
                     if (TWO_D) {
                         SA = row16_sum_lane0(SA);
                         SB = row16_sum_lane0(SB);
                     }
-                    const int cmp = shortcut_compare<TWO_D>(SA, A.hh, SB, B.hh);
+                    const int cmp = shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
                     certain = cmp != 0;
                     pickB = cmp > 0;
                 }
@@ -410,23 +440,20 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     a1 = pack_fp4<(j & 3)>(a1, xa0, xa1);
                     b1 = pack_fp4<(j & 3)>(b1, xb0, xb1);
                 }
-                if (RULE == FOS_RULE_MSE) {
+                if (SHORTCUT) {
                     const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
                     const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
-                    const float ra0 = fa.x - xa0, ra1 = fa.y - xa1, rb0 = fb.x - xb0, rb1 = fb.y - xb1;
-                    SA = __builtin_fmaf(ra0, ra0, SA);
-                    SA = __builtin_fmaf(ra1, ra1, SA);
-                    SB = __builtin_fmaf(rb0, rb0, SB);
-                    SB = __builtin_fmaf(rb1, rb1, SB);
+                    accumulate_scaled<RULE>(fa.x - xa0, fa.y - xa1, SA);
+                    accumulate_scaled<RULE>(fb.x - xb0, fb.y - xb1, SB);
                 }
             });
             bool pickB = false, certain = false;
-            if (RULE == FOS_RULE_MSE) {
+            if (SHORTCUT) {
                 if (TWO_D) {
                     SA = row16_sum_lane0(SA);
                     SB = row16_sum_lane0(SB);
                 }
-                const int cmp = shortcut_compare<TWO_D>(SA, A.hh, SB, B.hh);
+                const int cmp = shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
                 certain = cmp != 0;
                 pickB = cmp > 0;
             }
@@ -514,7 +541,7 @@ FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts
                 SA = row16_sum_lane0(SA);
                 SB = row16_sum_lane0(SB);
             }
-            const int cmp = shortcut_compare<TWO_D>(SA, 1.0f, SB, 1.0f);  // same scale: compare the sums
+            const int cmp = shortcut_compare<FOS_RULE_MSE, TWO_D>(SA, 1.0f, SB, 1.0f);  // same scale: compare the sums
             if (cmp > 0) return BlockOut{b0, b1, s | 0x80u};
             if (cmp < 0) return BlockOut{a0, a1, s};
             // undecided (uniform over the 16 lanes of a tile when TWO_D: both sums are tile sums)

@@ -326,7 +326,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3
 #endif
 }
 
-// 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): round to nearest, static and MSE rules.
+// 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): round to nearest, every rule.
 template <int RULE, bool PSEUDO>
 void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s);
 
@@ -357,7 +357,7 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         return;
     }
-    if constexpr (!SR && (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_MSE)) {
+    if constexpr (!SR) {
         launch_quantize_nvfp4_tiles<RULE, PSEUDO>(p, s);
         return;
     }

@@ -1,5 +1,5 @@
 // Pass 2 for NVFP4 with 16x16 scale tiles (block_scale_2d), round to nearest, rules static_6 /
-// static_4 and 4/6-MSE, on the row-contiguous lane mapping of the 1x16 kernel: a wavefront
+// static_4 and 4/6 with the MSE, MAE or abs-max rule, on the row-contiguous lane mapping of the 1x16 kernel: a wavefront
 // touches 4 rows x 512 contiguous bytes per step.
 //
 // Workgroup tile: 128 rows x two windows of 256 columns.  Wavefront w covers window w >> 1 and
@@ -61,9 +61,9 @@ FOS_DEVICE uint32_t tile_or(uint32_t v) {
     return a | b;
 }
 
-// Both candidates of one block in the scaled domain: codes, and (MSE) the sums of squared
-// rounding residuals added to SA / SB.
-template <bool MSE>
+// Both candidates of one block in the scaled domain: codes, and (adaptive rules) the rule's
+// reduction of the rounding residuals added to SA / SB.
+template <int RULE>
 FOS_DEVICE void block_candidates(const Block16 &blk, float invA, float invB, uint32_t &a0, uint32_t &a1, uint32_t &b0,
                                  uint32_t &b1, float &SA, float &SB) {
     a0 = a1 = b0 = b1 = 0;
@@ -73,17 +73,14 @@ FOS_DEVICE void block_candidates(const Block16 &blk, float invA, float invB, uin
         const float xa0 = scaled(x0, invA), xa1 = scaled(x1, invA);
         if (j < 4) a0 = pack_fp4<(j & 3)>(a0, xa0, xa1);
         else a1 = pack_fp4<(j & 3)>(a1, xa0, xa1);
-        if (MSE) {
+        if (RULE != FOS_RULE_STATIC_6) {
             const float xb0 = scaled(x0, invB), xb1 = scaled(x1, invB);
             if (j < 4) b0 = pack_fp4<(j & 3)>(b0, xb0, xb1);
             else b1 = pack_fp4<(j & 3)>(b1, xb0, xb1);
             const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
             const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
-            const float ra0 = fa.x - xa0, ra1 = fa.y - xa1, rb0 = fb.x - xb0, rb1 = fb.y - xb1;
-            SA = __builtin_fmaf(ra0, ra0, SA);
-            SA = __builtin_fmaf(ra1, ra1, SA);
-            SB = __builtin_fmaf(rb0, rb0, SB);
-            SB = __builtin_fmaf(rb1, rb1, SB);
+            accumulate_scaled<RULE>(fa.x - xa0, fa.y - xa1, SA);
+            accumulate_scaled<RULE>(fb.x - xb0, fb.y - xb1, SB);
         }
     });
 }
@@ -109,8 +106,8 @@ template <int RULE, bool FULL, bool PSEUDO>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_tiles_kernel(
     const QuantParams p) {
     constexpr bool STATIC = RULE == FOS_RULE_STATIC_6;
-    constexpr bool MSE = RULE == FOS_RULE_MSE;
-    static_assert(STATIC || MSE, "the other adaptive rules have no certified shortcut and stay on the DPP-row kernel");
+    constexpr bool ADAPTIVE = !STATIC;            // 4/6 with the MSE, MAE or abs-max rule
+    constexpr bool MAXRULE = RULE == FOS_RULE_ABS_MAX;  // the error is the largest term, not the sum
     __shared__ uint32_t red[4];
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
@@ -287,19 +284,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 const float xs = (sX != 0) ? x[m] * invX : 0.0f;
                 const float r = e2m1_round(fabsf(xs));
                 const float e = error_term<RULE>(div_errdiv(((xs < 0.0f ? -r : r) * sfX) * k.amax, k), x[m]);
-                chain = m == 0 ? e : chain + e;
+                chain = m == 0 ? e : (MAXRULE ? fmaxf(chain, e) : chain + e);
             }
-            // lanes 0..7 of DPP rows 0 (candidate "6") and 2 (candidate "4"): E[l] own, E[l+8] eight lanes
-            // on, O[l] and O[l+8] in the next DPP row
-            const float chain8 = dpp_move<kDppRowShl + 8>(0.0f, chain);
-            uint32_t ev, od, ev8, od8;
-            rows_pairs(f2u(chain), ev, od);
-            rows_pairs(f2u(chain8), ev8, od8);
-            const float a = ((chain + chain8) + u2f(od)) + u2f(od8);
-            float tot = a;
+            float tot_a, tot_b;
+            if (MAXRULE) {
+                // the largest term of each candidate's 32 lanes
 #pragma unroll
-            for (int step = 0; step < 7; ++step) tot = dpp_move<kDppRowShr + 1>(-0.0f, tot) + a;  // lane 7: ((a0 + a1) + ...) + a7
-            const float tot_a = u2f(__builtin_amdgcn_readlane(f2u(tot), 7)), tot_b = u2f(__builtin_amdgcn_readlane(f2u(tot), 39));
+                for (int off = 16; off >= 1; off >>= 1) chain = fmaxf(chain, __shfl_xor(chain, off));
+                tot_a = u2f(__builtin_amdgcn_readlane(f2u(chain), 0));
+                tot_b = u2f(__builtin_amdgcn_readlane(f2u(chain), 32));
+            } else {
+                // lanes 0..7 of DPP rows 0 (candidate "6") and 2 (candidate "4"): E[l] own, E[l+8] eight lanes
+                // on, O[l] and O[l+8] in the next DPP row
+                const float chain8 = dpp_move<kDppRowShl + 8>(0.0f, chain);
+                uint32_t ev, od, ev8, od8;
+                rows_pairs(f2u(chain), ev, od);
+                rows_pairs(f2u(chain8), ev8, od8);
+                const float a = ((chain + chain8) + u2f(od)) + u2f(od8);
+                float tot = a;
+#pragma unroll
+                for (int step = 0; step < 7; ++step) tot = dpp_move<kDppRowShr + 1>(-0.0f, tot) + a;  // lane 7: ((a0 + a1) + ...) + a7
+                tot_a = u2f(__builtin_amdgcn_readlane(f2u(tot), 7));
+                tot_b = u2f(__builtin_amdgcn_readlane(f2u(tot), 39));
+            }
             pickB = tot_b < tot_a;
         }
         const uint32_t src_lane = pickB ? 32 : 0;
@@ -371,7 +378,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
             const FastLutEntry A = lut[s6];
             FastLutEntry B = A;
-            if (MSE) B = lut[s4];
+            if (ADAPTIVE) B = lut[s4];
             // the hardware convert saturates at 6 where the reference's unclamped rounding gives 8:
             // that needs a sub-normal scale byte rounded down by more than 7/6; a zero scale byte
             // of a non-zero tile has no scaled domain
@@ -380,18 +387,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             float SA = 0.0f, SB = 0.0f;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                block_candidates<MSE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
+                block_candidates<RULE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 load(nt, 32 * nq + 4 * s, blk[s]);
             }
             int cmp = -1;
-            if (MSE) {
-                SA = tile_sum(SA);
-                SB = tile_sum(SB);
-                cmp = shortcut_compare<true>(SA, A.hh, SB, B.hh);
+            if (ADAPTIVE) {
+                SA = MAXRULE ? tile_max(SA) : tile_sum(SA);
+                SB = MAXRULE ? tile_max(SB) : tile_sum(SB);
+                cmp = shortcut_compare<RULE, true>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
             }
             // an all-zero tile came out as zero codes under the zero scale byte
             need_slow = !(bmax == 0.0f || (fast_ok && cmp != 0));
-            if (MSE && __builtin_amdgcn_ballot_w64(need_slow) != 0) {
+            if (ADAPTIVE && __builtin_amdgcn_ballot_w64(need_slow) != 0) {
                 // candidates that dequantise to the same values element by element tie: "6" wins
                 uint32_t viol = 1u;
                 if (fast_ok && e4m3_decode(s4) == 1.5f * e4m3_decode(s6)) {
@@ -405,9 +412,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                     need_slow = false;
                 }
             }
-            const bool pickB = MSE && cmp > 0;
+            const bool pickB = ADAPTIVE && cmp > 0;
             os = pickB ? s4 : s6;
-            if (MSE) {
+            if (ADAPTIVE) {
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
                     oc[s][0] = pickB ? cB[s][0] : oc[s][0];
@@ -495,5 +502,9 @@ template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, false>(QuantParams 
 template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, true>(QuantParams &, hipStream_t);
 template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, false>(QuantParams &, hipStream_t);
 template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, true>(QuantParams &, hipStream_t);
 
 }  // namespace fos
