@@ -139,7 +139,9 @@ struct RowsTile {
     uint32_t tile_y, tile_x;
 };
 
-template <int RULE, bool FULL, bool PSEUDO, bool SR>
+// IF4: the IF4 format with its MSE rule (E2M1 candidate against INT4 candidate on one scale,
+// quantize_block_if4_mse) instead of NVFP4.
+template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false>
 // (the stochastic instantiations hold two sets of scaled values and the Philox state: with 128
 // registers they spilled -- 30 MB of scratch traffic per launch at 8192 x 8192 -- and the launch
 // grid of three workgroups per compute unit leaves 168)
@@ -249,9 +251,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3
         // writes its zero codes and scales
         const bool padding_step = !FULL && t.row_base + step_row(g) + wave * 8 >= p.rows;
         BlockOut o{0u, 0u, 0u};
-        if (!padding_step)
-            o = quantize_block_nvfp4_fast<RULE, false, SR>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
-                                                           (uint64_t)(row * sf_cols + t.cb));
+        if (!padding_step) {
+            if constexpr (IF4) o = quantize_block_if4_mse<false>(b, k, enc_fast, rq, in_range, lut);
+            else o = quantize_block_nvfp4_fast<RULE, false, SR>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                                                                (uint64_t)(row * sf_cols + t.cb));
+        }
         if (PSEUDO) {
             uint32_t w[8];
             if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
@@ -383,6 +387,21 @@ static void by_rule(QuantParams &p, int rule, bool two_d, bool aligned, hipStrea
         case FOS_RULE_MSE: by_dim<FOS_RULE_MSE, PSEUDO, SR>(p, two_d, aligned, s); break;
         default: by_dim<FOS_RULE_ABS_MAX, PSEUDO, SR>(p, two_d, aligned, s); break;
     }
+}
+
+// IF4 with the MSE rule, round to nearest, 1x16 blocks, aligned input: the streaming kernel.
+void launch_quantize_if4_mse_rows(QuantParams &p, hipStream_t s) {
+    p.tiles_x = (int)((p.cols_p + 255) / 256);
+    const int64_t n = (p.rows_p / 128) * p.tiles_x;
+    int64_t grid = 768;
+    if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
+    if (grid > n) grid = n;
+    p.tile_map = kMapRowMajor;
+    if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
+    if (p.rows % 128 == 0 && p.cols % 256 == 0)
+        hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, true, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
 // `sr`: a stochastic style on an aligned input.  The fast exact evaluation is tied to the
