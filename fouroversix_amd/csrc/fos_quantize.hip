@@ -245,7 +245,8 @@ void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, h
         } else if constexpr (RULE == FOS_RULE_MSE) {
             // IF4 with the MSE rule: fast block formulation, on the streaming kernel for aligned 1x16
             // inputs and inside the generic kernel's mapping otherwise
-            if (two_d) launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
+            if (two_d && aligned && !p.pseudo_out) launch_quantize_if4_mse_tiles(p, s);
+            else if (two_d) launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
             else if (aligned && !p.pseudo_out) launch_quantize_if4_mse_rows(p, s);
             else launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
         } else {

@@ -172,6 +172,7 @@ void launch_quantize(QuantParams &p, bool aligned, hipStream_t s) {
 // only) a stochastic style.
 void launch_quantize_nvfp4_fast(QuantParams &p, int rule, bool two_d, bool aligned, bool sr, hipStream_t s);
 void launch_quantize_if4_mse_rows(QuantParams &p, hipStream_t s);
+void launch_quantize_if4_mse_tiles(QuantParams &p, hipStream_t s);
 
 // MXFP4 (fos_mxfp4.hip)
 int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,

@@ -85,6 +85,30 @@ FOS_DEVICE void block_candidates(const Block16 &blk, float invA, float invB, uin
     });
 }
 
+// IF4: the E2M1 candidate ("a") and the INT4 candidate ("b") of one block on their common scale,
+// with the sums of squared residuals in the scaled domain (quantize_block_if4_mse, for a tile).
+FOS_DEVICE void block_candidates_if4(const Block16 &blk, float inv, uint32_t &a0, uint32_t &a1, uint32_t &b0, uint32_t &b1,
+                                     float &SA, float &SB) {
+    a0 = a1 = b0 = b1 = 0;
+    static_for<0, 8>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const float x0 = scaled(u2f(blk.w[j] << 16), inv), x1 = scaled(u2f(blk.w[j] & 0xffff0000u), inv);
+        if (j < 4) a0 = pack_fp4<(j & 3)>(a0, x0, x1);
+        else a1 = pack_fp4<(j & 3)>(a1, x0, x1);
+        const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+        accumulate_scaled<FOS_RULE_MSE>(fa.x - x0, fa.y - x1, SA);
+        // INT4: rint(clamp(x * 7/6, -7, 7)); adding 1.5 * 2^23 rounds to nearest even and leaves the
+        // two's-complement integer in the low mantissa bits
+        const float t0 = __builtin_amdgcn_fmed3f(x0 * 1.16666666f, -7.0f, 7.0f) + 12582912.0f;
+        const float t1 = __builtin_amdgcn_fmed3f(x1 * 1.16666666f, -7.0f, 7.0f) + 12582912.0f;
+        const float q0 = t0 - 12582912.0f, q1 = t1 - 12582912.0f;
+        accumulate_scaled<FOS_RULE_MSE>(__builtin_fmaf(q0, 0.8571428571f, -x0), __builtin_fmaf(q1, 0.8571428571f, -x1), SB);
+        const uint32_t byte = (f2u(t0) & 0xfu) | ((f2u(t1) & 0xfu) << 4);
+        if (j < 4) b0 |= byte << (8 * (j & 3));
+        else b1 |= byte << (8 * (j & 3));
+    });
+}
+
 struct TilesPos {
     uint64_t x_base, codes_base, out_base;  // first input element / code byte / output element of the wavefront's share
     uint32_t x_bytes;    // extent of the input descriptor
@@ -102,7 +126,9 @@ FOS_DEVICE uint32_t quad_bytes(uint32_t l0, uint32_t l1, uint32_t l2, uint32_t l
     return __builtin_amdgcn_perm(p23, p01, 0x05040100u);
 }
 
-template <int RULE, bool FULL, bool PSEUDO>
+// IF4: the IF4 format with its MSE rule (both candidates on one scale; the chosen one is flagged in
+// bit 7 of the scale byte) instead of NVFP4.
+template <int RULE, bool FULL, bool PSEUDO, bool IF4 = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_tiles_kernel(
     const QuantParams p) {
     constexpr bool STATIC = RULE == FOS_RULE_STATIC_6;
@@ -275,7 +301,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         for (int off = 32; off >= 1; off >>= 1) bmax = fmaxf(bmax, __shfl_xor(bmax, off));
         uint32_t sX;
         float sfX, invX;
-        block_scale(k, bmax, !STATIC && cand_b, sX, sfX, invX);
+        block_scale(k, bmax, !STATIC && !IF4 && cand_b, sX, sfX, invX);
         bool pickB = false;
         if (!STATIC) {
             float chain = 0.0f;
@@ -283,7 +309,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             for (int m = 0; m < 8; ++m) {
                 const float xs = (sX != 0) ? x[m] * invX : 0.0f;
                 const float r = e2m1_round(fabsf(xs));
-                const float e = error_term<RULE>(div_errdiv(((xs < 0.0f ? -r : r) * sfX) * k.amax, k), x[m]);
+                float deq = div_errdiv(((xs < 0.0f ? -r : r) * sfX) * k.amax, k);
+                if (IF4) {
+                    // (select_intfloat, reference.py:328-425: the INT4 candidate on the same scale)
+                    const float qi = int4_round<false>(xs * 1.16666666f, 0.0f);
+                    const float deq_i = div_errdiv(((qi * sfX) * k.amax) * 0.8571428571f, k);
+                    deq = cand_b ? deq_i : deq;
+                }
+                const float e = error_term<RULE>(deq, x[m]);
                 chain = m == 0 ? e : (MAXRULE ? fmaxf(chain, e) : chain + e);
             }
             float tot_a, tot_b;
@@ -312,6 +345,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         const uint32_t src_lane = pickB ? 32 : 0;
         const uint32_t sP = __builtin_amdgcn_readlane(sX, src_lane);
         const float invP = u2f(__builtin_amdgcn_readlane(f2u(invX), src_lane));
+        const uint32_t s_out = IF4 && pickB ? sP + 128u : sP;  // what goes into the scale byte
         // codes: lane = (row, four columns)
         const uint32_t r = lane >> 2, cq = lane & 3;
         const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(rx, gbase + r * x_row + cq * 8u, 0, 0);
@@ -322,7 +356,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const uint32_t word = i < 2 ? w.x : w.y;
             const float xe = (i & 1) ? u2f(word & 0xffff0000u) : u2f(word << 16);
             const float xs = (sP != 0) ? xe * invP : 0.0f;
-            const uint32_t nib = e2m1_mag_code(e2m1_round(fabsf(xs))) | (xs < 0.0f ? 8u : 0u);
+            uint32_t nib = e2m1_mag_code(e2m1_round(fabsf(xs))) | (xs < 0.0f ? 8u : 0u);
+            if (IF4 && pickB) nib = (uint32_t)((int)int4_round<false>(xs * 1.16666666f, 0.0f)) & 0xfu;
             nibs |= nib << (4 * i);
             v[i] = e2m1_value(nib & 0xfu);
         }
@@ -350,9 +385,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         __builtin_amdgcn_raw_buffer_store_b16((uint16_t)nibs, rcodes, rstep * c_row + tl * 8u + cq * 2u, 0, 0);
         if (!tiled && cq == 0) {
             const BufferRsrc rsf = make_rsrc(reinterpret_cast<const void *>(uniform64((uint64_t)(p.sf + (int64_t)t.row0 * sf_cols))), 0xffffffffu);
-            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sP, rsf, rstep * (uint32_t)sf_cols + (uint32_t)cb_tile, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b8((uint8_t)s_out, rsf, rstep * (uint32_t)sf_cols + (uint32_t)cb_tile, 0, 0);
         }
-        return sP;
+        return s_out;
     };
 
     // one group: four blocks per lane in, codes (or dequantised values) out; returns the scale byte
@@ -378,7 +413,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
             const FastLutEntry A = lut[s6];
             FastLutEntry B = A;
-            if (ADAPTIVE) B = lut[s4];
+            if (ADAPTIVE && !IF4) B = lut[s4];
             // the hardware convert saturates at 6 where the reference's unclamped rounding gives 8:
             // that needs a sub-normal scale byte rounded down by more than 7/6; a zero scale byte
             // of a non-zero tile has no scaled domain
@@ -387,18 +422,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             float SA = 0.0f, SB = 0.0f;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
-                block_candidates<RULE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
+                if constexpr (IF4) block_candidates_if4(blk[s], A.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
+                else block_candidates<RULE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 load(nt, 32 * nq + 4 * s, blk[s]);
             }
             int cmp = -1;
             if (ADAPTIVE) {
                 SA = MAXRULE ? tile_max(SA) : tile_sum(SA);
                 SB = MAXRULE ? tile_max(SB) : tile_sum(SB);
-                cmp = shortcut_compare<RULE, true>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
+                // (IF4: one scale, so the two sums compare as they are)
+                if (IF4) cmp = shortcut_compare<FOS_RULE_MSE, true>(SA, 1.0f, SB, 1.0f);
+                else cmp = shortcut_compare<RULE, true>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
             }
             // an all-zero tile came out as zero codes under the zero scale byte
             need_slow = !(bmax == 0.0f || (fast_ok && cmp != 0));
-            if (ADAPTIVE && __builtin_amdgcn_ballot_w64(need_slow) != 0) {
+            if (ADAPTIVE && !IF4 && __builtin_amdgcn_ballot_w64(need_slow) != 0) {
                 // candidates that dequantise to the same values element by element tie: "6" wins
                 uint32_t viol = 1u;
                 if (fast_ok && e4m3_decode(s4) == 1.5f * e4m3_decode(s6)) {
@@ -413,7 +451,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 }
             }
             const bool pickB = ADAPTIVE && cmp > 0;
-            os = pickB ? s4 : s6;
+            os = IF4 ? (pickB ? s6 + 128u : s6) : (pickB ? s4 : s6);
             if (ADAPTIVE) {
 #pragma unroll
                 for (int s = 0; s < 4; ++s) {
@@ -496,6 +534,21 @@ void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s) {
         hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     else
         hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, false, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+}
+
+// IF4 with the MSE rule, round to nearest, 16x16 tiles, aligned input.
+void launch_quantize_if4_mse_tiles(QuantParams &p, hipStream_t s) {
+    p.tiles_x = (int)((p.cols_p + 511) / 512);
+    const int64_t n = (p.rows_p / 128) * p.tiles_x;
+    int64_t grid = 768;
+    if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
+    if (grid > n) grid = n;
+    p.tile_map = kMapSplitHalves;
+    if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
+    if (p.rows % 128 == 0 && p.cols % 512 == 0)
+        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<FOS_RULE_MSE, true, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<FOS_RULE_MSE, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
 template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, false>(QuantParams &, hipStream_t);
