@@ -181,6 +181,21 @@ def test_full_size_workloads_bit_exact(oracle, shape, kind, cfg):
             assert (t == t[:, :1]).all()
 
 
+@pytest.mark.parametrize("tile_map", range(1, 9))
+def test_tile_orders_give_the_same_bytes(monkeypatch, oracle, tile_map):
+    """FOS_QUANT_MAP only changes which workgroup quantizes which tile (row-major, one band per XCD,
+    column-major, the 16x16 kernel's column windows apart or side by side) and FOS_QUANT_GRID how many
+    workgroups share the tiles: the output does not depend on either, also for widths that leave an
+    incomplete run of windows and for ragged shapes."""
+    monkeypatch.setenv("FOS_QUANT_MAP", str(tile_map))
+    monkeypatch.setenv("FOS_QUANT_GRID", "24")
+    for shape in ((1024, 4096 + 1536), (384, 8192), (200, 1200)):
+        x = make_input("randn", shape, 17)
+        for cfg in (dict(scale_rule="mse"), dict(scale_rule="mse", block_scale_2d=True), dict(scale_rule="static_6", block_scale_2d=True),
+                    dict(dtype="if4", scale_rule="mse", block_scale_2d=True)):
+            assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), f"{shape} {cfg} map {tile_map}")
+
+
 @pytest.mark.parametrize("shape", [(100, 80), (16, 64), (1, 16), (130, 8), (257, 1000), (128, 72)])
 def test_ragged_shapes_are_zero_padded(oracle, shape):
     x = make_input("randn", shape, 3)
