@@ -324,11 +324,14 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     hipStream_t s = (hipStream_t)stream;
     uint32_t *partials = (uint32_t *)workspace;
     // (fp16 / fp32 inputs take the element-wise kernel: treat them as unaligned throughout)
-    const bool aligned = x_type == FOS_T_BF16 && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0);
+    // The streaming kernels address a 128-row tile with 32-bit byte offsets: a row pitch of 2^23
+    // elements or more (16 MiB rows) takes the element-wise kernel like an unaligned input.
+    constexpr int64_t kMaxPitch = int64_t{1} << 23;
+    const bool aligned = x_type == FOS_T_BF16 && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0) && ld < kMaxPitch;
     if (pseudo_out) {
         // only the NVFP4 round-to-nearest kernels have the fused epilogue
         if (dtype != FOS_DTYPE_NVFP4 || round_style != FOS_ROUND_NEAREST || !aligned) return FOS_E_UNSUPPORTED;
-        if (ldo < cols) return FOS_E_BAD_SHAPE;
+        if (ldo < cols || ldo >= kMaxPitch) return FOS_E_BAD_SHAPE;
         if (((uintptr_t)pseudo_out & 15) || (ldo % 8 != 0)) return FOS_E_BAD_ALIGNMENT;
     }
 

@@ -136,6 +136,7 @@ def pseudo_quantize_is_fused(x: torch.Tensor, dtype: int, round_style: int) -> b
         and x.stride(-1) == 1
         and x.shape[1] % 16 == 0
         and x.stride(0) % 8 == 0
+        and x.stride(0) < (1 << 23)  # (the streaming kernels' 32-bit tile offsets)
         and x.data_ptr() % 16 == 0
     )
 
