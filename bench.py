@@ -312,15 +312,15 @@ def main() -> int:
                                  amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")), K)
     q_achieved = algo_bytes / (quant_ms * 1e-3) / 1e9
     roofline = {
-        "kernel": "fos::quantize_nvfp4_rows_kernel<3, true, false, false> (pass 2: scale, 4/6 select, pack)",
+        "kernel": "fos::quantize_nvfp4_rows_kernel<3, true, false, false, false> (pass 2: scale, 4/6 select, pack)",
         "bound": "hbm",
         "achieved": round(q_achieved, 1),
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(q_achieved / HBM_PEAK_GBS, 4),
         # HBM bytes per launch of this kernel at 8192 x 8192, measured once with rocprofv3
-        # (FETCH_SIZE 65874.9 KiB x 2.00 calibration + WRITE_SIZE 41810.4 KiB x 1.00): no re-reads
-        "traffic": 177.7e6 if (rows, cols) == (8192, 8192) else None,
+        # (FETCH_SIZE 65870.9 KiB x 2.00 calibration + WRITE_SIZE 36864.0 KiB x 1.00): no re-reads
+        "traffic": 172.7e6 if (rows, cols) == (8192, 8192) else None,
         "kernel_ms": round(quant_ms, 5),
         "amax_pass_ms": round(amax_ms, 5),
         "amax_pass_GBs": round(elems * 2 / (amax_ms * 1e-3) / 1e9, 1),

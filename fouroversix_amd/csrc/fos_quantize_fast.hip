@@ -144,8 +144,8 @@ struct RowsTile {
 template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false>
 // (the stochastic instantiations hold two sets of scaled values and the Philox state: with 128
 // registers they spilled -- 30 MB of scratch traffic per launch at 8192 x 8192 -- and the launch
-// grid of three workgroups per compute unit leaves 168)
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3 : 4))) void quantize_nvfp4_rows_kernel(
+// grid of three workgroups per compute unit leaves 168; the IF4 instantiation spilled as well)
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR || IF4) ? 3 : 4))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
     __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][128];  // per wavefront: 4 scale tiles x 128 bytes
