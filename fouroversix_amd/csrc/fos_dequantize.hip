@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fos_buffer.h"
 #include "fos_quantize_fast.h"
 #include "fouroversix_hip.h"
 
@@ -101,7 +102,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
     }
     uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
     if (whole) {
-        *reinterpret_cast<uint4 *>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        stream_store(reinterpret_cast<uint4 *>(o), make_uint4(w[0], w[1], w[2], w[3]));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i)

@@ -503,7 +503,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1
             a_stage[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(a_row0 + a_off + i * 8 * kbytes), kq, 0));
     };
     // 128 codes of each B row; two register sets (loaded two steps ahead), one with two tiles
-    constexpr int kBSets = (WN == 2 || MT == 2 || MT == 4) ? 1 : 2;
+    constexpr int kBSets = (WN == 2 || MT == 2) ? 1 : 2;  // (the 4 x 1 form multiplies straight from these registers: two sets)
     typedef uint4 BCodes[WN][4];
     BCodes bst[kBSets];
     auto fetch_b_codes = [&](int64_t j, BCodes &b) {

@@ -19,6 +19,7 @@
 
 #include <cstdlib>
 
+#include "fos_buffer.h"
 #include "fos_quantize_fast.h"
 #include "fos_tuning.h"
 #include "fouroversix_hip.h"
@@ -137,7 +138,7 @@ __global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const M
             if (!col_ok) continue;
             const int rr = g * 32 + wave * 4 + j;
             const int64_t r = tile_y * 128 + rr;
-            *reinterpret_cast<uint32_t *>(p.codes + r * (p.cols_p >> 1) + (c0 >> 1)) = codes;
+            stream_store(reinterpret_cast<uint32_t *>(p.codes + r * (p.cols_p >> 1) + (c0 >> 1)), codes);
             if ((lane & 3) == 0) {
                 if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
                 else p.sf[r * sf_cols + cb] = (uint8_t)e;
@@ -251,7 +252,7 @@ __global__ __launch_bounds__(256) void dequantize_mxfp4_kernel(const MxDequantPa
     }
     uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
     if (whole) {
-        *reinterpret_cast<uint4 *>(o) = make_uint4(w[0], w[1], w[2], w[3]);
+        stream_store(reinterpret_cast<uint4 *>(o), make_uint4(w[0], w[1], w[2], w[3]));
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i)

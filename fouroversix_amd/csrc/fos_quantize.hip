@@ -10,6 +10,7 @@
 // the operation-by-operation form (IF4, stochastic rounding); NVFP4 round-to-nearest is
 // instantiated in fos_quantize_fast.hip.
 #include <atomic>
+#include <type_traits>
 #include <cstdlib>
 
 #include "fos_quantize_kernel.h"
@@ -41,32 +42,77 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
                                                              uint32_t *__restrict__ partials) {
     __shared__ uint32_t smem[4];
     const int64_t stride = (int64_t)gridDim.x * kThreads;
-    int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t first = (int64_t)blockIdx.x * kThreads + threadIdx.x;
     uint32_t m = 0;
     constexpr int U = 8;
-    for (; i + (U - 1) * stride < n_vec; i += U * stride) {
-        uint4 v[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) v[u] = x[i + u * stride];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            m = pk_max_u16(m, v[u].x & 0x7fff7fffu);
-            m = pk_max_u16(m, v[u].y & 0x7fff7fffu);
-            m = pk_max_u16(m, v[u].z & 0x7fff7fffu);
-            m = pk_max_u16(m, v[u].w & 0x7fff7fffu);
-        }
-    }
-    for (; i < n_vec; i += stride) {
-        uint4 v = x[i];
+    auto fold = [&](const uint4 &v) {
         m = pk_max_u16(m, v.x & 0x7fff7fffu);
         m = pk_max_u16(m, v.y & 0x7fff7fffu);
         m = pk_max_u16(m, v.z & 0x7fff7fffu);
         m = pk_max_u16(m, v.w & 0x7fff7fffu);
+    };
+    const int64_t n_full = n_vec / (U * stride);  // trips in which every thread has its U vectors
+    // the ragged end of the tensor ...
+    for (int64_t i = n_full * U * stride + first; i < n_vec; i += stride) fold(x[i]);
+    // ... and the full trips
+    for (int64_t k = 0; k < n_full; ++k) {
+        const int64_t i = k * U * stride + first;
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = x[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < U; ++u) fold(v[u]);
     }
     uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
     mm = block_max_u32(mm, smem);
     if (threadIdx.x == 0) {
         partials[2 * blockIdx.x] = mag16_to_f32_bits<IS_BF16>(mm);
+        partials[2 * blockIdx.x + 1] = 0u;
+    }
+}
+
+// bf16 input with cols % 2048 == 0, read so that pass 2 finds in L2 what this pass read last (clean lines
+// survive the kernel boundary).  The streaming pass-2 kernels give workgroup b the 128 x 256 units b,
+// b + grid, ... in row-major order, and the compute die (XCD) that takes workgroup b of a launch is b % 8:
+// with a multiple of 8 units to a row, die j quantizes the 512-byte windows j, j + 8, ... of every row,
+// starting with the top rows.  Here die j reads exactly those windows, bottom rows first, so the top rows are
+// what its L2 holds when pass 2 starts.  At any time the grid reads one contiguous range of whole rows (16
+// rows per workgroup and step at 8192 columns, 512 rows in all).  At 8192 x 8192 the scan itself takes
+// 0.3 us longer than the flat one and the pass 2 behind it 1-2.5 us less.
+__global__ __launch_bounds__(kThreads) void amax_units_kernel(const uint16_t *__restrict__ x, int64_t ld, uint32_t win_per_die,
+                                                              uint32_t n_winrows, uint32_t n_steps,
+                                                              uint32_t *__restrict__ partials) {
+    __shared__ uint32_t smem[4];
+    const uint32_t t = threadIdx.x;
+    const uint32_t die = blockIdx.x & 7u, slot = blockIdx.x >> 3;  // 32 workgroups to a die
+    uint32_t m = 0;
+    // a step of a workgroup = 64 window-rows (512 bytes each) = 8 loads of 16 bytes per thread; window-row q
+    // of a die is window q % win_per_die of row q / win_per_die.  Only the step at the bottom of the tensor
+    // can run past the end: it repeats the final window-row there.
+    auto scan = [&](uint32_t step, auto ragged) {
+        const uint32_t q0 = ((n_steps - 1 - step) * 32 + slot) * 64 + (t >> 5);
+        uint4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            uint32_t q = q0 + j * 8;
+            if (ragged) q = q < n_winrows ? q : n_winrows - 1;
+            const uint32_t row = q / win_per_die, win = q - row * win_per_die;
+            v[j] = *reinterpret_cast<const uint4 *>(x + (int64_t)row * ld + (die + 8 * win) * 256 + (t & 31) * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            m = pk_max_u16(m, v[j].x & 0x7fff7fffu);
+            m = pk_max_u16(m, v[j].y & 0x7fff7fffu);
+            m = pk_max_u16(m, v[j].z & 0x7fff7fffu);
+            m = pk_max_u16(m, v[j].w & 0x7fff7fffu);
+        }
+    };
+    scan(0, std::true_type{});
+    for (uint32_t step = 1; step < n_steps; ++step) scan(step, std::false_type{});
+    uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+    mm = block_max_u32(mm, smem);
+    if (threadIdx.x == 0) {
+        partials[2 * blockIdx.x] = mag16_to_f32_bits<true>(mm);
         partials[2 * blockIdx.x + 1] = 0u;
     }
 }
@@ -197,7 +243,13 @@ int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t l
                                cols, ld, partials);
         return n_partials;
     }
-    if (ld == cols && aligned) {
+    // the scan that leaves the first units of a streaming pass 2 in L2 (tensors of 16 MiB and more; window-rows per die = rows * cols / 2048, a step of the grid takes 32 * 64 of them)
+    const int64_t n_winrows = cols % 2048 == 0 ? rows * (cols / 2048) : 0;
+    if (aligned && n_winrows >= 4096 && n_winrows < (int64_t{1} << 31) && tuning().amax_units >= 0) {
+        n_partials = 256;
+        hipLaunchKernelGGL(amax_units_kernel, dim3(n_partials), dim3(kThreads), 0, s, (const uint16_t *)x, ld,
+                           (uint32_t)(cols / 2048), (uint32_t)n_winrows, (uint32_t)((n_winrows + 2047) / 2048), partials);
+    } else if (ld == cols && aligned) {
         const int64_t n_vec = rows * cols / 8;
         // each thread keeps 8 independent 128-bit loads in flight
         int64_t want = (n_vec + kThreads * 8 - 1) / (kThreads * 8);

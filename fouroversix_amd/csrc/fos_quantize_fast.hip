@@ -267,6 +267,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
                 // into the per-lane offset)
                 const uint32_t o_off = o_lane + step_row(g) * o_row;
                 const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
+                // (plain stores: the two halves of a line come from two instructions and meet in L2)
                 __builtin_amdgcn_raw_buffer_store_b128(d0, rout, o_off, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b128(d1, rout, o_off + 16u, 0, 0);
             }
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         }
         const u32x2 c01 = {o.c0, o.c1};
         const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
-        __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, step_row(g) * c_row, 0);
+        __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, step_row(g) * c_row, kStreamStore);
         if (tiled) stage[(g & 1) * 64 + (g >> 1) * 4] = (uint8_t)o.s;
         else p.sf[row * sf_cols + t.cb] = (uint8_t)o.s;
     };

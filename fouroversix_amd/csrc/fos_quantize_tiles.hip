@@ -258,6 +258,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 // goes into the per-lane offset)
                 const uint32_t o_off = o_lane + rstep * o_row;
                 const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
+                // (plain stores: the two halves of a line come from two instructions and meet in L2)
                 __builtin_amdgcn_raw_buffer_store_b128(d0, rout, o_off, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b128(d1, rout, o_off + 16u, 0, 0);
             }
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         if (pred && (FULL || t.cb < (int32_t)sf_cols)) {  // inside the padded width
             const u32x2 c01 = {c0, c1};
             const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
-            __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, __builtin_amdgcn_readfirstlane(rstep * c_row), 0);
+            __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, __builtin_amdgcn_readfirstlane(rstep * c_row), kStreamStore);
             if (!tiled) {
                 const BufferRsrc rsf = make_rsrc(reinterpret_cast<const void *>(uniform64((uint64_t)(p.sf + (int64_t)t.row0 * sf_cols))), 0xffffffffu);
                 __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sbyte, rsf, (uint32_t)((rstep + li) * (uint32_t)sf_cols + (uint32_t)t.cb), 0, 0);

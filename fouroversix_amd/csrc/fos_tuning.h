@@ -13,6 +13,7 @@ struct Tuning {
     std::atomic<int> mx_tile{0};      // FOS_MX_TILE
     std::atomic<int> quant_grid{0};   // FOS_QUANT_GRID
     std::atomic<int> amax_grid{0};    // FOS_AMAX_GRID
+    std::atomic<int> amax_units{0};   // FOS_AMAX_UNITS: -1 = flat pass 1 also ahead of a streaming pass 2
     std::atomic<int> quant_map{0};    // FOS_QUANT_MAP: tile order of the streaming quantize kernels (1 + TileMap)
 };
 

@@ -301,6 +301,45 @@ def test_caller_supplied_amax(oracle):
             assert_same_quantization(q, ref, f"{kind} {cfg}")
 
 
+@pytest.mark.parametrize(("rows", "cols", "ld"), [
+    (2051, 4096, 4096),     # window order (cols % 2048 == 0, >= 16 MiB), rows not a multiple of anything
+    (4096, 2048, 2048 + 64),  # the same scan over a strided view
+    (1024, 8192, 8192),     # exactly one step of the window-order scan
+    (1023, 8192, 8192),     # just below it: the flat scan
+    (3000, 6144, 6144),
+    (777, 14336, 14336),
+])
+def test_tensor_maximum_scan_covers_every_element(rows, cols, ld):
+    """pass 1 reads every element exactly where the tensor says it is: a single non-zero element, moved
+    through corners, row ends and random places, is the maximum each time (and a larger value in the
+    gap of a strided view is not)."""
+    from fouroversix_amd import _native as nat
+
+    L = nat.lib()
+    dev = torch.device("cuda", 0)
+    base = torch.zeros(rows, ld, dtype=torch.bfloat16, device=dev)
+    if ld > cols:
+        base[:, cols:] = 1000.0
+    amax = torch.zeros(1, dtype=torch.float32, device=dev)
+    ws_bytes = L.fos_quantize_workspace_bytes(rows, cols)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    stream = nat.current_stream(dev)
+    rng = np.random.default_rng(rows * 31 + cols)
+    spots = [(0, 0), (0, cols - 1), (rows - 1, 0), (rows - 1, cols - 1), (rows - 1, cols - 257), (rows // 2, 255), (rows // 2, 256),
+             (1, 2047), (rows - 2, 2048 % cols)]
+    spots += [(int(rng.integers(rows)), int(rng.integers(cols))) for _ in range(40)]
+    for k, (r, c) in enumerate(spots):
+        value = -(2.0 + k) if k % 2 else 2.0 + k
+        base[r, c] = value
+        nat.check(L.fos_amax(base.data_ptr(), nat.T_BF16, rows, cols, ld, amax.data_ptr(), ws.data_ptr(), ws_bytes, stream), "amax")
+        assert float(amax.item()) == abs(value), (rows, cols, ld, r, c)
+        base[r, c] = 0.0
+    # and the quantizer behind it sees the same maximum
+    base[rows - 1, cols - 1] = 3.0
+    q = fos.quantize(base[:, :cols], fos.QuantizationConfig(scale_rule="static_6"))
+    assert float(q.amax) == 3.0
+
+
 def test_concurrent_streams_do_not_share_the_workspace(oracle):
     """Two streams quantize different tensors at the same time (the two-launch path, which
     hands partial maxima from pass 1 to pass 2 through a per-stream workspace)."""
