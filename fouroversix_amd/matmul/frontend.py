@@ -68,6 +68,48 @@ def _members_fit(q: QuantizedTensor, values: torch.Tensor) -> bool:
     )
 
 
+# What the NVFP4 GEMM needs to know about an operand, looked up once per QuantizedTensor and kept on it
+# while its three tensors are the same objects (a layer's weights are the same object in every call):
+# (values, scale_factors, amax, usable, kernel_values, divisor, device, inner).  `usable`: NVFP4 in the
+# tiled scale layout whose members pass the op's checks, with an f32 maximum on the same GPU;
+# `kernel_values`: the codes the kernel reads (the real rows only for a small batch).
+_GEMM_RECORD = "_fos_gemm_record"
+
+
+def _gemm_record(q: QuantizedTensor) -> tuple:
+    values, sf, amax = q.values, q.scale_factors, q.amax
+    rec = q.__dict__.get(_GEMM_RECORD)
+    if (
+        rec is not None
+        and rec[0] is values
+        and rec[1] is sf
+        and rec[2] is amax
+        and rec[8] is q.scale_rule
+        and rec[9] is q.round_style
+        and rec[10] == q.original_shape
+        and rec[11] == q.padded_shape
+    ):
+        return rec
+    kernel_values = values
+    m_orig = q.original_shape[0]
+    if m_orig < 128 and values.dim() == 2 and values.shape[0] == 128 and values.shape[1] % 128 == 0:
+        kernel_values = values[:m_orig]  # small batch: only the real rows, so the kernel skips the padding
+    usable = (
+        q.dtype == DataType.nvfp4
+        and q.scale_factors_are_in_blackwell_layout
+        and type(values) is torch.Tensor
+        and values.is_cuda
+        and amax is not None
+        and amax.dtype == torch.float32
+        and amax.device == values.device
+        and _members_fit(q, kernel_values)
+    )
+    rec = (values, sf, amax, usable, kernel_values, dequantize_divisor(q) if usable else 0.0, values.device,
+           q.original_shape[1], q.scale_rule, q.round_style, q.original_shape, q.padded_shape)
+    q.__dict__[_GEMM_RECORD] = rec
+    return rec
+
+
 _UNIT_ALPHA: dict = {}
 
 
@@ -117,6 +159,29 @@ def quantized_matmul(
     if isinstance(out_dtype, str):
         out_dtype = DataType(out_dtype)
 
+    # two NVFP4 operands on one GPU: straight to the kernel, which forms alpha from the two maxima itself
+    # (same arithmetic as gemm_alpha, one launch less)
+    ra, rb = _gemm_record(input), _gemm_record(other)
+    if (
+        ra[3]
+        and rb[3]
+        and ra[6] == rb[6]
+        and ra[7] == rb[7]
+        and (out_dtype is DataType.bfloat16 or out_dtype is DataType.float16)
+        and not torch.compiler.is_compiling()
+    ):
+        d_amax = torch.zeros(1, dtype=torch.float32, device=ra[6]) if emit_amax else None
+        out = ops.gemm_nvfp4_from_amax(
+            ra[4], rb[0], ra[1], rb[1], ra[2], rb[2], ra[5] * rb[5],
+            torch.bfloat16 if out_dtype is DataType.bfloat16 else torch.float16, d_amax, checked=True,
+        )
+        m, n = input.original_shape[0], other.original_shape[0]
+        if out.shape[0] != m or out.shape[1] != n:
+            out = out[:m, :n]  # (the padding is zeros: same maximum)
+        if d_amax is not None:
+            attach_known_amax(out, d_amax)
+        return out
+
     if not is_supported(input, other, out_dtype=out_dtype):
         if _dequantize_form_applies(input, other, out_dtype):
             # formats without a native GEMM (IF4; mixed formats): the reference's PyTorch backend,
@@ -148,37 +213,15 @@ def quantized_matmul(
     if m_orig < 128 and a_values.shape[0] == 128 and a_values.shape[1] % 128 == 0:
         # small batch: hand over only the real rows, so the kernel skips the padding
         a_values = a_values[:m_orig]
-    a_amax, b_amax = input.amax, other.amax
-    if (
-        type(a_values) is torch.Tensor
-        and not torch.compiler.is_compiling()
-        and a_amax.dtype == torch.float32
-        and b_amax.dtype == torch.float32
-        and a_amax.is_cuda
-        and b_amax.device == a_amax.device == a_values.device
-    ):
-        # the kernel forms alpha from the two maxima itself (same arithmetic, one launch less)
-        den = dequantize_divisor(input) * dequantize_divisor(other)
-        d_amax = torch.zeros(1, dtype=torch.float32, device=a_values.device) if emit_amax else None
-        out = ops.gemm_nvfp4_from_amax(
-            a_values, other.values, input.scale_factors, other.scale_factors, a_amax, b_amax, den,
-            torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16, d_amax,
-            checked=_members_fit(input, a_values) and _members_fit(other, other.values),
-        )
-        out_shape = (input.original_shape[0], other.original_shape[0])
-        if tuple(out.shape) != out_shape:
-            out = out[: out_shape[0], : out_shape[1]]  # (the padding is zeros: same maximum)
-        if d_amax is not None:
-            attach_known_amax(out, d_amax)
-        return out
-    else:
-        alpha = gemm_alpha(input, other)
-        gemm = (
-            ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
-            if out_dtype == DataType.bfloat16
-            else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
-        )
-        out = gemm(a_values, other.values, input.scale_factors, other.scale_factors, alpha)
+    # (torch.compile, or maxima that are not f32 tensors on the GPU: alpha from its own small kernel or from
+    # torch arithmetic; emit_amax has no effect here and the next quantize finds the maximum itself)
+    alpha = gemm_alpha(input, other)
+    gemm = (
+        ops.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
+        if out_dtype == DataType.bfloat16
+        else ops.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt
+    )
+    out = gemm(a_values, other.values, input.scale_factors, other.scale_factors, alpha)
     out_shape = (input.original_shape[0], other.original_shape[0])
     if tuple(out.shape) != out_shape:
         out = out[: out_shape[0], : out_shape[1]]

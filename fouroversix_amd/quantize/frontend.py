@@ -183,16 +183,16 @@ def quantize(
         nat.SF_LINEAR if linear else nat.SF_TILED,
         None if config.dtype == DataType.mxfp4 else config.kwargs.get("amax", known_amax(x)),  # mxfp4 has no tensor scale
     )
-    return QuantizedTensor(
+    return QuantizedTensor.from_kernel(
         values,
         scale_factors,
         amax.reshape(()),
         config.dtype,
-        tuple(x.shape),
+        (x.shape[0], x.shape[1]),
         config.scale_rule,
         config.round_style,
         (values.shape[0], values.shape[1] * config.dtype.quantized_value_type.packing_factor),  # as the kernel padded it
-        scale_factors_are_in_blackwell_layout=not linear,
+        not linear,
     )
 
 

@@ -94,6 +94,23 @@ class QuantizedTensor:
         self.scale_factors = scale_factors
         self.amax = amax
 
+    @classmethod
+    def from_kernel(cls, values, scale_factors, amax, dtype, original_shape, scale_rule, round_style, padded_shape,
+                    tiled: bool) -> "QuantizedTensor":
+        """What ``quantize`` builds from the kernel's outputs: members of the final sizes and enum-typed
+        attributes, stored as they are (the constructor's conversions and padding have nothing to do)."""
+        q = object.__new__(cls)
+        q.dtype = dtype
+        q.original_shape = original_shape
+        q.scale_rule = scale_rule
+        q.round_style = round_style
+        q.scale_factors_are_in_blackwell_layout = tiled
+        q.padded_shape = padded_shape
+        q.values = values
+        q.scale_factors = scale_factors
+        q.amax = amax
+        return q
+
     @property
     def device(self) -> torch.device:
         return self.values.device
