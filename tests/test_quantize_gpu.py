@@ -340,6 +340,33 @@ def test_tensor_maximum_scan_covers_every_element(rows, cols, ld):
     assert float(q.amax) == 3.0
 
 
+def test_two_pass_quantize_replays_in_a_hip_graph():
+    """A 32 MiB input (tensor-maximum scan in window order + streaming pass 2, non-temporal code stores)
+    captured in a HIP graph: every replay, with eager work and synchronisations in between, equals the
+    eager result on the input's new contents."""
+    cfg = fos.QuantizationConfig(scale_rule="mse")
+    static_x = make_input("randn", (4096, 4096), 90).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fos.quantize(static_x, cfg)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_q = fos.quantize(static_x, cfg)
+    for i in range(4):
+        xi = make_input("randn", (4096, 4096), 91 + i).cuda() * float(i + 1)
+        static_x.copy_(xi)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = fos.quantize(xi, cfg)
+        torch.cuda.synchronize()
+        assert torch.equal(static_q.values, eager.values), f"replay {i}"
+        assert torch.equal(static_q.scale_factors.view(torch.uint8), eager.scale_factors.view(torch.uint8)), f"replay {i}"
+        assert float(static_q.amax) == float(eager.amax), f"replay {i}"
+
+
 def test_concurrent_streams_do_not_share_the_workspace(oracle):
     """Two streams quantize different tensors at the same time (the two-launch path, which
     hands partial maxima from pass 1 to pass 2 through a per-stream workspace)."""
