@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
     }
 }
 
-// bf16 input with cols % 2048 == 0, read so that pass 2 finds in L2 what this pass read last (clean lines
+// bf16 / fp16 input with cols % 2048 == 0, read so that pass 2 finds in L2 what this pass read last (clean lines
 // survive the kernel boundary).  The streaming pass-2 kernels give workgroup b the 128 x 256 units b,
 // b + grid, ... in row-major order, and the compute die (XCD) that takes workgroup b of a launch is b % 8:
 // with a multiple of 8 units to a row, die j quantizes the 512-byte windows j, j + 8, ... of every row,
@@ -79,6 +79,7 @@ __global__ __launch_bounds__(kThreads) void amax_flat_kernel(const uint4 *__rest
 // what its L2 holds when pass 2 starts.  At any time the grid reads one contiguous range of whole rows (16
 // rows per workgroup and step at 8192 columns, 512 rows in all).  At 8192 x 8192 the scan itself takes
 // 0.3 us longer than the flat one and the pass 2 behind it 1-2.5 us less.
+template <bool IS_BF16>
 __global__ __launch_bounds__(kThreads) void amax_units_kernel(const uint16_t *__restrict__ x, int64_t ld, uint32_t win_per_die,
                                                               uint32_t n_winrows, uint32_t n_steps,
                                                               uint32_t *__restrict__ partials) {
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(kThreads) void amax_units_kernel(const uint16_t *__
     uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
     mm = block_max_u32(mm, smem);
     if (threadIdx.x == 0) {
-        partials[2 * blockIdx.x] = mag16_to_f32_bits<true>(mm);
+        partials[2 * blockIdx.x] = mag16_to_f32_bits<IS_BF16>(mm);
         partials[2 * blockIdx.x + 1] = 0u;
     }
 }
@@ -221,6 +222,20 @@ namespace {
 int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, bool aligned, uint32_t *partials,
                 hipStream_t s) {
     int n_partials;
+    // bf16 / fp16: the scan that leaves the first units of a streaming pass 2 in L2 (tensors of 16 MiB and
+    // more; window-rows per die = rows * cols / 2048, a step of the grid takes 32 * 64 of them)
+    const int64_t n_winrows = cols % 2048 == 0 ? rows * (cols / 2048) : 0;
+    if (x_type != FOS_T_F32 && ((uintptr_t)x & 15) == 0 && ld % 8 == 0 && n_winrows >= 4096 && n_winrows < (int64_t{1} << 31) &&
+        tuning().amax_units >= 0) {
+        const uint32_t win = (uint32_t)(cols / 2048), steps = (uint32_t)((n_winrows + 2047) / 2048);
+        if (x_type == FOS_T_BF16)
+            hipLaunchKernelGGL((amax_units_kernel<true>), dim3(256), dim3(kThreads), 0, s, (const uint16_t *)x, ld, win,
+                               (uint32_t)n_winrows, steps, partials);
+        else
+            hipLaunchKernelGGL((amax_units_kernel<false>), dim3(256), dim3(kThreads), 0, s, (const uint16_t *)x, ld, win,
+                               (uint32_t)n_winrows, steps, partials);
+        return 256;
+    }
     if (x_type != FOS_T_BF16 && ld == cols && ((uintptr_t)x & 15) == 0 && (rows * cols) % 8 == 0) {
         // contiguous: the flat scans (fp16 shares the bf16 one, magnitudes order like bit patterns)
         const int64_t n_vec = rows * cols / (x_type == FOS_T_F32 ? 4 : 8);
@@ -243,13 +258,7 @@ int launch_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t l
                                cols, ld, partials);
         return n_partials;
     }
-    // the scan that leaves the first units of a streaming pass 2 in L2 (tensors of 16 MiB and more; window-rows per die = rows * cols / 2048, a step of the grid takes 32 * 64 of them)
-    const int64_t n_winrows = cols % 2048 == 0 ? rows * (cols / 2048) : 0;
-    if (aligned && n_winrows >= 4096 && n_winrows < (int64_t{1} << 31) && tuning().amax_units >= 0) {
-        n_partials = 256;
-        hipLaunchKernelGGL(amax_units_kernel, dim3(n_partials), dim3(kThreads), 0, s, (const uint16_t *)x, ld,
-                           (uint32_t)(cols / 2048), (uint32_t)n_winrows, (uint32_t)((n_winrows + 2047) / 2048), partials);
-    } else if (ld == cols && aligned) {
+    if (ld == cols && aligned) {
         const int64_t n_vec = rows * cols / 8;
         // each thread keeps 8 independent 128-bit loads in flight
         int64_t want = (n_vec + kThreads * 8 - 1) / (kThreads * 8);
@@ -285,7 +294,7 @@ void launch_typed(QuantParams &p, bool two_d, hipStream_t s) {
 
 template <int DT, int RULE>
 void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, hipStream_t s) {
-    if (p.x_type != FOS_T_BF16) {
+    if (p.x_type != FOS_T_BF16 && !(aligned && p.x_type == FOS_T_F16)) {
         if (round_style == FOS_ROUND_NEAREST) launch_typed<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, s);
         else launch_typed<DT, RULE, FOS_ROUND_STOCHASTIC>(p, two_d, s);
         return;
@@ -375,11 +384,14 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
 
     hipStream_t s = (hipStream_t)stream;
     uint32_t *partials = (uint32_t *)workspace;
-    // (fp16 / fp32 inputs take the element-wise kernel: treat them as unaligned throughout)
+    // (fp32 inputs, and fp16 ones outside the case below, take the element-wise kernel: they are treated as
+    // unaligned throughout)
     // The streaming kernels address a 128-row tile with 32-bit byte offsets: a row pitch of 2^23
     // elements or more (16 MiB rows) takes the element-wise kernel like an unaligned input.
     constexpr int64_t kMaxPitch = int64_t{1} << 23;
-    const bool aligned = x_type == FOS_T_BF16 && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0) && ld < kMaxPitch;
+    // fp16 input has a streaming form for NVFP4 codes with 1x16 blocks and round to nearest
+    const bool f16_streams = x_type == FOS_T_F16 && dtype == FOS_DTYPE_NVFP4 && round_style == FOS_ROUND_NEAREST && !block2d && !pseudo_out;
+    const bool aligned = (x_type == FOS_T_BF16 || f16_streams) && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0) && ld < kMaxPitch;
     if (pseudo_out) {
         // only the NVFP4 round-to-nearest kernels have the fused epilogue
         if (dtype != FOS_DTYPE_NVFP4 || round_style != FOS_ROUND_NEAREST || !aligned) return FOS_E_UNSUPPORTED;
@@ -406,7 +418,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         p.partials = (const uint32_t *)amax;
         p.n_partials = 0;
         p.amax_out = nullptr;
-    } else if (aligned && ld == cols && rows * cols <= kFusedAmaxElements) {
+    } else if (aligned && x_type == FOS_T_BF16 && ld == cols && rows * cols <= kFusedAmaxElements) {
         // decode-sized input: one launch, every workgroup of pass 2 finds the maximum itself
         p.partials = partials;
         p.n_partials = -1;

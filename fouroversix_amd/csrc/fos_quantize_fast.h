@@ -155,8 +155,11 @@ struct BlockOut {
     uint32_t c0, c1, s;
 };
 
+// F16: the block holds fp16 pairs instead of bf16 pairs (both convert to f32 exactly).
+template <bool F16 = false>
 FOS_DEVICE float block_element(const uint32_t *w, int idx) {
     const uint32_t word = w[idx >> 1];
+    if (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)((idx & 1) ? word >> 16 : word));
     return (idx & 1) ? u2f(word & 0xffff0000u) : u2f(word << 16);
 }
 
@@ -270,7 +273,7 @@ FOS_DEVICE bool exact_pick_b_1d(const float *x, uint32_t a0, uint32_t a1, uint32
 
 // Operation-by-operation form (sub-normal block scales, out-of-range tensors): the
 // arithmetic of quantize_block in fos_quantize_common.h, rolled.
-template <int RULE, bool TWO_D>
+template <int RULE, bool TWO_D, bool F16 = false>
 __device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantConsts k) {
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
     uint32_t w[8];
@@ -278,7 +281,7 @@ __device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantCo
     for (int i = 0; i < 8; ++i) w[i] = blk.w[i];
     float bmax = 0.0f;
 #pragma nounroll
-    for (int i = 0; i < 16; ++i) bmax = fmaxf(bmax, fabsf(block_element(w, i)));
+    for (int i = 0; i < 16; ++i) bmax = fmaxf(bmax, fabsf(block_element<F16>(w, i)));
     if (TWO_D) bmax = row16_max(bmax);
     uint32_t sA, sB = 0;
     float sfA, invA, sfB = 0.0f, invB = 0.0f;
@@ -292,7 +295,7 @@ __device__ __attribute__((noinline)) BlockOut generic_block(Block16 blk, QuantCo
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int idx = l + 8 * h;
-            const float x = block_element(w, idx);
+            const float x = block_element<F16>(w, idx);
             const float xsA = (sA != 0) ? x * invA : 0.0f;
             const float rA = e2m1_round(fabsf(xsA));
             const bool negA = xsA < 0.0f;
@@ -330,10 +333,15 @@ __device__ __attribute__((noinline)) BlockOut generic_block_sr(Block16 blk, Quan
 
 // One 1x16 block, NVFP4, any rule, round to nearest or (SR) a stochastic style; falls
 // back by itself.  `blkid` = row * (cols_p / 16) + block column keys the dither.
-template <int RULE, bool TWO_D, bool SR>
+// F16: fp16 elements (1x16 blocks, round to nearest).  Nothing in the formulation depends on the element
+// type beyond the conversion to f32: the scaled value is the reference's own x * inv, the division of
+// the block maximum by 6 or 4 is correctly rounded for every fp16 numerator too (checked exhaustively),
+// and fq * s * amax stays exact with the 11 significant bits of an fp16 maximum (2 + 4 + 11 <= 24).
+template <int RULE, bool TWO_D, bool SR, bool F16 = false>
 FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq,
                                               bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
                                               uint64_t blkid) {
+    static_assert(!F16 || (!TWO_D && !SR), "fp16 elements: 1x16 blocks, round to nearest");
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
     // the certified shortcut: MSE, and MAE for 1x16 blocks.  (Abs-max has one too, but 3 % of the
     // blocks of N(0,1) data tie exactly under that rule -- the largest residual belongs to an
@@ -344,8 +352,13 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
         float x[16];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            x[2 * i] = u2f(blk.w[i] << 16);
-            x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
+            if (F16) {
+                x[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)blk.w[i]);
+                x[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(blk.w[i] >> 16));
+            } else {
+                x[2 * i] = u2f(blk.w[i] << 16);
+                x[2 * i + 1] = u2f(blk.w[i] & 0xffff0000u);
+            }
         }
         float bmax = 0.0f;
 #pragma unroll
@@ -468,14 +481,14 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 else if (k.exact_ok) {
                     if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
                     else pickB = exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
-                } else return generic_block<RULE, TWO_D>(blk, k);
+                } else return generic_block<RULE, TWO_D, F16>(blk, k);
             }
             return BlockOut{pickB ? b0 : a0, pickB ? b1 : a1, pickB ? s4 : s6};
         }
         if (bmax == 0.0f) return BlockOut{0, 0, 0};  // an all-zero block: zero codes, zero scale
     }
     if constexpr (SR) return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);
-    else return generic_block<RULE, TWO_D>(blk, k);
+    else return generic_block<RULE, TWO_D, F16>(blk, k);
 }
 
 // ---------------------------------------------------------------------------------------

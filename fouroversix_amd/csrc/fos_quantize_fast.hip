@@ -141,7 +141,8 @@ struct RowsTile {
 
 // IF4: the IF4 format with its MSE rule (E2M1 candidate against INT4 candidate on one scale,
 // quantize_block_if4_mse) instead of NVFP4.
-template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false>
+// F16: fp16 elements instead of bf16 (NVFP4, round to nearest, codes out).
+template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false, bool F16 = false>
 // (the stochastic instantiations hold two sets of scaled values and the Philox state: with 128
 // registers they spilled -- 30 MB of scratch traffic per launch at 8192 x 8192 -- and the launch
 // grid of three workgroups per compute unit leaves 168; the IF4 instantiation spilled as well)
@@ -236,7 +237,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     k.dec = 1.0f / (p.c / k.amax);
     k.qdiv = p.qdiv;
     k.errdiv = p.errdiv;
-    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
+    // (the exact evaluation needs fq * s * amax exact: a maximum of the element type's significant bits)
+    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & (F16 ? 0x1fffu : 0xffffu)) == 0;
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         BlockOut o{0u, 0u, 0u};
         if (!padding_step) {
             if constexpr (IF4) o = quantize_block_if4_mse<false>(b, k, enc_fast, rq, in_range, lut);
-            else o = quantize_block_nvfp4_fast<RULE, false, SR>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+            else o = quantize_block_nvfp4_fast<RULE, false, SR, F16>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
                                                                 (uint64_t)(row * sf_cols + t.cb));
         }
         if (PSEUDO) {
@@ -356,6 +358,15 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         p.tile_map = kMapRowMajor;
         if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
+        if constexpr (!PSEUDO && !SR) {
+            if (p.x_type == FOS_T_F16) {
+                if (full)
+                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+                else
+                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+                return;
+            }
+        }
         if (full)
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else

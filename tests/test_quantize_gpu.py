@@ -89,8 +89,8 @@ def test_fp32_and_fp16_inputs_match_reference_vectors(golden_dir):
     dict(dtype="if4", scale_rule="abs_max", round_style="stochastic"),
 ], ids=str)
 def test_fp32_and_fp16_inputs_match_oracle(oracle, in_dtype, cfg):
-    """Every rule / format / rounding style on fp32 and fp16 data (element-wise kernel), aligned and
-    ragged shapes, strided rows; bf16 values handed over in the wider type give the bf16 kernels' bytes."""
+    """Every rule / format / rounding style on fp32 and fp16 data (element-wise kernel, and the streaming one for
+    aligned fp16 NVFP4 inputs with 1x16 blocks and round to nearest), aligned and ragged shapes, strided rows; bf16 values handed over in the wider type give the bf16 kernels' bytes."""
     g = torch.Generator("cpu").manual_seed(17)
     kwargs = {"seed": 7, "offset": 1} if "round_style" in cfg else {}
     okw = dict(seed=7, offset=1) if "round_style" in cfg else {}
@@ -108,6 +108,41 @@ def test_fp32_and_fp16_inputs_match_oracle(oracle, in_dtype, cfg):
         base = hip_quantize(xb, kwargs=kwargs, **cfg)
         assert torch.equal(same.values, base.values) and torch.equal(same.scale_factors.view(torch.uint8), base.scale_factors.view(torch.uint8))
         assert float(same.amax) == float(base.amax)
+
+
+@pytest.mark.parametrize("rule", NVFP4_RULES)
+def test_fp16_inputs_on_the_streaming_kernel(oracle, rule):
+    """Aligned fp16 inputs with 1x16 blocks and round to nearest run on the streaming kernel (fp16 instantiation):
+    bit-exact with the oracle at full size, on ragged shapes, on fp16's own corner values (sub-normals, the
+    largest finite values, 11-bit significands next to block maxima), with a caller's maximum of 24
+    significant bits (undecided blocks take the operation-by-operation form), and on strided rows."""
+    g = torch.Generator("cpu").manual_seed(23)
+    cfg = dict(scale_rule=rule)
+    big = (torch.randn(2048, 4096, generator=g) * 2.0).half()
+    big[5, 7] = 900.0  # an outlier: most block scales become small
+    assert_same_quantization(hip_quantize(big, **cfg), oracle.quantize(big, **cfg), f"fp16 2048x4096 {rule}")
+    flat = (torch.rand(8192, 2048, generator=g) * 4.0).half()  # >= 16 MiB, cols % 2048 == 0: window-order scan
+    assert_same_quantization(hip_quantize(flat, **cfg), oracle.quantize(flat, **cfg), f"fp16 8192x2048 {rule}")
+    for shape in ((130, 272), (100, 80), (16, 4096), (257, 1024)):
+        x = (torch.randn(*shape, generator=g) * 3.0).half()
+        assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), f"fp16 {shape} {rule}")
+    # corner values: sub-normals (down to 2^-24), 65504, values one fp16 ulp apart, exact grid values
+    c = torch.zeros(256, 256, dtype=torch.float16)
+    c[0, :16] = torch.tensor([6e-8, 1.2e-7, -6e-8, 5.96e-8] * 4, dtype=torch.float16)
+    c[1, :16] = torch.tensor([65504.0, -65504.0, 32752.0, 1.0] * 4, dtype=torch.float16)
+    c[2, :16] = torch.tensor([1.0, 1.0009765625, 0.99951171875, 1.5] * 4, dtype=torch.float16)
+    c[3:, :] = (torch.randn(253, 256, generator=g) * 1e-3).half()
+    for scale in (1.0, 2.0 ** -10):
+        x = (c.float() * scale).half()
+        assert_same_quantization(hip_quantize(x, **cfg), oracle.quantize(x, **cfg), f"fp16 corners x{scale} {rule}")
+    x = (torch.randn(512, 1024, generator=g)).half()
+    given = float(np.float32(float(x.abs().max()) * 1.2345678))
+    q = fos.quantize(x.cuda(), fos.QuantizationConfig(kwargs={"amax": torch.tensor(given, device="cuda")}, **cfg))
+    assert_same_quantization(q, oracle.quantize(x, amax=given, **cfg), f"fp16 amax given {rule}")
+    wide = torch.randn(256, 1024, generator=g).half().cuda()
+    view = wide[:, 256:768]
+    assert_same_quantization(fos.quantize(view, fos.QuantizationConfig(**cfg)), oracle.quantize(view.cpu().contiguous(), **cfg),
+                             f"fp16 strided {rule}")
 
 
 def test_fp32_and_fp16_inputs_other_paths(oracle):
