@@ -18,6 +18,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fos_buffer.h"
 #include "fos_quantize_common.h"
 #include "fouroversix_hip.h"
 
@@ -117,10 +118,16 @@ FOS_DEVICE void write_partials(uint32_t m, uint32_t z, uint32_t *partials) {
     }
 }
 
-// RHT without transposition: one thread per group of 16, grid-stride.
+// RHT without transposition: one thread per group of 16, grid-stride.  A lane's 32 output bytes would leave
+// as two stores of 16, each instruction covering half of every line; where the wavefront's 64 groups are
+// consecutive in one row (cols % 1024 == 0) they are exchanged through 2 KiB of LDS instead, so that lane l
+// stores the 16-byte pieces l and 64 + l of the 2 KiB run: whole lines per instruction, stored non-temporally.
 template <bool F16>
 __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParams p) {
+    __shared__ __attribute__((aligned(16))) uint4 swap[kThreads / 64][128];
     const int64_t groups_per_row = (p.cols + 15) >> 4;  // a last, partial group is completed with zeros
+    const bool runs = (groups_per_row & 63) == 0;        // (then n_units % 64 == 0 as well: whole wavefronts)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t m = 0, z = 0;
     for (int64_t g = (int64_t)blockIdx.x * kThreads + threadIdx.x; g < p.n_units; g += (int64_t)gridDim.x * kThreads) {
         const int64_t r = g / groups_per_row, cb = g - r * groups_per_row;
@@ -129,27 +136,48 @@ __global__ __launch_bounds__(kThreads) void rht_rows_kernel(const TransformParam
         rht16<F16>(w);
         track(w, m, z);
         uint4 *dst = reinterpret_cast<uint4 *>(p.y + r * p.ldy + cb * 16);
-        dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
-        dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        if (runs) {
+            swap[wave][2 * lane] = make_uint4(w[0], w[1], w[2], w[3]);
+            swap[wave][2 * lane + 1] = make_uint4(w[4], w[5], w[6], w[7]);
+            // (LDS operations of one wavefront complete in order: its own writes are visible to its reads)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const uint4 a = swap[wave][lane], b = swap[wave][64 + lane];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            uint4 *run = dst - 2 * lane;  // the wavefront's first group
+            stream_store(run + lane, a);
+            stream_store(run + 64 + lane, b);
+        } else {
+            dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+            dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        }
     }
     write_partials<F16>(m, z, p.partials);
 }
 
-// Transposition (optionally followed by the RHT along the new rows) through a 64 x 64 LDS
-// tile: rows of x come in as 128-byte runs, rows of y leave as 128-byte runs.  Groups of 16
-// that reach past the last row / column are completed with zeros (y is written in whole groups:
-// its rows hold a multiple of 16 elements).
+// Transposition (optionally followed by the RHT along the new rows) through an LDS tile of 64 rows x 128
+// columns of x: rows of x come in as 256-byte runs (eight threads to a row), rows of y leave as 128-byte
+// runs (four threads to a row of y, which holds 64 elements of this tile).  Groups of 16 that reach past
+// the last row / column are completed with zeros (y is written in whole groups: its rows hold a multiple of
+// 16 elements).
+constexpr int kTR = 64, kTC = 128;  // tile rows / columns of x (64 x 64: 3 % slower; 64 x 256, 128 x 128, 128 x 256: 1-4 % slower)
 template <bool RHT, bool F16>
 __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformParams p) {
-    constexpr int kPitchT = 66;  // halfs per LDS row: 33 dwords, odd, so a column walk changes bank every row
-    __shared__ uint16_t tile[64 * kPitchT];
+    constexpr int kPitchT = kTC + 2;  // halfs per LDS row: an odd number of dwords, so a column walk changes bank every row
+    __shared__ uint16_t tile[kTR * kPitchT];
     const int t = threadIdx.x;
     uint32_t m = 0, z = 0;
+    constexpr int kChunks = kTC / 16, kRowsPerPass = kThreads / kChunks;
+    constexpr int kRowGroups = kTR / 16, kLaneGroups = kRowGroups < 4 ? kRowGroups : 4, kGroupPasses = kRowGroups / kLaneGroups;
+    constexpr int kColsPerPass = kThreads / kLaneGroups;
     for (int64_t u = blockIdx.x; u < p.n_units; u += gridDim.x) {
         const int64_t ty = u / p.tiles_x, tx = u - ty * p.tiles_x;
-        const int64_t r0 = ty * 64, c0 = tx * 64;
-        {
-            const int row = t >> 2, chunk = t & 3;
+        const int64_t r0 = ty * kTR, c0 = tx * kTC;
+#pragma unroll
+        for (int i = 0; i < kTR / kRowsPerPass; ++i) {
+            const int row = t / kChunks + kRowsPerPass * i, chunk = t % kChunks;
             uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             if (r0 + row < p.rows && c0 + chunk * 16 < p.cols) load_group(p, r0 + row, c0 + chunk * 16, w);
             uint32_t *d = reinterpret_cast<uint32_t *>(tile + row * kPitchT + chunk * 16);
@@ -157,8 +185,11 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
             for (int j = 0; j < 8; ++j) d[j] = w[j];
         }
         __syncthreads();
-        {
-            const int rb = t & 3, c = t >> 2;  // output row c0 + c, output columns r0 + 16 rb ...
+#pragma unroll
+        for (int i = 0; i < kGroupPasses * (kTC / kColsPerPass); ++i) {
+            // output row c0 + c, output columns r0 + 16 rb ...; a wavefront spans at most four row groups, which
+            // keeps its 16-bit LDS reads on distinct banks
+            const int rb = t % kLaneGroups + kLaneGroups * (i % kGroupPasses), c = t / kLaneGroups + kColsPerPass * (i / kGroupPasses);
             if (c0 + c < p.cols && r0 + rb * 16 < p.rows) {
                 uint32_t w[8];
 #pragma unroll
@@ -168,6 +199,8 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
                 }
                 if (RHT) rht16<F16>(w);
                 track(w, m, z);
+                // (exchanging the pieces through LDS so that every store instruction covers whole lines, as
+                // rht_rows_kernel does, changed nothing here: 68.5 us either way)
                 uint4 *dst = reinterpret_cast<uint4 *>(p.y + (c0 + c) * p.ldy + r0 + rb * 16);
                 dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
                 dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
@@ -215,8 +248,8 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
     int64_t grid;
     constexpr int64_t kMaxGrid = 1024;  // pairs the workspace holds
     if (transpose) {
-        p.tiles_x = (int)((cols + 63) / 64);
-        p.n_units = ((rows + 63) / 64) * p.tiles_x;
+        p.tiles_x = (int)((cols + kTC - 1) / kTC);
+        p.n_units = ((rows + kTR - 1) / kTR) * p.tiles_x;
         grid = p.n_units < kMaxGrid ? p.n_units : kMaxGrid;
         if (rht && f16) hipLaunchKernelGGL((transpose_kernel<true, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else if (rht) hipLaunchKernelGGL((transpose_kernel<true, false>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
