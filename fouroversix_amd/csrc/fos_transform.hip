@@ -170,40 +170,59 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
     const int t = threadIdx.x;
     uint32_t m = 0, z = 0;
     constexpr int kChunks = kTC / 16, kRowsPerPass = kThreads / kChunks;
-    constexpr int kRowGroups = kTR / 16, kLaneGroups = kRowGroups < 4 ? kRowGroups : 4, kGroupPasses = kRowGroups / kLaneGroups;
-    constexpr int kColsPerPass = kThreads / kLaneGroups;
+    // this thread's two groups of 16 input elements of tile u (rows t / 8 and 32 + t / 8, columns 16 (t % 8) ...)
+    auto fetch = [&](int64_t u, uint32_t (&w)[kTR / kRowsPerPass][8]) {
+        const int64_t ty = u / p.tiles_x, tx = u - ty * p.tiles_x;
+#pragma unroll
+        for (int i = 0; i < kTR / kRowsPerPass; ++i) {
+            const int64_t r = ty * kTR + t / kChunks + kRowsPerPass * i, c = tx * kTC + (t % kChunks) * 16;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) w[i][j] = 0;
+            if (r < p.rows && c < p.cols) load_group(p, r, c, w[i]);
+        }
+    };
+    uint32_t next[kTR / kRowsPerPass][8];
+    if ((int64_t)blockIdx.x < p.n_units) fetch(blockIdx.x, next);
     for (int64_t u = blockIdx.x; u < p.n_units; u += gridDim.x) {
         const int64_t ty = u / p.tiles_x, tx = u - ty * p.tiles_x;
         const int64_t r0 = ty * kTR, c0 = tx * kTC;
 #pragma unroll
         for (int i = 0; i < kTR / kRowsPerPass; ++i) {
             const int row = t / kChunks + kRowsPerPass * i, chunk = t % kChunks;
-            uint32_t w[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (r0 + row < p.rows && c0 + chunk * 16 < p.cols) load_group(p, r0 + row, c0 + chunk * 16, w);
             uint32_t *d = reinterpret_cast<uint32_t *>(tile + row * kPitchT + chunk * 16);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) d[j] = w[j];
+            for (int j = 0; j < 8; ++j) d[j] = next[i][j];
         }
         __syncthreads();
+        // the next tile's loads are in flight while this one is turned round and written
+        if (u + gridDim.x < p.n_units) fetch(u + gridDim.x, next);
+        {
+            // a thread turns one group of 16 rows of a column PAIR round: 16 dword reads (row stride 65 dwords:
+            // the 64 lanes of a wavefront, 4 row groups x 16 column pairs, hit 64 different banks) give the two
+            // output rows c0 + 2 cp and c0 + 2 cp + 1, output columns r0 + 16 rb ...
+            static_assert(kTR == 64 && kTC == 128 && kThreads == 256, "one column pair and row group per thread");
+            const int rb = t & 3, cp = t >> 2;
+            const uint32_t *col = reinterpret_cast<const uint32_t *>(tile) + rb * 16 * (kPitchT / 2) + cp;
+            uint32_t d[16];
 #pragma unroll
-        for (int i = 0; i < kGroupPasses * (kTC / kColsPerPass); ++i) {
-            // output row c0 + c, output columns r0 + 16 rb ...; a wavefront spans at most four row groups, which
-            // keeps its 16-bit LDS reads on distinct banks
-            const int rb = t % kLaneGroups + kLaneGroups * (i % kGroupPasses), c = t / kLaneGroups + kColsPerPass * (i / kGroupPasses);
-            if (c0 + c < p.cols && r0 + rb * 16 < p.rows) {
-                uint32_t w[8];
+            for (int k = 0; k < 16; ++k) d[k] = col[k * (kPitchT / 2)];
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t a = tile[(rb * 16 + 2 * j) * kPitchT + c], b = tile[(rb * 16 + 2 * j + 1) * kPitchT + c];
-                    w[j] = a | (b << 16);
+            for (int h = 0; h < 2; ++h) {
+                const int c = 2 * cp + h;
+                if (c0 + c < p.cols && r0 + rb * 16 < p.rows) {
+                    uint32_t w[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        w[j] = h ? __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x07060302u)   // the two high halves
+                                 : __builtin_amdgcn_perm(d[2 * j + 1], d[2 * j], 0x05040100u);  // the two low halves
+                    if (RHT) rht16<F16>(w);
+                    track(w, m, z);
+                    // (exchanging the pieces through LDS so that every store instruction covers whole lines, as
+                    // rht_rows_kernel does, is worth 1 us of 62 here)
+                    uint4 *dst = reinterpret_cast<uint4 *>(p.y + (c0 + c) * p.ldy + r0 + rb * 16);
+                    dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+                    dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
                 }
-                if (RHT) rht16<F16>(w);
-                track(w, m, z);
-                // (exchanging the pieces through LDS so that every store instruction covers whole lines, as
-                // rht_rows_kernel does, changed nothing here: 68.5 us either way)
-                uint4 *dst = reinterpret_cast<uint4 *>(p.y + (c0 + c) * p.ldy + r0 + rb * 16);
-                dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
-                dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
             }
         }
         __syncthreads();
