@@ -17,6 +17,7 @@ void load_tuning() {
     g_tuning.gemm_tile = env_int("FOS_GEMM_TILE");
     g_tuning.gemm_splitk = env_int("FOS_GEMM_SPLITK");
     g_tuning.mx_tile = env_int("FOS_MX_TILE");
+    g_tuning.mx_quant = env_int("FOS_MX_QUANT");
     g_tuning.quant_grid = env_int("FOS_QUANT_GRID");
     g_tuning.amax_grid = env_int("FOS_AMAX_GRID");
     g_tuning.quant_map = env_int("FOS_QUANT_MAP");

@@ -156,6 +156,141 @@ __global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_kernel(const M
     }
 }
 
+// Streaming form for 16-byte aligned rows with cols % 16 == 0: the lane mapping and launch shape of the NVFP4
+// 1x16 kernel (fos_quantize_fast.hip).  A lane owns 16 consecutive elements (two 128-bit buffer loads, one
+// 64-bit non-temporal store of codes), two neighbouring lanes own a 1x32 block (its maximum is one quad
+// permute).  A wavefront covers 4 rows x 512 contiguous bytes per step; a 256-thread workgroup walks a
+// 128 x 256 tile in eight steps with the loads three steps ahead, across tile boundaries; 768 workgroups stride
+// over the tiles, die b % 8 taking the 512-byte windows b % 8, b % 8 + 8, ... of every row.  Wavefront w owns
+// rows 32 q + 8 w + 4 h + i (step 2 q + h, i = lane >> 4): in the 128x4 scale layout the scales of rows r,
+// r + 32, r + 64, r + 96 share a 16-byte unit, so its 32 rows' scales are 128 contiguous bytes of each of the
+// tile's two scale tiles, assembled in 256 bytes of LDS and written by the wavefront itself (no workgroup
+// barrier).  A ragged tile's descriptor ends with the tensor's last row and lanes past the last column get an
+// offset beyond it: both read zeros, which is the padding the reference adds.
+struct MxRowsTile {
+    uint64_t x_base, codes_base;
+    uint32_t x_bytes, x_off;
+    int64_t row_base, cb;  // first row of the tile; this lane's 16-element column group in the tensor
+    uint32_t tile_y, tile_x;
+};
+
+template <bool FULL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void quantize_mxfp4_rows_kernel(const MxQuantParams p) {
+    __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][64];  // per wavefront: 2 scale tiles x 128 bytes
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t sf_cols = p.cols_p >> 5;
+    const int lb = lane & 15;               // 16-element column group inside the tile
+    const int rl = wave * 8 + (lane >> 4);  // this lane's row in step 0
+    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    const int64_t code_pitch = p.cols_p >> 1;
+    const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
+    const uint32_t x_lane = (uint32_t)(rl * p.ld + lb * 16) * 2u, x_row = (uint32_t)p.ld * 2u;
+    const uint32_t c_lane = (uint32_t)(rl * code_pitch + lb * 8), c_row = (uint32_t)code_pitch;
+    auto step_row = [](int g) { return 32 * (g >> 1) + 4 * (g & 1); };
+    // scale byte of (q, h, i; block column b = lb >> 1) in the wavefront's staging area: 128 bytes per scale
+    // tile b >> 2, unit 4 h + i, byte 4 q + (b & 3)
+    uint8_t *stage = reinterpret_cast<uint8_t *>(sf_stage[wave]) + (lb >> 3) * 128 + (lane >> 4) * 16 + ((lb >> 1) & 3);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *p.amax = 1.0f;  // the reference reports amax = 1 (reference.py:573-578)
+
+    auto open_tile = [&](uint32_t tile, bool valid) {
+        MxRowsTile t;
+        t.tile_y = tile / (uint32_t)p.tiles_x;
+        t.tile_x = tile - t.tile_y * (uint32_t)p.tiles_x;
+        t.row_base = (int64_t)t.tile_y * 128;
+        const int64_t col_base = (int64_t)t.tile_x * 256;
+        t.cb = (int64_t)t.tile_x * 16 + lb;
+        uint32_t x_bytes = valid ? 0xffffffffu : 0u;
+        if (!FULL && valid) {
+            const int64_t left = ((p.rows - t.row_base) * p.ld - col_base) * 2;
+            x_bytes = left <= 0 ? 0u : (left > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)left);
+        }
+        t.x_bytes = __builtin_amdgcn_readfirstlane(x_bytes);
+        t.x_base = uniform64((uint64_t)(p.x + t.row_base * p.ld + col_base));
+        t.codes_base = uniform64((uint64_t)(p.codes + t.row_base * code_pitch + col_base / 2));
+        t.x_off = (FULL || t.cb * 16 < p.cols) ? x_lane : 0x80000000u;
+        return t;
+    };
+    auto load = [&](const MxRowsTile &t, int g, uint32_t (&w)[8]) {
+        const BufferRsrc rx = make_rsrc(reinterpret_cast<const void *>(uniform64(t.x_base)), __builtin_amdgcn_readfirstlane(t.x_bytes));
+        u32x4 lo, hi;
+        if (FULL) {
+            lo = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off, step_row(g) * x_row, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + 16u, step_row(g) * x_row, 0);
+        } else {
+            // the range check covers the per-lane offset only: keep the step inside it
+            lo = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + step_row(g) * x_row, 0, 0);
+            hi = __builtin_amdgcn_raw_buffer_load_b128(rx, t.x_off + step_row(g) * x_row + 16u, 0, 0);
+        }
+        w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
+        w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
+    };
+    auto process = [&](const MxRowsTile &t, int g, const uint32_t (&w)[8]) {
+        // block maximum: 16 elements of this lane, then the neighbour's (all lanes: the permute needs both)
+        uint32_t m = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m = pk_max_u16(m, w[i] & 0x7fff7fffu);
+        uint32_t mm = (m & 0xffffu) > (m >> 16) ? (m & 0xffffu) : (m >> 16);
+        const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)mm, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+        mm = mm > other ? mm : other;
+        if (!FULL && t.cb >= (p.cols_p >> 4)) return;  // past the padded width
+        const float s_hp = u2f(mm << 16) / p.qmax;
+        const uint32_t u = f2u(s_hp);
+        uint32_t e = (u >> 23) & 0xffu;
+        if (u & 0x7fffffu) e = (e + 1u) & 0xffu;  // round up to the next power of two
+        // 1 / 2^(e - 127); e == 0 marks an all-zero block (values become 0), 255 is inf / NaN
+        const float inv = e == 0u || e == 255u ? 0.0f : (e == 254u ? u2f(0x00400000u) : u2f((254u - e) << 23));
+        uint32_t c0 = 0, c1 = 0;
+        static_for<0, 4>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            // + 0: a negative zero (also one produced by underflow) must not keep its sign; a negative value
+            // that rounds to zero does (the reference multiplies by sign(x), and sign(-0.0) = 0)
+            c0 = pack_fp4<j>(c0, __builtin_fmaf(u2f(w[j] << 16), inv, 0.0f), __builtin_fmaf(u2f(w[j] & 0xffff0000u), inv, 0.0f));
+            c1 = pack_fp4<j>(c1, __builtin_fmaf(u2f(w[4 + j] << 16), inv, 0.0f), __builtin_fmaf(u2f(w[4 + j] & 0xffff0000u), inv, 0.0f));
+        });
+        const u32x2 c01 = {c0, c1};
+        const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
+        __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, c_lane, step_row(g) * c_row, kStreamStore);
+        if ((lane & 1) == 0) {
+            if (tiled) stage[(g & 1) * 64 + (g >> 1) * 4] = (uint8_t)e;
+            else p.sf[(t.row_base + step_row(g) + rl) * sf_cols + (t.cb >> 1)] = (uint8_t)e;
+        }
+    };
+
+    uint32_t tile = blockIdx.x;
+    MxRowsTile cur = open_tile(tile, tile < n_tiles);
+    uint32_t ring[4][8];
+    load(cur, 0, ring[0]);
+    load(cur, 1, ring[1]);
+    load(cur, 2, ring[2]);
+    while (tile < n_tiles) {
+        const uint32_t next = tile + gridDim.x;
+        const bool has_next = next < n_tiles;
+        const MxRowsTile nxt = open_tile(has_next ? next : tile, has_next);  // without a next tile: loads of nothing
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g + 3 < 8) load(cur, g + 3, ring[(g + 3) & 3]);
+            else load(nxt, g + 3 - 8, ring[(g + 3) & 3]);
+            process(cur, g, ring[g & 3]);
+        }
+        if (tiled) {
+            // the wavefront's own 2 x 128 bytes: written above by its lanes, read back here in output order
+            // (LDS operations of one wavefront complete in order)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int64_t group = (int64_t)cur.tile_x * 2 + (lane >> 4);
+            if (lane < 32 && (FULL || group < (sf_cols >> 2))) {
+                const uint2 v = reinterpret_cast<const uint2 *>(sf_stage[wave])[lane];
+                *reinterpret_cast<uint2 *>(p.sf + ((int64_t)cur.tile_y * (sf_cols >> 2) + group) * 512 + wave * 128 + (lane & 15) * 8) = v;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        cur = nxt;
+        tile = next;
+    }
+}
+
 int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
                           uint8_t *sf, float *amax, hipStream_t s) {
     MxQuantParams p;
@@ -171,6 +306,19 @@ int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld,
     const int64_t grid = (p.rows_p / 128) * p.tiles_x;
     if (grid > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     p.amax = amax;
+    if (p.vector_loads && cols % 16 == 0 && ld < (int64_t{1} << 23) && tuning().mx_quant != 1) {
+        // the streaming form (32-bit byte offsets inside a 128-row tile: rows of less than 16 MiB)
+        p.tiles_x = (int)((p.cols_p + 255) / 256);
+        const int64_t n = (p.rows_p / 128) * p.tiles_x;
+        int64_t launch = 768;
+        if (const int forced = tuning().quant_grid) launch = forced > 0 ? forced : launch;
+        if (launch > n) launch = n;
+        if (rows % 128 == 0 && cols % 256 == 0)
+            hipLaunchKernelGGL(quantize_mxfp4_rows_kernel<true>, dim3((unsigned)launch), dim3(256), 0, s, p);
+        else
+            hipLaunchKernelGGL(quantize_mxfp4_rows_kernel<false>, dim3((unsigned)launch), dim3(256), 0, s, p);
+        return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+    }
     if (p.vector_loads && rows % 128 == 0 && cols % 512 == 0)
         hipLaunchKernelGGL(quantize_mxfp4_kernel<true>, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
     else

@@ -11,6 +11,7 @@ struct Tuning {
     std::atomic<int> gemm_tile{0};    // FOS_GEMM_TILE
     std::atomic<int> gemm_splitk{0};  // FOS_GEMM_SPLITK
     std::atomic<int> mx_tile{0};      // FOS_MX_TILE
+    std::atomic<int> mx_quant{0};     // FOS_MX_QUANT: 1 = the tile kernel of the MXFP4 quantizer also for aligned inputs
     std::atomic<int> quant_grid{0};   // FOS_QUANT_GRID
     std::atomic<int> amax_grid{0};    // FOS_AMAX_GRID
     std::atomic<int> amax_units{0};   // FOS_AMAX_UNITS: -1 = flat pass 1 also ahead of a streaming pass 2

@@ -79,6 +79,43 @@ def test_mxfp4_quantize_dequantize_match_oracle(oracle, kind, shape, scale, rule
     assert np.array_equal(fos.dequantize(q, torch.float16).cpu().numpy().view(np.uint16), rdeq.astype(np.float16).view(np.uint16))
 
 
+def test_mxfp4_streaming_kernel_full_size_and_layouts(oracle, monkeypatch):
+    """Aligned inputs run on the streaming kernel: bit-exact with the oracle at 8192 x 4096 and on a strided
+    view, identical to the tile kernel, and its row-major scale output (C ABI) is the tiled one re-ordered."""
+    from fouroversix_amd import _native as nat
+
+    x = make_input("outlier", (8192, 4096), 77)
+    ref = oracle.quantize_mxfp4(x, scale_rule="static_6")
+    q = fos.quantize(x.cuda(), mx_config())
+    assert np.array_equal(u8(q.values), ref.values) and np.array_equal(u8(q.scale_factors).reshape(-1), ref.scale_factors)
+    monkeypatch.setenv("FOS_MX_QUANT", "1")  # the tile kernel
+    q_tile = fos.quantize(x.cuda(), mx_config())
+    monkeypatch.delenv("FOS_MX_QUANT")
+    assert torch.equal(q_tile.values, q.values) and torch.equal(q_tile.scale_factors.view(torch.uint8), q.scale_factors.view(torch.uint8))
+    wide = make_input("randn", (384, 2048), 78).cuda()
+    view = wide[:, 512:1536]
+    rv = oracle.quantize_mxfp4(view.cpu().contiguous(), scale_rule="static_4")
+    qv = fos.quantize(view, mx_config("static_4"))
+    assert np.array_equal(u8(qv.values), rv.values) and np.array_equal(u8(qv.scale_factors).reshape(-1), rv.scale_factors)
+    # row-major scales through the C ABI (ragged rows, half a 256-column tile at the end)
+    L = nat.lib()
+    rows, cols = 200, 640
+    xs = make_input("randn", (rows, cols), 79).cuda()
+    rows_p, cols_p = 256, 640
+    outs = {}
+    for layout in (nat.SF_TILED, nat.SF_LINEAR):
+        codes = torch.zeros(rows_p, cols_p // 2, dtype=torch.uint8, device="cuda")
+        sf = torch.zeros(rows_p * cols_p // 32, dtype=torch.uint8, device="cuda")
+        amax = torch.zeros(1, dtype=torch.float32, device="cuda")
+        ws = torch.empty(L.fos_quantize_workspace_bytes(rows, cols), dtype=torch.uint8, device="cuda")
+        nat.check(L.fos_quantize(xs.data_ptr(), nat.T_BF16, rows, cols, cols, 2, 0, 0, 0, 0, 0, layout, codes.data_ptr(), sf.data_ptr(),
+                                 amax.data_ptr(), 0, ws.data_ptr(), ws.numel(), nat.current_stream(xs.device)), "quantize")
+        torch.cuda.synchronize()
+        outs[layout] = (codes.cpu().numpy(), sf.cpu().numpy())
+    assert np.array_equal(outs[nat.SF_TILED][0], outs[nat.SF_LINEAR][0])
+    assert np.array_equal(oracle.from_blocked(outs[nat.SF_TILED][1], rows_p, cols_p // 32).reshape(-1), outs[nat.SF_LINEAR][1])
+
+
 def test_mxfp4_unsupported_configurations():
     x = make_input("randn", (128, 128), 1).cuda()
     for bad in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True),
