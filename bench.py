@@ -351,7 +351,7 @@ def main() -> int:
                                  amax.data_ptr(), 1, ws.data_ptr(), ws_bytes, stream), "quantize")), K)
     q_achieved = algo_bytes / (quant_ms * 1e-3) / 1e9
     roofline = {
-        "kernel": "fos::quantize_nvfp4_rows_kernel<3, true, false, false, false> (pass 2: scale, 4/6 select, pack)",
+        "kernel": "fos::quantize_nvfp4_rows_kernel<3, true, false, false, false, false> (pass 2: scale, 4/6 select, pack)",
         "bound": "hbm",
         "achieved": round(q_achieved, 1),
         "peak": HBM_PEAK_GBS,
