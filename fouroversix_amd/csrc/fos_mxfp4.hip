@@ -174,7 +174,9 @@ struct MxRowsTile {
     uint32_t tile_y, tile_x;
 };
 
-template <bool FULL>
+// F16: fp16 elements instead of bf16 (magnitudes of either type order like their bit patterns; both convert
+// to f32 exactly).
+template <bool FULL, bool F16 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void quantize_mxfp4_rows_kernel(const MxQuantParams p) {
     __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][64];  // per wavefront: 2 scale tiles x 128 bytes
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -233,19 +235,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void q
         const uint32_t other = (uint32_t)__builtin_amdgcn_mov_dpp((int)mm, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
         mm = mm > other ? mm : other;
         if (!FULL && t.cb >= (p.cols_p >> 4)) return;  // past the padded width
-        const float s_hp = u2f(mm << 16) / p.qmax;
+        const float bmax = F16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)mm) : u2f(mm << 16);
+        const float s_hp = bmax / p.qmax;
         const uint32_t u = f2u(s_hp);
         uint32_t e = (u >> 23) & 0xffu;
         if (u & 0x7fffffu) e = (e + 1u) & 0xffu;  // round up to the next power of two
         // 1 / 2^(e - 127); e == 0 marks an all-zero block (values become 0), 255 is inf / NaN
         const float inv = e == 0u || e == 255u ? 0.0f : (e == 254u ? u2f(0x00400000u) : u2f((254u - e) << 23));
+        auto lo_of = [](uint32_t word) { return F16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)word) : u2f(word << 16); };
+        auto hi_of = [](uint32_t word) { return F16 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(word >> 16)) : u2f(word & 0xffff0000u); };
         uint32_t c0 = 0, c1 = 0;
         static_for<0, 4>([&](auto jc) {
             constexpr int j = decltype(jc)::value;
             // + 0: a negative zero (also one produced by underflow) must not keep its sign; a negative value
             // that rounds to zero does (the reference multiplies by sign(x), and sign(-0.0) = 0)
-            c0 = pack_fp4<j>(c0, __builtin_fmaf(u2f(w[j] << 16), inv, 0.0f), __builtin_fmaf(u2f(w[j] & 0xffff0000u), inv, 0.0f));
-            c1 = pack_fp4<j>(c1, __builtin_fmaf(u2f(w[4 + j] << 16), inv, 0.0f), __builtin_fmaf(u2f(w[4 + j] & 0xffff0000u), inv, 0.0f));
+            c0 = pack_fp4<j>(c0, __builtin_fmaf(lo_of(w[j]), inv, 0.0f), __builtin_fmaf(hi_of(w[j]), inv, 0.0f));
+            c1 = pack_fp4<j>(c1, __builtin_fmaf(lo_of(w[4 + j]), inv, 0.0f), __builtin_fmaf(hi_of(w[4 + j]), inv, 0.0f));
         });
         const u32x2 c01 = {c0, c1};
         const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
@@ -291,7 +296,70 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void q
     }
 }
 
-int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
+// fp32 inputs, and fp16 ones that the streaming kernel does not take: the tile shape and scale staging of
+// quantize_mxfp4_kernel with elements read one by one and converted to f32 (exact for both types), which is
+// where the reference's arithmetic starts (`.float()`, reference.py:149-181).
+template <bool F32>
+__global__ __launch_bounds__(kMxQuantThreads) void quantize_mxfp4_typed_kernel(const MxQuantParams p) {
+    __shared__ uint32_t sf_stage[4 * 128];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lb = lane >> 2;  // block column inside the tile
+    const int64_t sf_cols = p.cols_p >> 5;
+    const int64_t tile_y = blockIdx.x / p.tiles_x, tile_x = blockIdx.x - tile_y * p.tiles_x;
+    const int64_t cb = tile_x * 16 + lb;
+    const int64_t c0 = tile_x * 512 + lane * 8;  // first column of this lane's 8 elements
+    const bool col_ok = cb < sf_cols;
+    const bool tiled = p.sf_layout == FOS_SF_TILED_128X4;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *p.amax = 1.0f;
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int rr = g * 32 + wave * 4 + j;
+            const int64_t r = tile_y * 128 + rr;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[i] = 0.0f;
+                if (r < p.rows && c0 + i < p.cols) {
+                    if (F32) v[i] = reinterpret_cast<const float *>(p.x)[r * p.ld + c0 + i];
+                    else v[i] = (float)__builtin_bit_cast(_Float16, p.x[r * p.ld + c0 + i]);
+                }
+            }
+            // block maximum over the four lanes of the block (all lanes: the permutes need their neighbours)
+            float bmax = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) bmax = fmaxf(bmax, fabsf(v[i]));
+            bmax = u2f(quad_max_u32(f2u(bmax)));  // non-negative floats order like their bit patterns
+            const float s_hp = bmax / p.qmax;
+            const uint32_t u = f2u(s_hp);
+            uint32_t e = (u >> 23) & 0xffu;
+            if (u & 0x7fffffu) e = (e + 1u) & 0xffu;
+            const float inv = e == 0u || e == 255u ? 0.0f : (e == 254u ? u2f(0x00400000u) : u2f((254u - e) << 23));
+            uint32_t codes = 0;
+            static_for<0, 4>([&](auto jc) {
+                constexpr int q = decltype(jc)::value;
+                codes = pack_fp4<q>(codes, __builtin_fmaf(v[2 * q], inv, 0.0f), __builtin_fmaf(v[2 * q + 1], inv, 0.0f));
+            });
+            if (!col_ok) continue;
+            *reinterpret_cast<uint32_t *>(p.codes + r * (p.cols_p >> 1) + (c0 >> 1)) = codes;
+            if ((lane & 3) == 0) {
+                if (tiled) reinterpret_cast<uint8_t *>(sf_stage)[(lb >> 2) * 512 + (rr & 31) * 16 + (rr >> 5) * 4 + (lb & 3)] = (uint8_t)e;
+                else p.sf[r * sf_cols + cb] = (uint8_t)e;
+            }
+        }
+    }
+    if (tiled) {
+        __syncthreads();
+        const int t = threadIdx.x >> 6;  // wavefronts 0-3: one scale tile each, 512 bytes, 8 per lane
+        const int64_t group = tile_x * 4 + t;
+        if (t < 4 && group < (sf_cols >> 2)) {
+            uint2 *out = reinterpret_cast<uint2 *>(p.sf + (tile_y * (sf_cols >> 2) + group) * 512);
+            out[lane] = reinterpret_cast<const uint2 *>(sf_stage)[threadIdx.x];
+        }
+    }
+}
+
+int launch_quantize_mxfp4(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
                           uint8_t *sf, float *amax, hipStream_t s) {
     MxQuantParams p;
     p.x = static_cast<const uint16_t *>(x);
@@ -306,17 +374,28 @@ int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld,
     const int64_t grid = (p.rows_p / 128) * p.tiles_x;
     if (grid > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     p.amax = amax;
-    if (p.vector_loads && cols % 16 == 0 && ld < (int64_t{1} << 23) && tuning().mx_quant != 1) {
+    const bool streams = x_type != FOS_T_F32 && p.vector_loads && cols % 16 == 0 && ld < (int64_t{1} << 23) &&
+                         (tuning().mx_quant != 1 || x_type == FOS_T_F16);
+    if (!streams && x_type != FOS_T_BF16) {
+        if (x_type == FOS_T_F32) hipLaunchKernelGGL(quantize_mxfp4_typed_kernel<true>, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
+        else hipLaunchKernelGGL(quantize_mxfp4_typed_kernel<false>, dim3((unsigned)grid), dim3(kMxQuantThreads), 0, s, p);
+        return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+    }
+    if (streams) {
         // the streaming form (32-bit byte offsets inside a 128-row tile: rows of less than 16 MiB)
         p.tiles_x = (int)((p.cols_p + 255) / 256);
         const int64_t n = (p.rows_p / 128) * p.tiles_x;
         int64_t launch = 768;
         if (const int forced = tuning().quant_grid) launch = forced > 0 ? forced : launch;
         if (launch > n) launch = n;
-        if (rows % 128 == 0 && cols % 256 == 0)
-            hipLaunchKernelGGL(quantize_mxfp4_rows_kernel<true>, dim3((unsigned)launch), dim3(256), 0, s, p);
-        else
-            hipLaunchKernelGGL(quantize_mxfp4_rows_kernel<false>, dim3((unsigned)launch), dim3(256), 0, s, p);
+        const bool full = rows % 128 == 0 && cols % 256 == 0;
+        if (x_type == FOS_T_F16) {
+            if (full) hipLaunchKernelGGL((quantize_mxfp4_rows_kernel<true, true>), dim3((unsigned)launch), dim3(256), 0, s, p);
+            else hipLaunchKernelGGL((quantize_mxfp4_rows_kernel<false, true>), dim3((unsigned)launch), dim3(256), 0, s, p);
+        } else {
+            if (full) hipLaunchKernelGGL((quantize_mxfp4_rows_kernel<true, false>), dim3((unsigned)launch), dim3(256), 0, s, p);
+            else hipLaunchKernelGGL((quantize_mxfp4_rows_kernel<false, false>), dim3((unsigned)launch), dim3(256), 0, s, p);
+        }
         return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
     }
     if (p.vector_loads && rows % 128 == 0 && cols % 512 == 0)

@@ -360,12 +360,13 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     if (dtype == FOS_DTYPE_MXFP4) {
         // one streaming kernel; no tensor maximum, no workspace
         if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
-        if (x_type != FOS_T_BF16 || pseudo_out || block2d || round_style != FOS_ROUND_NEAREST || amax_is_input ||
-            (rule != FOS_RULE_STATIC_6 && rule != FOS_RULE_STATIC_4))
+        if ((x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) || pseudo_out || block2d ||
+            round_style != FOS_ROUND_NEAREST || amax_is_input || (rule != FOS_RULE_STATIC_6 && rule != FOS_RULE_STATIC_4))
             return FOS_E_UNSUPPORTED;
         if (sf_layout != FOS_SF_LINEAR && sf_layout != FOS_SF_TILED_128X4) return FOS_E_UNSUPPORTED;
-        if (((uintptr_t)x & 1) || ((uintptr_t)codes & 15) || ((uintptr_t)sf & 7) || ((uintptr_t)amax & 3)) return FOS_E_BAD_ALIGNMENT;
-        return launch_quantize_mxfp4(x, rows, cols, ld, rule, sf_layout, codes, sf, amax, (hipStream_t)stream);
+        if (((uintptr_t)x & (x_type == FOS_T_F32 ? 3 : 1)) || ((uintptr_t)codes & 15) || ((uintptr_t)sf & 7) || ((uintptr_t)amax & 3))
+            return FOS_E_BAD_ALIGNMENT;
+        return launch_quantize_mxfp4(x, x_type, rows, cols, ld, rule, sf_layout, codes, sf, amax, (hipStream_t)stream);
     }
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if (x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) return FOS_E_UNSUPPORTED;

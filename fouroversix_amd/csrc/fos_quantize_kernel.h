@@ -175,7 +175,7 @@ void launch_quantize_if4_mse_rows(QuantParams &p, hipStream_t s);
 void launch_quantize_if4_mse_tiles(QuantParams &p, hipStream_t s);
 
 // MXFP4 (fos_mxfp4.hip)
-int launch_quantize_mxfp4(const void *x, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
+int launch_quantize_mxfp4(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, int rule, int sf_layout, uint8_t *codes,
                           uint8_t *sf, float *amax, hipStream_t s);
 
 }  // namespace fos

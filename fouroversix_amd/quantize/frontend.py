@@ -38,10 +38,6 @@ def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | Non
         return f"input must live on the GPU, got {x.device}"
     if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         return f"input must be bfloat16, float16 or float32, got {x.dtype}"
-    if x.dtype != torch.bfloat16 and config.dtype == DataType.mxfp4:
-        # the reference converts any input with `.float()` (quantize/pytorch/reference.py:577,593,596);
-        # here the element-wise nvfp4 / if4 kernel reads the other two types
-        return f"mxfp4 takes bfloat16 input only, got {x.dtype}"
     if x.dtype == torch.float32 and (config.rht or config.transpose):
         # (the reference's fp32 product with the Hadamard matrix is a library fp32 matmul, whose
         # summation order is not fixed: there is nothing bit-exact to match)
@@ -106,7 +102,7 @@ def quantize(
     x: torch.Tensor,
     config: QuantizationConfig | None = None,
 ) -> QuantizedTensor | torch.Tensor:
-    """Quantize a 2-D bf16 (nvfp4 / if4: also fp16 or fp32) GPU tensor to a block-scaled 4-bit format.
+    """Quantize a 2-D bf16, fp16 or fp32 GPU tensor to a block-scaled 4-bit format.
 
     With no config: NVFP4, 1x16 blocks, round-to-nearest, 4/6 selection by block MSE.
     ``config.kwargs`` may carry ``seed`` / ``offset`` (ints) keying the dither of the

@@ -88,8 +88,8 @@ _GEMM_WS_BYTES: dict[tuple[int, int, int], int] = {}
 def _quantize_impl(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
     if x.dim() != 2:
         raise RuntimeError("quantize: x must be 2-D")
-    if x.dtype not in nat.TORCH_TO_T or (dtype == MXFP4 and x.dtype != torch.bfloat16):
-        raise RuntimeError(f"quantize: x must be bfloat16 (float16 / float32 for nvfp4 and if4), got {x.dtype}")
+    if x.dtype not in nat.TORCH_TO_T:
+        raise RuntimeError(f"quantize: x must be bfloat16, float16 or float32, got {x.dtype}")
     if x.stride(-1) != 1:
         raise RuntimeError("quantize: x must be contiguous on the last dim")
     nat.require_gpu_tensor(x, "x")

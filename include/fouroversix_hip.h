@@ -88,8 +88,8 @@ int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, 
  *   x_type      FOS_T_BF16; FOS_T_F16 and FOS_T_F32 (the reference converts its input with
  *               `.float()`, reference.py:577,593,596; its native op takes bf16 and fp16,
  *               csrc/quantize/fp4_quant.cu:134-136) give the same results; aligned fp16 rows
- *               with NVFP4, 1x16 blocks and round to nearest run at the bf16 kernels' speed,
- *               the other cases on an element-wise kernel below it
+ *               with NVFP4 (1x16 blocks, round to nearest) or MXFP4 run at the bf16 kernels'
+ *               speed, the other cases on element-wise kernels below it
  *   dtype       FOS_DTYPE_*; rule FOS_RULE_* (IF4 takes only the adaptive rules)
  *   round_style FOS_ROUND_*; seed/offset key the Philox dither of the stochastic styles
  *   block2d     non-zero: one scale and one decision per 16x16 tile

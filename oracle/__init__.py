@@ -354,12 +354,22 @@ def pad_bits_mx(xb: np.ndarray) -> np.ndarray:
 
 
 def quantize_mxfp4(x, *, scale_rule="static_6") -> OracleQuantized:
+    """``x``: bf16 tensor / uint16 bit array, or an fp16 / fp32 torch tensor (the reference converts
+    whatever it is given with ``.float()``; pinned by tests/golden/mxfp4_input_dtypes.npz)."""
     assert scale_rule in ("static_6", "static_4")
-    xb = bf16_bits(x)
-    orig = tuple(int(v) for v in xb.shape)
-    xp = pad_bits_mx(xb)
-    mp, np_ = xp.shape
-    blocks = bf16_bits_to_f32(xp).reshape(-1, 32)
+    if not isinstance(x, np.ndarray) and str(x.dtype) in ("torch.float16", "torch.float32"):
+        xf = x.detach().cpu().float().contiguous().numpy()
+        orig = tuple(int(v) for v in xf.shape)
+        xp32 = np.zeros((-(-orig[0] // 128) * 128, -(-orig[1] // 128) * 128), dtype=np.float32)
+        xp32[: orig[0], : orig[1]] = xf
+        mp, np_ = xp32.shape
+        blocks = xp32.reshape(-1, 32)
+    else:
+        xb = bf16_bits(x)
+        orig = tuple(int(v) for v in xb.shape)
+        xp = pad_bits_mx(xb)
+        mp, np_ = xp.shape
+        blocks = bf16_bits_to_f32(xp).reshape(-1, 32)
     qmax = np.float32(6.0 if scale_rule == "static_6" else 4.0)
     s_hp = (np.abs(blocks).max(axis=1) / qmax).astype(np.float32)
     u = s_hp.view(np.uint32)

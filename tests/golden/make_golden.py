@@ -287,6 +287,28 @@ def write_input_dtype_vectors(quantize, QuantizationConfig) -> None:  # noqa: N8
     print("wrote input_dtypes", len(out))
 
 
+def write_mxfp4_input_dtype_vectors(quantize, QuantizationConfig) -> None:  # noqa: N803
+    """MXFP4 on fp32 and fp16 inputs: quantize_to_mxfp4 converts its input with `.float()`
+    (quantize/pytorch/reference.py:149-181) like the other formats."""
+    out: dict[str, np.ndarray] = {}
+    for name, shape, seed in [("randn_128x256", (128, 256), 71), ("ragged_100x80", (100, 80), 72), ("wide_64x1024", (64, 1024), 73)]:
+        g = torch.Generator("cpu").manual_seed(seed)
+        base = torch.randn(*shape, generator=g) * 3.0
+        base[1, :32] = 0
+        base[2, 5] = -0.0
+        base[3, :8] *= 1e-4
+        for tname, x in (("f32", base), ("f16", base.half())):
+            out[f"{name}.{tname}.x"] = x.numpy().copy() if tname == "f32" else x.numpy().view(np.uint16).copy()
+            for rule in ("static_6", "static_4"):
+                q = quantize(x.clone(), QuantizationConfig(backend="pytorch", dtype="mxfp4", scale_rule=rule))
+                key = f"{name}.{tname}.{rule}"
+                out[key + ".values"] = u8(q.values)
+                out[key + ".sf"] = u8(q.scale_factors)
+                out[key + ".padded"] = np.array(q.padded_shape)
+    np.savez_compressed(os.path.join(HERE, "mxfp4_input_dtypes.npz"), **out)
+    print("wrote mxfp4_input_dtypes", len(out))
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--only-input-dtypes", action="store_true", help="write only input_dtypes.npz")
@@ -296,12 +318,16 @@ def main() -> None:
     ap.add_argument("--only-mxfp4", action="store_true", help="write only mxfp4.npz")
     ap.add_argument("--only-ragged-transpose", action="store_true", help="write only ragged_transpose.npz")
     ap.add_argument("--only-transform-fp16", action="store_true", help="write only transform_fp16.npz")
+    ap.add_argument("--only-mxfp4-dtypes", action="store_true", help="write only mxfp4_input_dtypes.npz")
     args = ap.parse_args()
 
     fos = import_reference()
     from fouroversix import QuantizationConfig, dequantize, quantize, quantized_matmul  # noqa: PLC0415
 
     torch.set_num_threads(os.cpu_count() or 1)
+    write_mxfp4_input_dtype_vectors(quantize, QuantizationConfig)
+    if args.only_mxfp4_dtypes:
+        return
     write_fp16_transform_vectors()
     if args.only_transform_fp16:
         return

@@ -67,7 +67,8 @@ def test_argument_checks_need_no_device(native):
     assert q(ld=32) == -1
     assert q(x_type=3) == -3
     assert q(x_type=2, x=p + 2) == -2  # fp32 elements: 4-byte aligned
-    assert q(x_type=1, dtype=2, rule=0) == -3  # MXFP4 reads bf16 only
+    assert q(x_type=3, dtype=2, rule=0) == -3  # MXFP4: the same three element types
+    assert q(x_type=2, dtype=2, rule=0, x=p + 2) == -2
     assert q(dtype=7) == -3
     assert q(rule=9) == -3
     assert q(dtype=1, rule=0) == -3  # IF4 has no static rule

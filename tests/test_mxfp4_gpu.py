@@ -116,6 +116,33 @@ def test_mxfp4_streaming_kernel_full_size_and_layouts(oracle, monkeypatch):
     assert np.array_equal(oracle.from_blocked(outs[nat.SF_TILED][1], rows_p, cols_p // 32).reshape(-1), outs[nat.SF_LINEAR][1])
 
 
+def test_mxfp4_fp32_and_fp16_inputs(oracle, golden_dir):
+    """fp32 and fp16 inputs (the reference converts with `.float()`): the reference's vectors, and the oracle
+    on aligned (streaming kernel for fp16), ragged and strided inputs."""
+    d = np.load(os.path.join(golden_dir, "mxfp4_input_dtypes.npz"))
+    keys = sorted(k[: -len(".values")] for k in d.files if k.endswith(".values"))
+    assert len(keys) == 12
+    for base in keys:
+        name, tname, rule = base.split(".")
+        raw = d[f"{name}.{tname}.x"]
+        x = torch.from_numpy(raw.copy()) if tname == "f32" else torch.from_numpy(raw.view(np.int16).copy()).view(torch.float16)
+        q = fos.quantize(x.cuda(), mx_config(rule))
+        assert tuple(q.padded_shape) == tuple(d[base + ".padded"]), base
+        assert np.array_equal(u8(q.values), d[base + ".values"]), base
+        assert np.array_equal(u8(q.scale_factors).reshape(-1), d[base + ".sf"].reshape(-1)), base
+        assert float(q.amax) == 1.0
+    g = torch.Generator("cpu").manual_seed(9)
+    for dt in (torch.float16, torch.float32):
+        for shape in ((1024, 2048), (130, 528), (300, 200), (64, 96)):
+            x = (torch.randn(*shape, generator=g) * 2.5).to(dt)
+            x[0, :4] = torch.tensor([6e-8, -6e-8, 65504.0, -0.0]).to(dt)
+            ref = oracle.quantize_mxfp4(x, scale_rule="static_6")
+            for xin in (x.cuda(), torch.nn.functional.pad(x, (0, 3)).cuda()[:, : shape[1]]):  # second: odd row pitch
+                q = fos.quantize(xin, mx_config())
+                assert np.array_equal(u8(q.values), ref.values), (dt, shape)
+                assert np.array_equal(u8(q.scale_factors).reshape(-1), ref.scale_factors), (dt, shape)
+
+
 def test_mxfp4_unsupported_configurations():
     x = make_input("randn", (128, 128), 1).cuda()
     for bad in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True),

@@ -305,6 +305,23 @@ def test_stochastic_rounding_known_answers(oracle):
     assert abs(float((deq - xf).mean())) < 2e-3
 
 
+def test_mxfp4_fp32_and_fp16_inputs_match_reference_vectors(oracle, golden_dir):
+    """MXFP4 on inputs with more significant bits than bf16 (the reference converts with `.float()`)."""
+    import torch
+
+    d = np.load(os.path.join(golden_dir, "mxfp4_input_dtypes.npz"))
+    keys = sorted(k[: -len(".values")] for k in d.files if k.endswith(".values"))
+    assert len(keys) == 12
+    for base in keys:
+        name, tname, rule = base.split(".")
+        raw = d[f"{name}.{tname}.x"]
+        x = torch.from_numpy(raw.copy()) if tname == "f32" else torch.from_numpy(raw.view(np.int16).copy()).view(torch.float16)
+        q = oracle.quantize_mxfp4(x, scale_rule=rule)
+        assert tuple(q.padded_shape) == tuple(d[base + ".padded"]), base
+        assert np.array_equal(q.values, d[base + ".values"]), base
+        assert np.array_equal(q.scale_factors, d[base + ".sf"].reshape(-1)), base
+
+
 def test_mxfp4_matches_reference_vectors(oracle, golden_dir):
     """MXFP4 quantize / dequantize / matmul restatement against vectors written by the
     reference's PyTorch backend (quantize/pytorch/reference.py:149-181, quantize/backend.py:89-160):
