@@ -149,7 +149,8 @@ template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false, bool F16 
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR || IF4) ? 3 : 4))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
-    __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][128];  // per wavefront: 4 scale tiles x 128 bytes
+    // per wavefront: 4 scale tiles x 128 bytes (pseudo-quantize: the 2 KiB of a step's output instead)
+    __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][PSEUDO ? 512 : 128];
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -243,7 +244,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
     const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
-    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
+    // pseudo-quantize: the table also serves the dequantization, whose divisor c is the selection's for the
+    // adaptive rules; the static rules make no selection, so their table is built with c
+    constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
+    QuantConsts kt = k;
+    if (PSEUDO && kStaticRule) kt.errdiv = p.c;
+    const bool deq_lut = PSEUDO && in_range && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, kt);
     __syncthreads();
 
     auto process = [&](const RowsTile &t, int g, const Block16 &b) {
@@ -260,15 +267,35 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         }
         if (PSEUDO) {
             uint32_t w[8];
-            if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+            if (deq_lut) dequant_block_bf16_lut(o, lut[o.s & 0x7fu], w);
+            else if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
             else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
-            if (FULL || (row < p.rows && t.cb * 16 < p.cols)) {
+            const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
+            if constexpr (FULL) {
+                // A lane's 32 bytes would leave as two stores of 16, each instruction covering half of every
+                // line.  The wavefront's 4 rows x 512 bytes go through its staging area instead (free in a
+                // pseudo-quantize launch, which writes no scales): lane l then stores the 16-byte pieces l and
+                // 64 + l of those 2 KiB, whole lines per instruction, non-temporally.
+                uint4 *swap = reinterpret_cast<uint4 *>(sf_stage[wave]);
+                swap[2 * lane] = make_uint4(w[0], w[1], w[2], w[3]);
+                swap[2 * lane + 1] = make_uint4(w[4], w[5], w[6], w[7]);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const uint4 a = swap[lane], b = swap[64 + lane];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                const u32x4 d0 = {a.x, a.y, a.z, a.w}, d1 = {b.x, b.y, b.z, b.w};
+                // piece l: row l >> 5 of the step, bytes 16 (l & 31) ...; piece 64 + l: two rows further down
+                const uint32_t o_off = (uint32_t)(wave * 8 + step_row(g) + (lane >> 5)) * o_row + (uint32_t)(lane & 31) * 16u;
+                __builtin_amdgcn_raw_buffer_store_b128(d0, rout, o_off, 0, kStreamStore);
+                __builtin_amdgcn_raw_buffer_store_b128(d1, rout, o_off + 2u * o_row, 0, kStreamStore);
+            } else if (row < p.rows && t.cb * 16 < p.cols) {
                 const u32x4 d0 = {w[0], w[1], w[2], w[3]}, d1 = {w[4], w[5], w[6], w[7]};
                 // (a 128-bit buffer store with a scalar offset register reads its data late: a VALU
                 // write to the data registers right behind it reached memory in tests, so the step goes
                 // into the per-lane offset)
                 const uint32_t o_off = o_lane + step_row(g) * o_row;
-                const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
                 // (plain stores: the two halves of a line come from two instructions and meet in L2)
                 __builtin_amdgcn_raw_buffer_store_b128(d0, rout, o_off, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b128(d1, rout, o_off + 16u, 0, 0);

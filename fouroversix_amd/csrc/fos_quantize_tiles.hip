@@ -238,7 +238,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     const float rq = sgpr(1.0f / k.qdiv), rc = sgpr(1.0f / p.c);
     k.rerr = sgpr(1.0f / k.errdiv);
     k.fast_div = in_range && k.errdiv == 1536.0f;
-    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
+    // pseudo-quantize: the table also serves the dequantization (divisor c: the selection's for the adaptive
+    // rules; the static rules make no selection, so their table is built with c)
+    constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
+    QuantConsts kt = k;
+    if (PSEUDO && kStaticRule) kt.errdiv = p.c;
+    const bool deq_lut = PSEUDO && in_range && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, kt);
     __syncthreads();
 
 #ifdef FOS_TRACE
@@ -250,7 +256,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         if (PSEUDO) {
             uint32_t w[8];
             const BlockOut o{c0, c1, sbyte};
-            if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+            if (deq_lut) dequant_block_bf16_lut(o, lut[sbyte & 0x7fu], w);
+            else if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
             else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
             if (pred && (FULL || (row < rows32 && t.cb < cols16))) {
                 const u32x4 d0 = {w[0], w[1], w[2], w[3]}, d1 = {w[4], w[5], w[6], w[7]};
