@@ -401,6 +401,35 @@ def test_two_pass_quantize_replays_in_a_hip_graph():
         assert float(static_q.amax) == float(eager.amax), f"replay {i}"
 
 
+@pytest.mark.parametrize("cfg", [dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True), dict(dtype="mxfp4", scale_rule="static_6")],
+                         ids=["nvfp4-mse-1d", "nvfp4-static6-2d", "mxfp4"])
+def test_tensors_beyond_four_gib(cfg):
+    """A 49152 x 49152 input (4.5 GiB, 2^31.2 elements): byte offsets and element counts beyond 32 bits.  Its
+    quantization equals that of its four row bands quantized on their own with the tensor's maximum."""
+    rows = cols = 49152
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.empty(rows, cols, dtype=torch.bfloat16, device="cuda")
+    for r in range(0, rows, 8192):
+        x[r : r + 8192] = torch.randn(8192, cols, generator=g, device="cuda").bfloat16()
+    x[rows - 1, cols - 1] = 40.0  # the maximum sits in the last element
+    q = fos.quantize(x, fos.QuantizationConfig(**cfg))
+    mx = cfg.get("dtype") == "mxfp4"
+    if not mx:
+        assert float(q.amax) == 40.0
+    block = 32 if mx else 16
+    sf = q.scale_factors.view(torch.uint8).reshape(-1)
+    band = rows // 4
+    for i in range(4):
+        kw = {} if mx else {"kwargs": {"amax": q.amax.reshape(1)}}
+        qb = fos.quantize(x[i * band : (i + 1) * band], fos.QuantizationConfig(**cfg, **kw))
+        assert torch.equal(qb.values, q.values[i * band : (i + 1) * band]), (cfg, i)
+        n = band * cols // block  # the tiled layout keeps 128-row bands contiguous
+        assert torch.equal(qb.scale_factors.view(torch.uint8).reshape(-1), sf[i * n : (i + 1) * n]), (cfg, i)
+        del qb
+    del x, q
+    torch.cuda.empty_cache()
+
+
 def test_concurrent_streams_do_not_share_the_workspace(oracle):
     """Two streams quantize different tensors at the same time (the two-launch path, which
     hands partial maxima from pass 1 to pass 2 through a per-stream workspace)."""
