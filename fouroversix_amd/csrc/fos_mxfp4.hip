@@ -581,6 +581,54 @@ FOS_DEVICE void mx_tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) 
     tn = in_band / rows;
 }
 
+// Epilogue of the tile kernels.  acc[i][j][4 g + e] is D[m][n] with m = 32 i + r and
+// n = 32 j + 8 g + 4 h + e (r = lane & 31, h = lane >> 5) of the wavefront's block: stored from
+// the registers, an instruction would touch 32 rows with 16 bytes each (1.6 bytes written to
+// memory per byte of output).  Each wavefront turns a 32-row tile round in its own piece of
+// the operand staging, which is idle by now (the caller has waited for every wavefront), and
+// stores whole rows of its block, 16 bytes per lane.
+template <int WM, int WN, bool OUT_BF16>
+FOS_DEVICE void mx_store_rows(const mx_v16f (&acc)[WM][WN], uint8_t *lds, int wave, int lane, float alpha, uint16_t *D,
+                              int64_t ldd, int64_t m_base, int64_t n_base) {
+    constexpr int kRowBytes = WN * 64, kEpiPitch = kRowBytes + 16;
+    constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerPass = 64 / kLanesPerRow;
+    const int r = lane & 31, h = lane >> 5;
+    uint8_t *epi = lds + wave * 32 * kEpiPitch;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+#pragma unroll
+        for (int j = 0; j < WN; ++j) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint32_t w[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float2_t v = {alpha * acc[i][j][4 * g + 2 * e], alpha * acc[i][j][4 * g + 2 * e + 1]};
+                    if (OUT_BF16) {
+                        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+                    } else {
+                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
+                    }
+                }
+                *reinterpret_cast<uint2 *>(epi + r * kEpiPitch + (j * 32 + 8 * g + 4 * h) * 2) = make_uint2(w[0], w[1]);
+            }
+        }
+        // (LDS operations of one wavefront complete in order: its own writes are visible to its reads)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int t = 0; t < 32 / kRowsPerPass; ++t) {
+            const int row = t * kRowsPerPass + lane / kLanesPerRow, c16 = lane % kLanesPerRow;
+            const uint4 v = *reinterpret_cast<const uint4 *>(epi + row * kEpiPitch + c16 * 16);
+            *reinterpret_cast<uint4 *>(D + (m_base + i * 32 + row) * ldd + n_base + c16 * 8) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
 template <int WAVES_M, int WAVES_N, int WM, int WN, bool OUT_BF16>
 __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const MxGemmParams p) {
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
@@ -733,31 +781,9 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_mxfp4_kernel(const
         kstep(no{}, ks, 0, st[0], st[1], sc[0], sc[1]);
     }
 
-    const float alpha = *p.alpha;
-    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-        const int64_t m = m0 + wm * WM * 32 + i * 32 + r;
-#pragma unroll
-        for (int j = 0; j < WN; ++j) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * h;
-                uint32_t w[2];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const float2_t v = {alpha * acc[i][j][4 * g + 2 * e], alpha * acc[i][j][4 * g + 2 * e + 1]};
-                    if (OUT_BF16) {
-                        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-                    } else {
-                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
-                    }
-                }
-                *reinterpret_cast<uint2 *>(D + m * p.ldd + n) = make_uint2(w[0], w[1]);
-            }
-        }
-    }
+    static_assert(2 * (BM + BN) * kMxPitch >= WAVES_M * WAVES_N * 32 * (WN * 64 + 16), "epilogue staging fits the operand buffers");
+    __syncthreads();  // every wavefront is done reading the operand buffers
+    mx_store_rows<WM, WN, OUT_BF16>(acc, mx_lds, wave, lane, *p.alpha, reinterpret_cast<uint16_t *>(p.D), p.ldd, a_row0, b_row0);
 }
 
 template <int WAVES_M, int WAVES_N, int WM, int WN>
@@ -926,34 +952,12 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_dma_kernel(const MxGemmParams 
                 }
         }
     }
-    // loads still in flight write LDS: drain them before the workgroup gives its LDS up
+    // loads still in flight write LDS: drain them before the stages are used again
     MX_WAIT_VMCNT(0);
+    __syncthreads();  // ... those of every wavefront, and all fragment reads are done
 
-    const float alpha = *p.alpha;
-    uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-        const int64_t m = m0 + wm * WM * 32 + i * 32 + r;
-#pragma unroll
-        for (int j = 0; j < WN; ++j) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int64_t n = n0 + wn * WN * 32 + j * 32 + 8 * g + 4 * h;
-                uint32_t w[2];
-#pragma unroll
-                for (int e = 0; e < 2; ++e) {
-                    const float2_t v = {alpha * acc[i][j][4 * g + 2 * e], alpha * acc[i][j][4 * g + 2 * e + 1]};
-                    if (OUT_BF16) {
-                        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-                    } else {
-                        w[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, mx_half2_t));
-                    }
-                }
-                *reinterpret_cast<uint2 *>(D + m * p.ldd + n) = make_uint2(w[0], w[1]);
-            }
-        }
-    }
+    mx_store_rows<WM, WN, OUT_BF16>(acc, mx_lds, wave, lane, *p.alpha, reinterpret_cast<uint16_t *>(p.D), p.ldd,
+                                     m0 + wm * WM * 32, n0 + wn * WN * 32);
 }
 
 static int launch_gemm_mxfp4_dma(MxGemmParams &p, int out_type, hipStream_t s) {
@@ -978,7 +982,7 @@ extern "C" int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
     if (M <= 0 || N <= 0 || K <= 0 || M % 128 != 0 || N % 128 != 0 || K % 128 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
     if (out_type != FOS_T_BF16 && out_type != FOS_T_F16) return FOS_E_UNSUPPORTED;
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)sfA & 15) || ((uintptr_t)sfB & 15) ||
-        ((uintptr_t)D & 7) || (ldd % 4 != 0) || ((uintptr_t)alpha & 3))
+        ((uintptr_t)D & 15) || (ldd % 8 != 0) || ((uintptr_t)alpha & 3))
         return FOS_E_BAD_ALIGNMENT;
     if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 22)) return FOS_E_BAD_SHAPE;  // a 256-row panel of packed codes stays below 2^31 bytes (32-bit buffer offsets)
     MxGemmParams p;

@@ -235,6 +235,7 @@ size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * (src/fouroversix/csrc/bindings.cpp:26-35, src/fouroversix/matmul/cutlass/backend.py:79-110).
  *   A u8 [M, K/2], B u8 [N, K/2]; sfA, sfB E8M0 bytes in the FOS_SF_TILED_128X4 layout of
  *   [M, K/32] / [N, K/32]; M, N, K multiples of 128 (the padded shapes fos_quantize produces).
+ *   D bf16 / fp16 [M, ldd], 16-byte aligned, ldd a multiple of 8 (rows are stored 16 bytes per lane).
  */
 int fos_gemm_mxfp4(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
                    const float *alpha, int64_t M, int64_t N, int64_t K,
