@@ -1017,7 +1017,7 @@ static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
 
 // Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
 // caller's workspace for splits * M * N FP32 partials).
-enum { kPlanBig, kPlanSmall, kPlanSkinny };
+enum { kPlanBig, kPlanMid, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
@@ -1027,7 +1027,7 @@ constexpr int kTargetWorkgroups = 256;
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
     g.narrow = g.wide = 0;
-    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 1 = no weight-streaming kernel
+    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 256 = 256 x 128 tile wherever M allows, 1 = no weight-streaming kernel
     int64_t steps, tiles;
     if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32 || tile == 64)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
@@ -1051,6 +1051,19 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
         g.kind = kPlanBig;
+        g.splits = 1;
+        g.ksteps_per_split = (int)(K / BK);
+        return g;
+    } else if ((M % 256 == 0) && tile != 128 &&
+               (tile == 256 || ((M / 256) * (N / 128) > 128 && (M / 256) * (N / 128) <= 256) || (M / 256) * (N / 128) > 384)) {
+        // 256 x 128 tiles, one workgroup of eight wavefronts per compute unit, where the 256 x 256
+        // ones would leave compute units idle: B is converted by two wavefronts instead of by
+        // two per 128 rows.  Measured against the 128 x 128 tiles (two workgroups per compute
+        // unit) at K = 4096, by the number T of 256 x 128 tiles: T = 128 57 against 47 us; 192: 65
+        // against 77; 256: 75 against 89; 384: 132-135 against 130; 448: 139 against 159; 896: 224
+        // against 284 -- so not where they cover half of the compute units or one and a half
+        // times all of them.
+        g.kind = kPlanMid;
         g.splits = 1;
         g.ksteps_per_split = (int)(K / BK);
         return g;
@@ -1140,6 +1153,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     p.ksteps_per_split = g.ksteps_per_split;
     switch (g.kind) {
         case kPlanBig: return launch_gemm<2, 4, 4, 2>(p, out_type, s);
+        case kPlanMid: return launch_gemm<2, 4, 4, 1>(p, out_type, s);
         case kPlanSkinny:
             // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);

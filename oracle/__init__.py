@@ -325,10 +325,11 @@ def gemm_nvfp4(values_a, sf_rows_a, values_b, sf_rows_b, alpha, threads=None):
     m, n, k = values_a.shape[0], values_b.shape[0], values_a.shape[1] * 2
     o16 = np.zeros((m, n), dtype=np.uint16)
     o32 = np.zeros((m, n), dtype=np.float32)
-    lib().fos_oracle_gemm_nvfp4(
-        _ptr(np.ascontiguousarray(values_a)), _ptr(np.ascontiguousarray(values_b)),
-        _ptr(np.ascontiguousarray(sf_rows_a)), _ptr(np.ascontiguousarray(sf_rows_b)),
-        float(alpha), m, n, k, _ptr(o16), _ptr(o32), threads or default_threads())
+    # (named, so that the copies made for strided arguments live until the call returns)
+    va, vb = np.ascontiguousarray(values_a), np.ascontiguousarray(values_b)
+    sa, sb = np.ascontiguousarray(sf_rows_a), np.ascontiguousarray(sf_rows_b)
+    lib().fos_oracle_gemm_nvfp4(_ptr(va), _ptr(vb), _ptr(sa), _ptr(sb),
+                                float(alpha), m, n, k, _ptr(o16), _ptr(o32), threads or default_threads())
     return o16, o32
 
 
