@@ -205,7 +205,7 @@ def extras(dev, steps: int) -> dict:
     del xs
     mse = fos.QuantizationConfig(scale_rule="mse")
     for m, nn, k in ((16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336), (128, 4096, 4096), (128, 14336, 4096),
-                     (128, 4096, 14336), (2048, 14336, 4096)):
+                     (128, 4096, 14336), (2048, 14336, 4096), (2048, 4096, 4096), (2048, 4096, 14336)):
         qa = fos.quantize(make_activation(m, k, 7).to(dev), mse)
         qb = fos.quantize(make_activation(nn, k, 8).to(dev), mse)
         out[f"gemm_nvfp4_{m}x{nn}x{k}_us"] = us(lambda: fos.quantized_matmul(qa, qb))
