@@ -15,12 +15,19 @@
 // of the MFMAs.  Only A goes through LDS: with both operands there, LDS traffic (fragment
 // reads plus staging writes) took as many cycles per K step as the MFMAs themselves -- a build
 // without the B fragment reads ran 13 % faster -- so each wavefront loads the packed rows of its
-// own B columns (two wavefronts share them: the second finds them in the vector cache) and
-// turns them into MFMA operands in registers.  Within a K step the contraction index is
-// permuted the same way for both operands: the 16-wide slice kk of lane half h covers
-// k = 32 h + 8 kk ... + 7, so that a lane's B codes are 16 contiguous bytes.  The big tile (256 x 256, 8
-// wavefronts of 128 x 64) keeps LDS reads at ~75 % of their bandwidth; a 128 x 128 tile
-// serves shapes that are not multiples of 256 or too small to fill the chip otherwise.
+// own B columns and turns them into MFMA operands in registers.  Within a K step the
+// contraction index is permuted the same way for both operands: the 16-wide slice kk of lane
+// half h covers k = 32 h + 8 kk ... + 7, so that a lane's B codes are 16 contiguous bytes.
+// The wavefronts of a workgroup sit side by side along N, each with all BM rows and 32
+// columns (256 x 256 tile: 8 wavefronts of 256 x 32; 128 x 128 tile: 4 of 128 x 32), so every
+// code of either operand is converted once per workgroup.  With two rows of wavefronts (128 x 64
+// and 64 x 64 per wavefront) the two wavefronts that share B columns both converted them: the
+// arrangement here reads twice the A fragments from LDS per MFMA and still measured faster,
+// 8192^3 811 -> 790 us, 4096^3 107.5 -> 105.0 us in alternating series on one box, and
+// 3072 x 4096 x 4096 131 -> 105 us, 1152 x 4096 x 4096 71 -> 56 us on the 128 x 128 tile (a
+// 256 x 128 tile of 8 wavefronts of 128 x 32 in two rows lost to it wherever 256 x 256 tiles
+// are too few to fill the chip), with bit-identical outputs.  The 128 x 128 tile serves
+// shapes that are not multiples of 256 or too small to fill the chip otherwise.
 // Workgroups are numbered so that the tiles resident on one XCD (blockIdx % 8) form a
 // compact block of the output, which keeps their A/B panels in that XCD's L2.
 #include <hip/hip_runtime.h>
@@ -1017,7 +1024,7 @@ static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
 
 // Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
 // caller's workspace for splits * M * N FP32 partials).
-enum { kPlanBig, kPlanMid, kPlanSmall, kPlanSkinny };
+enum { kPlanBig, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
@@ -1027,7 +1034,7 @@ constexpr int kTargetWorkgroups = 256;
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
     g.narrow = g.wide = 0;
-    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 256 = 256 x 128 tile wherever M allows, 1 = no weight-streaming kernel
+    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 256 = 256 x 256 tile wherever M and N allow, 1 = no weight-streaming kernel
     int64_t steps, tiles;
     if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32 || tile == 64)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
@@ -1048,22 +1055,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
             g.wide = 1;
             tiles = (N / 64) * (M > 64 ? 2 : 1);
         }
-    } else if ((M % 256 == 0) && (N % 256 == 0) && (M / 256) * (N / 256) >= 256 && tile != 128) {
+    } else if ((M % 256 == 0) && (N % 256 == 0) && ((M / 256) * (N / 256) >= 256 || tile == 256) && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
         g.kind = kPlanBig;
-        g.splits = 1;
-        g.ksteps_per_split = (int)(K / BK);
-        return g;
-    } else if ((M % 256 == 0) && tile != 128 &&
-               (tile == 256 || ((M / 256) * (N / 128) > 128 && (M / 256) * (N / 128) <= 256) || (M / 256) * (N / 128) > 384)) {
-        // 256 x 128 tiles, one workgroup of eight wavefronts per compute unit, where the 256 x 256
-        // ones would leave compute units idle: B is converted by two wavefronts instead of by
-        // two per 128 rows.  Measured against the 128 x 128 tiles (two workgroups per compute
-        // unit) at K = 4096, by the number T of 256 x 128 tiles: T = 128 57 against 47 us; 192: 65
-        // against 77; 256: 75 against 89; 384: 132-135 against 130; 448: 139 against 159; 896: 224
-        // against 284 -- so not where they cover half of the compute units or one and a half
-        // times all of them.
-        g.kind = kPlanMid;
         g.splits = 1;
         g.ksteps_per_split = (int)(K / BK);
         return g;
@@ -1152,8 +1146,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     p.splits = g.splits;
     p.ksteps_per_split = g.ksteps_per_split;
     switch (g.kind) {
-        case kPlanBig: return launch_gemm<2, 4, 4, 2>(p, out_type, s);
-        case kPlanMid: return launch_gemm<2, 4, 4, 1>(p, out_type, s);
+        case kPlanBig: return launch_gemm<1, 8, 8, 1>(p, out_type, s);
         case kPlanSkinny:
             // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);
@@ -1166,7 +1159,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
             if (M <= 32) return launch_skinny<1, 1>(p, out_type, s);
             if (M <= 64) return g.wide ? launch_skinny<2, 2>(p, out_type, s) : launch_skinny<2, 1>(p, out_type, s);
             return g.wide ? launch_skinny<2, 2>(p, out_type, s, 2) : launch_skinny<4, 1>(p, out_type, s);
-        default: return launch_gemm<2, 2, 2, 2>(p, out_type, s);
+        default: return launch_gemm<1, 4, 4, 1>(p, out_type, s);
     }
 }
 

@@ -166,11 +166,11 @@ def test_gemm_split_k_matches_unsplit(monkeypatch, m, n, k, env):
     close(unsplit, run(None, rows=qa.values.shape[0])[:m])
 
 
-@pytest.mark.parametrize(("m", "n", "k"), [(512, 384, 1088), (256, 128, 64), (768, 1024, 4160)])
+@pytest.mark.parametrize(("m", "n", "k"), [(512, 256, 1088), (256, 256, 64), (768, 1024, 4160)])
 def test_gemm_tile_kernels_agree_bitwise(monkeypatch, oracle, m, n, k):
-    """The 256 x 128 tile (the planner's choice where 256 x 256 tiles would leave compute
-    units idle; forced here) contracts K in the same order as the 128 x 128 tile: whole
-    outputs are bit-identical, bf16 and fp16, and a sample matches the oracle."""
+    """The 256 x 256 tile (the planner's choice from 256 such tiles on; forced here) and
+    the 128 x 128 tile contract K in the same order: whole outputs are bit-identical,
+    bf16 and fp16, and a sample matches the oracle."""
     from fouroversix_amd import _native as nat
 
     L = nat.lib()
@@ -197,7 +197,7 @@ def test_gemm_tile_kernels_agree_bitwise(monkeypatch, oracle, m, n, k):
     sa = oracle.from_blocked(u8(qa.scale_factors).reshape(-1), va.shape[0], k // 16)
     sb = oracle.from_blocked(u8(qb.scale_factors).reshape(-1), vb.shape[0], k // 16)
     ref, _ = oracle.gemm_nvfp4(va[:m:3], sa[:m:3], vb[:n], sb[:n], float(alpha))
-    check(bits16(out[::3]), ref, oracle, f"256x128 tiles, {m}x{n}x{k}")
+    check(bits16(out[::3]), ref, oracle, f"256x256 tiles, {m}x{n}x{k}")
 
 
 def test_linear_layer_forward(oracle):
