@@ -60,12 +60,20 @@ FOS_DEVICE float div_const(float x, float y, float r) {
     return __builtin_fmaf(__builtin_fmaf(-y, q0, x), r, q0);
 }
 
+// a * b + c on 24-bit unsigned a, b in one instruction (the compiler turns a multiplication by a
+// one-bit value into a sign-extending bit-field extract, an AND and an addition: three)
+FOS_DEVICE uint32_t mad_u24(uint32_t a, uint32_t b, uint32_t c) {
+    uint32_t d;
+    asm("v_mad_u32_u24 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
 // deq - x for one decoded candidate value fq (on the E2M1 grid).
 FOS_DEVICE float candidate_residual(float fq, const FastLutEntry &e, float x) {
     const uint32_t fb = f2u(fq);
     const float p2 = u2f(fb & 0xffbfffffu);                    // 1.5 * 2^j -> 2^j
     const uint32_t three = (fb >> 22) & 1u;                    // fq in {1.5, 3, 6}
-    const float mult = u2f(__umul24(three, e.delta) + f2u(e.d1));
+    const float mult = u2f(mad_u24(three, e.delta, f2u(e.d1)));
     return __builtin_fmaf(p2, mult, -x);
 }
 
@@ -420,8 +428,8 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     pickB = cmp > 0;
                 }
                 if (!certain) {
-                    bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
-                    if (TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
+                    bool tie = SHORTCUT && e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
+                    if (SHORTCUT && TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                     if (tie) pickB = false;
                     else if (k.exact_ok) {
                         if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
@@ -471,9 +479,10 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 pickB = cmp > 0;
             }
             if (!certain) {
-                // exact ties by construction first (cheap), the full evaluation otherwise
-                bool tie = e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
-                if (TWO_D) {
+                // exact ties by construction first (cheap), the full evaluation otherwise (a rule
+                // without a shortcut evaluates every block exactly, ties included: no pre-check)
+                bool tie = SHORTCUT && e4m3_decode(s4) == 1.5f * e4m3_decode(s6) && (tie_violations(a0, b0) | tie_violations(a1, b1)) == 0;
+                if (SHORTCUT && TWO_D) {
                     // every row of the tile must agree
                     tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                 }
@@ -604,7 +613,7 @@ FOS_DEVICE void dequant_block_bf16_lut(const BlockOut &o, const FastLutEntry &e,
             const uint32_t fb = f2u(v[h]);
             const float p2 = u2f(fb & 0xffbfffffu);  // 1.5 * 2^j -> 2^j (sign and zero kept)
             const uint32_t three = (fb >> 22) & 1u;
-            q[h] = p2 * u2f(__umul24(three, e.delta) + f2u(e.d1));
+            q[h] = p2 * u2f(mad_u24(three, e.delta, f2u(e.d1)));
         }
         w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_t));
     });
