@@ -25,88 +25,111 @@ struct DequantParams {
 
 // One thread per 8 consecutive elements, i.e. half a 1x16 block (consecutive threads =
 // consecutive octets of a row: a wavefront reads 256 contiguous bytes of codes and writes
-// 1 KiB per store instruction).  `p.fast_div`: the divisor is one of the constants for which
-// the 3-operation division is exact; it is used when amax is far enough from the ends of
-// the float range for every quotient to be normal or zero.
+// 1 KiB per store instruction); blockIdx.y walks the rows.  `p.fast_div`: the divisor is one
+// of the constants for which the 3-operation division is exact; it is used when amax is far
+// enough from the ends of the float range for every quotient to be normal or zero.
+// When, besides, amax has at most 8 significant bits (the maximum of a bf16 tensor), value *
+// scale * amax is exact and its quotient is (power of two) x RN(g / c) or x RN(1.5 g / c) with
+// g = scale * amax (see dequant_block_bf16_lut): the two quotients are formed once per thread
+// and an element costs four operations instead of eight.
 template <int DT, int OUT>
 __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) {
     const int64_t sf_cols = p.cols_p >> 4;
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t opr = (p.cols + 7) >> 3;  // octets per row
-    if (idx >= p.rows * opr) return;
-    const int64_t r = idx / opr, oc = idx - r * opr, cb = oc >> 1;
-    const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
-    const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
-                             ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
-                             : r * sf_cols + cb;
-    const uint32_t sb = p.sf[sofs];
+    const int64_t oc = (int64_t)blockIdx.x * 256 + threadIdx.x, cb = oc >> 1;
+    if (oc >= opr) return;
     const float amax = *p.amax;
-    const float sf = e4m3_decode(sb & 0x7fu);
+    const bool fast = p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f;
+    const bool table = fast && (f2u(amax) & 0xffffu) == 0;
+    const float rc = 1.0f / p.divisor;
+    for (int64_t r = blockIdx.y; r < p.rows; r += gridDim.y) {
+        const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
+        const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
+                                 ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
+                                 : r * sf_cols + cb;
+        const uint32_t sb = p.sf[sofs];
+        const float sf = e4m3_decode(sb & 0x7fu);
 
-    // value * scale, as the fp16 product of the reference (exact for E2M1 values)
-    float f[8];
-    if (DT == FOS_DTYPE_IF4 && (sb & 0x80u)) {
-        const _Float16 s16 = (_Float16)sf;
-        const float six_sevenths = (float)(6.0 / 7.0);
+        float f[8];
+        const bool int_block = DT == FOS_DTYPE_IF4 && (sb & 0x80u);
+        if (table && !int_block && (sb & 0x7fu) != 0x7fu) {
+            const float g = sf * amax;  // exact: 4 + 8 significant bits
+            const float d1 = div_const(g, p.divisor, rc), d15 = div_const(1.5f * g, p.divisor, rc);
+            const uint32_t delta = f2u(d15) - f2u(d1);
+            static_for<0, 4>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                const float2_t v = unpack_fp4<j>(q);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t code = (q >> (4 * i)) & 0xfu;
-            const int iv = ((int)(code << 28)) >> 28;
-            f[i] = p.f32_product ? ((float)iv * six_sevenths) * sf : (float)((_Float16)((float)iv * six_sevenths) * s16);
+                for (int h = 0; h < 2; ++h) {
+                    const uint32_t fb = f2u(v[h]);
+                    f[2 * j + h] = u2f(fb & 0xffbfffffu) * u2f(mad_u24((fb >> 22) & 1u, delta, f2u(d1)));
+                }
+            });
+        } else {
+            // value * scale, as the fp16 product of the reference (exact for E2M1 values)
+            if (int_block) {
+                const _Float16 s16 = (_Float16)sf;
+                const float six_sevenths = (float)(6.0 / 7.0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t code = (q >> (4 * i)) & 0xfu;
+                    const int iv = ((int)(code << 28)) >> 28;
+                    f[i] = p.f32_product ? ((float)iv * six_sevenths) * sf : (float)((_Float16)((float)iv * six_sevenths) * s16);
+                }
+            } else {
+                static_for<0, 4>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const float2_t v = unpack_fp4<j>(q);
+                    f[2 * j] = v.x * sf;
+                    f[2 * j + 1] = v.y * sf;
+                });
+            }
+            if (fast) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float t = f[i] * amax;
+                    f[i] = u2f((f2u(div_const(t, p.divisor, rc)) & 0x7fffffffu) | (f2u(t) & 0x80000000u));
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = (f[i] * amax) / p.divisor;
+            }
         }
-    } else {
-        static_for<0, 4>([&](auto jc) {
-            constexpr int j = decltype(jc)::value;
-            const float2_t v = unpack_fp4<j>(q);
-            f[2 * j] = v.x * sf;
-            f[2 * j + 1] = v.y * sf;
-        });
-    }
-    if (p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f) {
-        const float rc = 1.0f / p.divisor;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float t = f[i] * amax;
-            f[i] = u2f((f2u(div_const(t, p.divisor, rc)) & 0x7fffffffu) | (f2u(t) & 0x80000000u));
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] = (f[i] * amax) / p.divisor;
-    }
 
-    const int64_t c0 = oc * 8;
-    const bool whole = p.vector_stores && c0 + 8 <= p.cols;
-    if (OUT == FOS_T_F32) {
-        float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
+        const int64_t c0 = oc * 8;
+        const bool whole = p.vector_stores && c0 + 8 <= p.cols;
+        if (OUT == FOS_T_F32) {
+            float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
+            if (whole) {
+                reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
+                reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (c0 + i < p.cols) o[i] = f[i];
+            }
+            continue;
+        }
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float2_t v = {f[2 * j], f[2 * j + 1]};
+            if (OUT == FOS_T_F16) {
+                typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+                w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2_t));
+            } else {
+                typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+            }
+        }
+        uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
         if (whole) {
-            reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
-            reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
+            stream_store(reinterpret_cast<uint4 *>(o), make_uint4(w[0], w[1], w[2], w[3]));
         } else {
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (c0 + i < p.cols) o[i] = f[i];
+                if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
         }
-        return;
-    }
-    uint32_t w[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float2_t v = {f[2 * j], f[2 * j + 1]};
-        if (OUT == FOS_T_F16) {
-            typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2_t));
-        } else {
-            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-            w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-        }
-    }
-    uint16_t *o = reinterpret_cast<uint16_t *>(p.out) + r * p.ldo + c0;
-    if (whole) {
-        stream_store(reinterpret_cast<uint4 *>(o), make_uint4(w[0], w[1], w[2], w[3]));
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (c0 + i < p.cols) o[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
     }
 }
 
@@ -160,9 +183,9 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.fast_div = p.divisor == 1536.0f || p.divisor == 1792.0f || p.divisor == 2688.0f;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
-    const int64_t n_octets = rows * ((cols + 7) / 8);
-    if ((n_octets + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
-    dim3 grid((unsigned)((n_octets + 255) / 256));
+    const int64_t opr = (cols + 7) / 8;
+    if ((opr + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    dim3 grid((unsigned)((opr + 255) / 256), (unsigned)(rows < 65535 ? rows : 65535));
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FOS_DTYPE_IF4) launch_dequant<FOS_DTYPE_IF4>(p, out_type, grid, s);
     else launch_dequant<FOS_DTYPE_NVFP4>(p, out_type, grid, s);
