@@ -350,6 +350,15 @@ extern "C" int fos_amax(const void *x, int x_type, int64_t rows, int64_t cols, i
 // L2, so it stops paying early: per call inside a HIP graph, one launch against two, 1 x 4096
 // 5.0 against 6.5 us, 16 x 1024 6.2 against 6.9, 16 x 2048 7.35 against 7.3, 16 x 4096 10.1 against 7.3.
 constexpr int64_t kFusedAmaxElements = 16384;
+// Outside a stream capture the host is the slower side at these sizes (a launch costs it about
+// 3 us; through the Python frontend 16 x 4096 takes 16 us per call in one launch and 19 in two,
+// more than either form on the GPU), so eager calls keep the single launch up to 128 KiB.
+constexpr int64_t kFusedAmaxElementsEager = 65536;
+
+static bool stream_is_capturing(hipStream_t s) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(s, &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+}
 
 // Shared body of fos_quantize and fos_pseudo_quantize (pseudo_out != null: bf16 round trip
 // instead of codes / scales).
@@ -422,7 +431,8 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         p.partials = (const uint32_t *)amax;
         p.n_partials = 0;
         p.amax_out = nullptr;
-    } else if (aligned && x_type == FOS_T_BF16 && ld == cols && rows * cols <= kFusedAmaxElements) {
+    } else if (aligned && x_type == FOS_T_BF16 && ld == cols &&
+               (rows * cols <= kFusedAmaxElements || (rows * cols <= kFusedAmaxElementsEager && !stream_is_capturing(s)))) {
         // decode-sized input: one launch, every workgroup of pass 2 finds the maximum itself
         p.partials = partials;
         p.n_partials = -1;
