@@ -21,6 +21,7 @@ struct DequantParams {
     int fast_div;       // divisor is 1536, 1792 or 2688 (exact 3-operation division)
     int vector_stores;  // out and ldo allow 16-byte stores of whole blocks
     int f32_product;    // value * scale formed in fp32 instead of fp16 (differs for IF4's integer blocks)
+    int wave_lines;     // fp32 output: whole wavefronts inside a row (cols % 512 == 0) and 16-byte stores allowed
 };
 
 // One thread per 8 consecutive elements, i.e. half a 1x16 block (consecutive threads =
@@ -42,6 +43,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
     const bool fast = p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f;
     const bool table = fast && (f2u(amax) & 0xffffu) == 0;
     const float rc = 1.0f / p.divisor;
+    __shared__ float4 swap[OUT == FOS_T_F32 ? 4 : 1][OUT == FOS_T_F32 ? 128 : 1];
     for (int64_t r = blockIdx.y; r < p.rows; r += gridDim.y) {
         const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
         const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
@@ -100,7 +102,24 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
         const bool whole = p.vector_stores && c0 + 8 <= p.cols;
         if (OUT == FOS_T_F32) {
             float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
-            if (whole) {
+            if (p.wave_lines) {
+                // a lane's 32 bytes as two stores 16 bytes apart would leave every instruction
+                // writing half of each line it touches: the wavefront turns its 2 KiB round in LDS
+                // and stores two contiguous KiB
+                const int lane = threadIdx.x & 63;
+                float4 *mine = swap[threadIdx.x >> 6];
+                mine[2 * lane] = make_float4(f[0], f[1], f[2], f[3]);
+                mine[2 * lane + 1] = make_float4(f[4], f[5], f[6], f[7]);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                const float4 lo = mine[lane], hi = mine[64 + lane];
+                uint4 *ow = reinterpret_cast<uint4 *>(o - 8 * lane);  // the wavefront's first element
+                stream_store(ow + lane, __builtin_bit_cast(uint4, lo));
+                stream_store(ow + 64 + lane, __builtin_bit_cast(uint4, hi));
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+            } else if (whole) {
                 reinterpret_cast<float4 *>(o)[0] = make_float4(f[0], f[1], f[2], f[3]);
                 reinterpret_cast<float4 *>(o)[1] = make_float4(f[4], f[5], f[6], f[7]);
             } else {
@@ -183,6 +202,7 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.fast_div = p.divisor == 1536.0f || p.divisor == 1792.0f || p.divisor == 2688.0f;
     const int64_t esize = out_type == FOS_T_F32 ? 4 : 2;
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
+    p.wave_lines = out_type == FOS_T_F32 && p.vector_stores && cols % 512 == 0;
     const int64_t opr = (cols + 7) / 8;
     if ((opr + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
     dim3 grid((unsigned)((opr + 255) / 256), (unsigned)(rows < 65535 ? rows : 65535));

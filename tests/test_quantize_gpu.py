@@ -564,14 +564,17 @@ def test_activation_style_stochastic_seeds(oracle, rule):
 
 @pytest.mark.parametrize(("dtype", "rule"), [("nvfp4", "mse"), ("nvfp4", "static_4"), ("if4", "mse")])
 @pytest.mark.parametrize("out", [torch.bfloat16, torch.float16, torch.float32])
-def test_dequantize_bit_exact(oracle, dtype, rule, out):
-    x = make_input("tiny_blocks", (200, 144), 9)
+@pytest.mark.parametrize(("kind", "shape"), [("tiny_blocks", (200, 144)),
+                                             ("randn", (300, 1024)),  # whole wavefronts per row: fp32 output as whole lines
+                                             ("randn", (3, 2560))])
+def test_dequantize_bit_exact(oracle, dtype, rule, out, kind, shape):
+    x = make_input(kind, shape, 9)
     q = hip_quantize(x, dtype=dtype, scale_rule=rule)
     ref = oracle.quantize(x, dtype=dtype, scale_rule=rule)
     expect = torch.from_numpy(oracle.dequantize(ref.values, ref.scale_rows, ref.amax, dtype=dtype, scale_rule=rule,
-                                                original_shape=(200, 144)).copy()).to(out)
+                                                original_shape=shape).copy()).to(out)
     got = fos.dequantize(q, out).cpu()
-    assert got.shape == (200, 144) and got.dtype == out
+    assert got.shape == shape and got.dtype == out
     assert torch.equal(got.view(torch.int16 if out != torch.float32 else torch.int32),
                        expect.view(torch.int16 if out != torch.float32 else torch.int32))
 
