@@ -36,20 +36,24 @@ struct DequantParams {
 template <int DT, int OUT>
 __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) {
     const int64_t sf_cols = p.cols_p >> 4;
-    const int64_t opr = (p.cols + 7) >> 3;  // octets per row
-    const int64_t oc = (int64_t)blockIdx.x * 256 + threadIdx.x, cb = oc >> 1;
+    const uint32_t opr = (uint32_t)((p.cols + 7) >> 3);  // octets per row
+    // (32-bit column quantities: the row parts of every address are wavefront-uniform and stay on
+    // the scalar unit, a thread adds a 32-bit offset)
+    const uint32_t oc = blockIdx.x * 256u + threadIdx.x, cb = oc >> 1;
     if (oc >= opr) return;
+    const uint32_t sf_col_off = p.sf_layout == FOS_SF_TILED_128X4 ? (cb >> 2) * 512u + (cb & 3u) : cb;
     const float amax = *p.amax;
     const bool fast = p.fast_div && amax >= 0x1p-100f && amax <= 0x1p100f;
     const bool table = fast && (f2u(amax) & 0xffffu) == 0;
     const float rc = 1.0f / p.divisor;
     __shared__ float4 swap[OUT == FOS_T_F32 ? 4 : 1][OUT == FOS_T_F32 ? 128 : 1];
     for (int64_t r = blockIdx.y; r < p.rows; r += gridDim.y) {
-        const uint32_t q = *reinterpret_cast<const uint32_t *>(p.codes + r * (p.cols_p >> 1) + oc * 4);
-        const int64_t sofs = p.sf_layout == FOS_SF_TILED_128X4
-                                 ? ((r >> 7) * (sf_cols >> 2) + (cb >> 2)) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + (cb & 3)
-                                 : r * sf_cols + cb;
-        const uint32_t sb = p.sf[sofs];
+        const uint8_t *row_codes = p.codes + r * (p.cols_p >> 1);
+        const uint8_t *row_sf = p.sf + (p.sf_layout == FOS_SF_TILED_128X4
+                                            ? (r >> 7) * (sf_cols >> 2) * 512 + (r & 31) * 16 + ((r & 127) >> 5) * 4
+                                            : r * sf_cols);
+        const uint32_t q = *reinterpret_cast<const uint32_t *>(row_codes + oc * 4u);
+        const uint32_t sb = row_sf[sf_col_off];
         const float sf = e4m3_decode(sb & 0x7fu);
 
         float f[8];
@@ -98,7 +102,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const DequantParams p) 
             }
         }
 
-        const int64_t c0 = oc * 8;
+        const uint32_t c0 = oc * 8u;
         const bool whole = p.vector_stores && c0 + 8 <= p.cols;
         if (OUT == FOS_T_F32) {
             float *o = reinterpret_cast<float *>(p.out) + r * p.ldo + c0;
@@ -204,7 +208,7 @@ extern "C" int fos_dequantize(const uint8_t *codes, const uint8_t *sf, const flo
     p.vector_stores = ((uintptr_t)out & 15) == 0 && (ldo * esize) % 16 == 0;
     p.wave_lines = out_type == FOS_T_F32 && p.vector_stores && cols % 512 == 0;
     const int64_t opr = (cols + 7) / 8;
-    if ((opr + 255) / 256 > 0x7fffffffLL) return FOS_E_BAD_SHAPE;
+    if (cols_p > 0x7fffffffLL) return FOS_E_BAD_SHAPE;  // 32-bit column offsets in the kernel
     dim3 grid((unsigned)((opr + 255) / 256), (unsigned)(rows < 65535 ? rows : 65535));
     hipStream_t s = (hipStream_t)stream;
     if (dtype == FOS_DTYPE_IF4) launch_dequant<FOS_DTYPE_IF4>(p, out_type, grid, s);
