@@ -357,7 +357,11 @@ constexpr int64_t kFusedAmaxElementsEager = 65536;
 
 static bool stream_is_capturing(hipStream_t s) {
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    return hipStreamIsCapturing(s, &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &status) != hipSuccess) {
+        (void)hipGetLastError();  // the query's own failure must not read as a failed launch later
+        return true;
+    }
+    return status != hipStreamCaptureStatusNone;
 }
 
 // Shared body of fos_quantize and fos_pseudo_quantize (pseudo_out != null: bf16 round trip
