@@ -401,6 +401,36 @@ def test_two_pass_quantize_replays_in_a_hip_graph():
         assert float(static_q.amax) == float(eager.amax), f"replay {i}"
 
 
+@pytest.mark.parametrize("shape", [(16, 4096), (4, 4096), (16, 1024), (1, 8192), (16, 4064)])
+def test_decode_sized_quantize_eager_and_captured(oracle, shape):
+    """Decode-sized inputs take one launch (every workgroup scans the tensor for its maximum) up to
+    32 KiB, and up to 128 KiB when the call is not being captured; above, two launches.  Eager
+    and captured calls of the same input -- which differ in form between those limits -- give the
+    same bytes, those of the oracle, on every replay."""
+    cfg = fos.QuantizationConfig(scale_rule="mse")
+    static_x = make_input("randn", shape, 70).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fos.quantize(static_x, cfg)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_q = fos.quantize(static_x, cfg)
+    for i in range(3):
+        xi = make_input("randn", shape, 71 + i) * float(2 * i + 1)
+        static_x.copy_(xi.cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = fos.quantize(xi.cuda(), cfg)
+        ref = oracle.quantize(xi, scale_rule="mse")
+        for q in (static_q, eager):
+            assert np.array_equal(u8(q.values), ref.values), f"replay {i}"
+            assert np.array_equal(u8(q.scale_factors), ref.scale_factors), f"replay {i}"
+            assert float(q.amax) == float(ref.amax), f"replay {i}"
+
+
 @pytest.mark.parametrize("cfg", [dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=True), dict(dtype="mxfp4", scale_rule="static_6")],
                          ids=["nvfp4-mse-1d", "nvfp4-static6-2d", "mxfp4"])
 def test_tensors_beyond_four_gib(cfg):
