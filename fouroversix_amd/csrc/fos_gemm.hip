@@ -27,7 +27,9 @@
 // 3072 x 4096 x 4096 131 -> 105 us, 1152 x 4096 x 4096 71 -> 56 us on the 128 x 128 tile (a
 // 256 x 128 tile of 8 wavefronts of 128 x 32 in two rows lost to it wherever 256 x 256 tiles
 // are too few to fill the chip), with bit-identical outputs.  The 128 x 128 tile serves
-// shapes that are not multiples of 256 or too small to fill the chip otherwise.
+// shapes that are not multiples of 256 or too small to fill the chip otherwise, and a 128 x 256
+// tile (the template with BM = 128 and eight wavefronts: half of the threads stage A) those
+// that it covers with one workgroup per compute unit.
 // Workgroups are numbered so that the tiles resident on one XCD (blockIdx % 8) form a
 // compact block of the output, which keeps their A/B panels in that XCD's L2.
 #include <hip/hip_runtime.h>
@@ -156,7 +158,8 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     constexpr bool OUT_BF16 = OUT == kOutBF16;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
-    static_assert(BM == kThreadsG / 2, "one thread per half row of A");
+    static_assert(2 * BM <= kThreadsG, "one thread per half row of A (wavefronts beyond the first 2 * BM threads stage nothing)");
+    constexpr bool kAllStage = 2 * BM == kThreadsG;
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
     _Float16 *lds_a[2] = {lds, lds + BM * kPitch};
 
@@ -171,6 +174,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     // buffer loads (wave-uniform base + per-thread 32-bit offset + scalar K offset), which
     // keeps 64-bit address arithmetic out of the loop
     const int ld_row = tid >> 1, ld_half = tid & 1;
+    const bool stager = __builtin_amdgcn_readfirstlane(tid) < 2 * BM;  // wavefront-uniform
     const BufferRsrc ra = make_rsrc(p.A + m0 * kbytes, (uint32_t)(BM * kbytes));
     const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(BN * kbytes));
     const BufferRsrc rsa = make_rsrc(p.sfA + (m0 >> 7) * sf_groups * 512, (uint32_t)((BM >> 7) * sf_groups * 512));
@@ -196,8 +200,10 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     typedef Staged<WN> StagedT;
     auto fetch = [&](int64_t ks, StagedT &s) {
         const uint32_t kq = (uint32_t)(ks0 + ks) * 32u, ksf = (uint32_t)(ks0 + ks) * 512u;
-        s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
-        s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
+        if (kAllStage || stager) {
+            s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
+            s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
+        }
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
             s.qb[j] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)qb_off[j], (int)kq, 0));
@@ -206,6 +212,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     };
     // quarter q (0..3) of the staged A data -> 8 halfs in LDS buffer `buf`
     auto stage_quarter = [&](const StagedT &s, int buf, int q) {
+        if (!kAllStage && !stager) return;
         const uint32_t wa = q == 0 ? s.qa.x : q == 1 ? s.qa.y : q == 2 ? s.qa.z : s.qa.w;
         // this thread's two block scales: bytes 2*ld_half, 2*ld_half + 1
         const half2_t sa2 = e4m3x2_to_half2(s.sa >> (16 * ld_half));
@@ -1034,7 +1041,7 @@ static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
 
 // Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
 // caller's workspace for splits * M * N FP32 partials).
-enum { kPlanBig, kPlanSmall, kPlanSkinny };
+enum { kPlanBig, kPlanWide, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
@@ -1044,7 +1051,7 @@ constexpr int kTargetWorkgroups = 256;
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     GemmPlan g;
     g.narrow = g.wide = 0;
-    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 256 = 256 x 256 tile wherever M and N allow, 1 = no weight-streaming kernel
+    const int tile = tuning().gemm_tile;  // tuning / tests: 128 = small tile, 129 = 128 x 256 tile and 256 = 256 x 256 tile wherever M and N allow, 1 = no weight-streaming kernel
     int64_t steps, tiles;
     if (M <= 128 && K % 256 == 0 && (tile == 0 || tile == 16 || tile == 32 || tile == 64)) {
         // one 128-row band: weight streaming, steps of 256 along K shared by 8 wavefronts
@@ -1068,6 +1075,18 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
     } else if ((M % 256 == 0) && (N % 256 == 0) && ((M / 256) * (N / 256) >= 256 || tile == 256) && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
         g.kind = kPlanBig;
+        g.splits = 1;
+        g.ksteps_per_split = (int)(K / BK);
+        return g;
+    } else if (tile != 128 && M % 128 == 0 && N % 256 == 0 && M >= 128 &&
+               (tile == 129 || ((M / 128) * (N / 256) > 128 && (M / 128) * (N / 256) <= 256))) {
+        // 128 x 256 tiles (eight wavefronts of 128 x 32; the first four stage A) where they give
+        // every compute unit at most one workgroup and more than half of them one: A is converted
+        // once per 256 columns instead of once per 128.  Against the 128 x 128 tile, alternating
+        // runs: 2048 x 4096 x 4096 71.9 -> 69.3 us, 2048 x 4096 x 14336 242.5 -> 228 us,
+        // 1792 x 4096 x 4096 67.0 -> 64.6 us; with 1.5 workgroups per compute unit
+        // (3072 x 4096 x 4096) 109 -> 123 us, with half a one (1024 x 4096 x 4096) 41.7 -> 51.8 us.
+        g.kind = kPlanWide;
         g.splits = 1;
         g.ksteps_per_split = (int)(K / BK);
         return g;
@@ -1157,6 +1176,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     p.ksteps_per_split = g.ksteps_per_split;
     switch (g.kind) {
         case kPlanBig: return launch_gemm<1, 8, 8, 1>(p, out_type, s);
+        case kPlanWide: return launch_gemm<1, 8, 4, 1>(p, out_type, s);
         case kPlanSkinny:
             // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);

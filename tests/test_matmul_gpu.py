@@ -168,9 +168,10 @@ def test_gemm_split_k_matches_unsplit(monkeypatch, m, n, k, env):
 
 @pytest.mark.parametrize(("m", "n", "k"), [(512, 256, 1088), (256, 256, 64), (768, 1024, 4160)])
 def test_gemm_tile_kernels_agree_bitwise(monkeypatch, oracle, m, n, k):
-    """The 256 x 256 tile (the planner's choice from 256 such tiles on; forced here) and
-    the 128 x 128 tile contract K in the same order: whole outputs are bit-identical,
-    bf16 and fp16, and a sample matches the oracle."""
+    """The 256 x 256 tile (the planner's choice from 256 such tiles on; forced here), the
+    128 x 256 tile (its choice where that covers the chip once; forced here) and the
+    128 x 128 tile contract K in the same order: whole outputs are bit-identical, bf16 and
+    fp16, and a sample matches the oracle."""
     from fouroversix_amd import _native as nat
 
     L = nat.lib()
@@ -192,6 +193,7 @@ def test_gemm_tile_kernels_agree_bitwise(monkeypatch, oracle, m, n, k):
 
     for out_dtype in (torch.bfloat16, torch.float16):
         assert torch.equal(run("256", out_dtype), run("128", out_dtype))
+        assert torch.equal(run("129", out_dtype), run("128", out_dtype))  # 128 x 256 tiles
     out = run("256", torch.bfloat16)
     va, vb = u8(qa.values), u8(qb.values)
     sa = oracle.from_blocked(u8(qa.scale_factors).reshape(-1), va.shape[0], k // 16)
