@@ -57,27 +57,63 @@ def event_ms(fn, steps):
 
 def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv=1024, ffn=14336):
     """Per layer: on-the-fly activation quantize (4/6-MSE, 1x16) + FP4 GEMM for q/k/v/o and
-    gate/up/down against weights pre-quantized 4/6-MSE with 16x16 blocks; each projection
-    re-quantizes its input, as the reference's linear layer does.  No attention, no
-    nonlinearity: the output of q feeds o, the output of gate feeds down."""
+    gate/up/down against weights pre-quantized 4/6-MSE with 16x16 blocks.  No attention, no
+    nonlinearity: the output of q feeds o, the output of o feeds gate / up, the output of gate
+    feeds down.  The headline figure is an nn.Module of nn.Linear layers converted with
+    ``quantize_model`` (every projection quantizes its own input, as the reference's linear layer
+    does; a GEMM output that goes straight into the next projection brings its maximum along);
+    beside it the same chain with ``emit_output_amax=False`` and as hand-written calls of
+    ``quantized_matmul`` on the same weights."""
     import torch
+    import torch.nn as nn
 
     import fouroversix_amd as fos
 
-    wcfg = fos.QuantizationConfig(scale_rule="mse", block_scale_2d=True)
     acfg = fos.QuantizationConfig(scale_rule="mse")
     shapes = [("q", hidden, hidden), ("k", kv, hidden), ("v", kv, hidden), ("o", hidden, hidden),
               ("gate", ffn, hidden), ("up", ffn, hidden), ("down", hidden, ffn)]
+
+    class Projections(nn.Module):
+        def __init__(self):
+            super().__init__()
+            for name, n, k in shapes:
+                setattr(self, name, nn.Linear(k, n, bias=False, device=dev, dtype=torch.bfloat16))
+
+        def forward(self, x):
+            q = self.q(x)
+            self.k(x)
+            self.v(x)
+            h = self.o(q)
+            gate = self.gate(h)
+            self.up(h)
+            return self.down(gate)
+
     g = torch.Generator(device=dev).manual_seed(7)
-    weights = []
-    for _ in range(layers):
-        layer = {}
-        for name, n, k in shapes:
-            w = (0.02 * torch.randn(n, k, generator=g, device=dev)).bfloat16()
-            layer[name] = fos.quantize(w, wcfg)
-            del w
-        weights.append(layer)
+    model = nn.Sequential(*[Projections() for _ in range(layers)])
+    with torch.no_grad():
+        for lin in model.modules():
+            if isinstance(lin, nn.Linear):
+                lin.weight.copy_((0.02 * torch.randn(lin.weight.shape, generator=g, device=dev)).bfloat16())
+    model_cfg = fos.ModelQuantizationConfig(weight_scale_2d=True, modules_to_not_convert=[])
+    fos.quantize_model(model, model_cfg)
+    for lin in model.modules():
+        if isinstance(lin, fos.FourOverSixLinear):
+            lin.quantize_weight_()
+    torch.cuda.empty_cache()
+    weights = [{name: getattr(layer, name).quantized_weight() for name, _, _ in shapes} for layer in model]
     x0 = torch.randn(tokens, hidden, generator=g, device=dev).bfloat16()
+
+    def step_module():
+        with torch.no_grad():
+            return model(x0)
+
+    def step_module_no_amax():
+        model_cfg.emit_output_amax = False
+        try:
+            with torch.no_grad():
+                return model(x0)
+        finally:
+            model_cfg.emit_output_amax = True
 
     def step():
         x = x0
@@ -129,18 +165,27 @@ def linear_stack(dev, steps, warmup, layers=32, tokens=8 * 2048, hidden=4096, kv
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
 
-    sec = timed(step)
+    assert model_cfg.emit_output_amax, "the module path hands the GEMM-recorded maximum on by default"
+    sec = timed(step_module)
+    sec_module_no_amax = timed(step_module_no_amax)
+    sec_raw = timed(step)
     sec_shared = timed(step_shared)
     sec_amax = timed(step_amax)
     flops = 2.0 * tokens * sum(n * k for _, n, k in shapes) * layers
+
+    def fig(s):
+        return {"ms_per_step": round(s * 1e3, 3), "tokens_per_s": round(tokens / s, 1)}
+
     return {
         "workload": f"{layers} layers x (q,k,v,o,gate,up,down) quantize+GEMM, {tokens} tokens, hidden {hidden}, "
-                    f"kv {kv}, ffn {ffn}",
+                    f"kv {kv}, ffn {ffn}; nn.Module converted with quantize_model (default config + weight_scale_2d)",
         "ms_per_step": round(sec * 1e3, 3),
         "tokens_per_s": round(tokens / sec, 1),
         "TFLOP/s": round(flops / sec / 1e12, 1),
-        "shared_activation_quantize": {"ms_per_step": round(sec_shared * 1e3, 3), "tokens_per_s": round(tokens / sec_shared, 1)},
-        "shared_and_gemm_recorded_amax": {"ms_per_step": round(sec_amax * 1e3, 3), "tokens_per_s": round(tokens / sec_amax, 1)},
+        "module_without_recorded_amax": fig(sec_module_no_amax),
+        "raw_calls": fig(sec_raw),
+        "shared_activation_quantize": fig(sec_shared),
+        "shared_and_gemm_recorded_amax": fig(sec_amax),
     }
 
 

@@ -156,7 +156,16 @@ struct QuantConsts {
     // significant bits, which every maximum of bf16 data has but a caller-supplied one need
     // not -- and the divisor 1536; without both, undecided blocks take the generic form.
     bool exact_ok = false;
+    // The certified shortcuts of the adaptive rules model the reference's error sums with relative
+    // rounding errors.  That holds while the reference's own fp32 arithmetic -- squares of residuals of
+    // the size of amax / 1536 times a block scale down to 2^-9, sums of up to 256 of them -- neither
+    // underflows nor overflows (a tensor of values around 2^-70 has all its squared errors flushed to
+    // zero or rounded as sub-normals there, and every block ties): tensor maxima in [2^-40, 2^40].
+    // Beyond, every block takes the exact evaluation.
+    bool shortcut_ok = false;
 };
+
+FOS_DEVICE bool shortcut_range(float amax) { return amax >= 0x1p-40f && amax <= 0x1p40f; }
 
 // v / k.errdiv with IEEE rounding (the sign of a zero quotient may differ; callers subtract).
 FOS_DEVICE float div_errdiv(float v, const QuantConsts &k) {

@@ -35,10 +35,19 @@ struct FastLutEntry {
     float inv;       // 1 / (dec * s)                       (0 for s == 0)
     float d1;        // RN((s * amax) / errdiv)             factor for fq in {.5, 1, 2, 4}
     uint32_t delta;  // bits((s * amax) / 1024) - bits(d1)  added for fq in {1.5, 3, 6}
-    float hh;        // d1 * d1: weight of this scale's sum of squares in the shortcut
+    float hh;        // weight of this scale's sum of squares in the shortcut: (d1 / 2^e)^2 with 2^e <= amax < 2^(e+1)
+                     // (d1^2 itself leaves fp32's normal range for tensors whose maximum is far from 1); the
+                     // product form of the MSE shortcut keeps d1 / 2^e here instead
 };
 
+// 2^-e for 2^e <= amax < 2^(e+1) (a normal amax)
+FOS_DEVICE float amax_norm(float amax) {
+    const uint32_t e = (f2u(amax) >> 23) & 0xffu;
+    return u2f((254u - (e < 1u ? 1u : (e > 253u ? 253u : e))) << 23);
+}
+
 // Entry for scale byte `s` (0..127); built with the reference's operations.
+template <bool PRODUCT_FORM = false>
 FOS_DEVICE FastLutEntry make_lut_entry(uint32_t s, const QuantConsts &k) {
     FastLutEntry e;
     const float sf = e4m3_decode(s);
@@ -46,7 +55,8 @@ FOS_DEVICE FastLutEntry make_lut_entry(uint32_t s, const QuantConsts &k) {
     const float g = sf * k.amax;
     e.d1 = g / k.errdiv;
     e.delta = f2u((1.5f * g) / k.errdiv) - f2u(e.d1);  // 1.5 g is exact; with errdiv = 1536 this is g / 1024
-    e.hh = e.d1 * e.d1;
+    const float hn = e.d1 * amax_norm(k.amax);
+    e.hh = PRODUCT_FORM ? hn : hn * hn;
     return e;
 }
 
@@ -150,6 +160,51 @@ FOS_DEVICE void accumulate_scaled(float r0, float r1, float &S) {
 template <int RULE>
 FOS_DEVICE float shortcut_weight(const FastLutEntry &e) {
     return RULE == FOS_RULE_MSE ? e.hh : e.d1;
+}
+
+// ---------------------------------------------------------------------------------------
+// 4/6-MSE shortcut in product form (bf16 elements, 1x16 blocks)
+// ---------------------------------------------------------------------------------------
+//
+// E_k = sum_i (h_k fq_i - x_i)^2 = h_k^2 F_k - 2 h_k G_k + sum_i x_i^2 with F_k = sum fq_i^2 and
+// G_k = sum fq_i x_i, and the last term is the same for both candidates:
+//     (E_4 - E_6) / 2 = h_4 q_4 - h_6 q_6,     q_k = (h_k / 2) F_k - G_k.
+// F_k and G_k come from v_dot2_f32_bf16 on the codes converted to bf16 pairs and the block's
+// packed elements AS LOADED (no unpacking, no scaled residuals): three instructions per element
+// pair and candidate where the residual form needs five.  Both sums are exact: a non-zero fq_i
+// needs a scaled magnitude above 1/4 and the block's largest is below 7, so the elements that
+// contribute span fewer than five binades; with 8 significant bits each, every product fq_i x_i
+// (fq_i = j / 2, j <= 12) is a multiple of 2^(e - 8) for the smallest such element's exponent e,
+// and every partial sum of the 16 stays below 2^(e + 13): 21 bits.  F_k <= 16 * 36 in units of 1/4.
+// What is left to bound:
+//  * the reference's own roundings.  Its dequantised value is c_i * d1 or c_i * (d1 (+) delta),
+//    within 2u (4u for a maximum with more than 8 significant bits) of h_k fq_i with h_k = d1;
+//    its residual, square and summation add 1 + 1 + 9 roundings: with scaled residuals of at
+//    most 1 (sum at most 16, sum of squares S at most 16)
+//        |E_ref - E_k| <= h_k^2 u (200 sqrt(S) + 11 S) <= 976 u h_k^2,          u = 2^-24;
+//  * three roundings here (q_k, h_k q_k, the difference): <= 3u (|h_6 q_6| + |h_4 q_4|) on the half difference.
+// Tolerance on the half difference: 2^-14 (h_6^2 + h_4^2) + 2^-21 (|h_6 q_6| + |h_4 q_4|), i.e. 2048u per
+// candidate against 976u and 8u against 3u.  One factor h_k of every product is taken relative to
+// the tensor maximum's power of two (FastLutEntry::hh in its product form), so that nothing
+// leaves fp32's normal range for the tensor maxima the shortcuts are used with (QuantConsts::shortcut_ok).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// Byte SEL of `word` -> the two E2M1 values as a bf16 pair (low nibble first).
+template <int SEL>
+FOS_DEVICE bf16x2_t unpack_fp4_bf16(uint32_t word) {
+    return __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(word, 1.0f, SEL);
+}
+
+FOS_DEVICE float dot2_bf16(bf16x2_t a, bf16x2_t b, float c) { return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false); }
+
+// +1: the second candidate's error is surely smaller; -1: surely not; 0: within the tolerance.
+FOS_DEVICE int product_compare(float FA, float GA, const FastLutEntry &A, float FB, float GB, const FastLutEntry &B) {
+    const float qA = __builtin_fmaf(0.5f * A.d1, FA, -GA), qB = __builtin_fmaf(0.5f * B.d1, FB, -GB);
+    const float pA = A.hh * qA, pB = B.hh * qB;  // (hh: d1 over the maximum's power of two)
+    const float D = pB - pA;
+    const float T = __builtin_fmaf(0x1p-21f, fabsf(pA) + fabsf(pB), 0x1p-14f * __builtin_fmaf(A.hh, A.d1, B.hh * B.d1));
+    if (fabsf(D) > T) return D < 0.0f ? 1 : -1;
+    return 0;
 }
 
 // The two rare paths are real function calls (arguments and results by value, in
@@ -345,11 +400,14 @@ __device__ __attribute__((noinline)) BlockOut generic_block_sr(Block16 blk, Quan
 // type beyond the conversion to f32: the scaled value is the reference's own x * inv, the division of
 // the block maximum by 6 or 4 is correctly rounded for every fp16 numerator too (checked exhaustively),
 // and fq * s * amax stays exact with the 11 significant bits of an fp16 maximum (2 + 4 + 11 <= 24).
-template <int RULE, bool TWO_D, bool SR, bool F16 = false>
+// PRODUCT: the MSE shortcut in its product form (bf16 elements, 1x16 blocks, round to nearest; the table built
+// with make_lut_entry<true>).
+template <int RULE, bool TWO_D, bool SR, bool F16 = false, bool PRODUCT = false>
 FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq,
                                               bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
                                               uint64_t blkid) {
     static_assert(!F16 || (!TWO_D && !SR), "fp16 elements: 1x16 blocks, round to nearest");
+    static_assert(!PRODUCT || (RULE == FOS_RULE_MSE && !TWO_D && !SR && !F16), "product form: MSE, 1x16, bf16, round to nearest");
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
     // the certified shortcut: MSE, and MAE for 1x16 blocks.  (Abs-max has one too, but 3 % of the
     // blocks of N(0,1) data tie exactly under that rule -- the largest residual belongs to an
@@ -423,7 +481,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                         SA = row16_sum_lane0(SA);
                         SB = row16_sum_lane0(SB);
                     }
-                    const int cmp = shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
+                    const int cmp = k.shortcut_ok ? shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B)) : 0;
                     certain = cmp != 0;
                     pickB = cmp > 0;
                 }
@@ -449,7 +507,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
             }
             const FastLutEntry B = lut[s4];
             uint32_t a0 = 0, a1 = 0, b0 = 0, b1 = 0;
-            float SA = 0.0f, SB = 0.0f;
+            float SA = 0.0f, SB = 0.0f, GA = 0.0f, GB = 0.0f;  // (product form: SA / SB hold F)
             static_for<0, 8>([&](auto jc) {
                 constexpr int j = decltype(jc)::value;
                 const float xa0 = scaled(x[2 * j], A.inv), xa1 = scaled(x[2 * j + 1], A.inv);
@@ -461,7 +519,7 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     a1 = pack_fp4<(j & 3)>(a1, xa0, xa1);
                     b1 = pack_fp4<(j & 3)>(b1, xb0, xb1);
                 }
-                if (SHORTCUT) {
+                if constexpr (!PRODUCT && SHORTCUT) {
                     const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
                     const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
                     accumulate_scaled<RULE>(fa.x - xa0, fa.y - xa1, SA);
@@ -469,12 +527,28 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 }
             });
             bool pickB = false, certain = false;
-            if (SHORTCUT) {
+            if constexpr (PRODUCT) {
+                // (from the finished code words: decoding byte j while the word is still being filled made the
+                // compiler keep a copy of every intermediate word)
+                static_for<0, 8>([&](auto jc) {
+                    constexpr int j = decltype(jc)::value;
+                    const bf16x2_t fa = unpack_fp4_bf16<(j & 3)>(j < 4 ? a0 : a1);
+                    const bf16x2_t fb = unpack_fp4_bf16<(j & 3)>(j < 4 ? b0 : b1);
+                    const bf16x2_t xw = __builtin_bit_cast(bf16x2_t, blk.w[j]);
+                    GA = dot2_bf16(fa, xw, GA);
+                    SA = dot2_bf16(fa, fa, SA);
+                    GB = dot2_bf16(fb, xw, GB);
+                    SB = dot2_bf16(fb, fb, SB);
+                });
+                const int cmp = k.shortcut_ok ? product_compare(SA, GA, A, SB, GB, B) : 0;
+                certain = cmp != 0;
+                pickB = cmp > 0;
+            } else if (SHORTCUT) {
                 if (TWO_D) {
                     SA = row16_sum_lane0(SA);
                     SB = row16_sum_lane0(SB);
                 }
-                const int cmp = shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
+                const int cmp = k.shortcut_ok ? shortcut_compare<RULE, TWO_D>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B)) : 0;
                 certain = cmp != 0;
                 pickB = cmp > 0;
             }
@@ -563,7 +637,7 @@ FOS_DEVICE BlockOut quantize_block_if4_mse(const Block16 &blk, const QuantConsts
                 SA = row16_sum_lane0(SA);
                 SB = row16_sum_lane0(SB);
             }
-            const int cmp = shortcut_compare<FOS_RULE_MSE, TWO_D>(SA, 1.0f, SB, 1.0f);  // same scale: compare the sums
+            const int cmp = k.shortcut_ok ? shortcut_compare<FOS_RULE_MSE, TWO_D>(SA, 1.0f, SB, 1.0f) : 0;  // same scale: compare the sums
             if (cmp > 0) return BlockOut{b0, b1, s | 0x80u};
             if (cmp < 0) return BlockOut{a0, a1, s};
             // undecided (uniform over the 16 lanes of a tile when TWO_D: both sums are tile sums)

@@ -55,6 +55,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     k.qdiv = p.qdiv;
     k.errdiv = p.errdiv;
     k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
+    k.shortcut_ok = shortcut_range(k.amax);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
@@ -218,11 +219,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     uint32_t tile = blockIdx.x;
     RowsTile cur = open_tile(tile, tile < n_tiles);
     Block16 ring[4];
-#ifdef FOS_TRACE
-    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime(), tr_c0 = __builtin_amdgcn_s_memtime();
-    uint64_t tr_tile[5] = {0, 0, 0, 0, 0};
-    int tr_n = 0;
-#endif
     load(cur, 0, ring[0]);
     load(cur, 1, ring[1]);
     load(cur, 2, ring[2]);
@@ -240,6 +236,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     k.errdiv = p.errdiv;
     // (the exact evaluation needs fq * s * amax exact: a maximum of the element type's significant bits)
     k.exact_ok = k.errdiv == 1536.0f && (amax_bits & (F16 ? 0x1fffu : 0xffffu)) == 0;
+    k.shortcut_ok = shortcut_range(k.amax);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
@@ -250,7 +247,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     QuantConsts kt = k;
     if (PSEUDO && kStaticRule) kt.errdiv = p.c;
     const bool deq_lut = PSEUDO && in_range && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
-    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, kt);
+    // the MSE decision in its product form (bf16 elements, round to nearest)
+    constexpr bool kProduct = RULE == FOS_RULE_MSE && !SR && !IF4 && !F16;
+    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry<kProduct>(threadIdx.x, kt);
     __syncthreads();
 
     auto process = [&](const RowsTile &t, int g, const Block16 &b) {
@@ -262,8 +261,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         BlockOut o{0u, 0u, 0u};
         if (!padding_step) {
             if constexpr (IF4) o = quantize_block_if4_mse<false>(b, k, enc_fast, rq, in_range, lut);
-            else o = quantize_block_nvfp4_fast<RULE, false, SR, F16>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
-                                                                (uint64_t)(row * sf_cols + t.cb));
+            else o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                                                                          (uint64_t)(row * sf_cols + t.cb));
         }
         if (PSEUDO) {
             uint32_t w[8];
@@ -342,22 +341,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         }
         cur = nxt;
         tile = next;
-#ifdef FOS_TRACE
-        if (tr_n < 5) tr_tile[tr_n++] = __builtin_amdgcn_s_memrealtime();
-#endif
     }
-#ifdef FOS_TRACE
-    if (lane == 0) {
-        // trace record behind the scale bytes: {start, end (100 MHz ticks), shader cycles, tile ends...}
-        uint64_t *rec = reinterpret_cast<uint64_t *>(p.sf + p.rows_p * sf_cols) + (blockIdx.x * 4 + wave) * 8;
-        rec[0] = tr_t0;
-        rec[1] = __builtin_amdgcn_s_memrealtime();
-        rec[2] = __builtin_amdgcn_s_memtime() - tr_c0;
-        for (int i = 0; i < 3; ++i) rec[3 + i] = tr_tile[i];
-        rec[6] = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20) /* XCC_ID */;
-        rec[7] = __builtin_amdgcn_s_getreg((32 - 1) << 11 | 0 << 6 | 4) /* HW_ID */;
-    }
-#endif
 }
 
 // 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): round to nearest, every rule.

@@ -31,6 +31,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
     k.qdiv = p.qdiv;
     k.errdiv = p.errdiv;
     k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
+    k.shortcut_ok = shortcut_range(k.amax);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
 
     // The fast formulation assumes that no intermediate leaves the normal fp32 range,

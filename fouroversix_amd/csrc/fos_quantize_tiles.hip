@@ -212,11 +212,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     // or with three wavefronts per SIMD and deeper queues, the launch took as long or longer --
     // wavefronts whose first loads were served late then finished late.)
     Block16 blk[4];
-#ifdef FOS_TRACE
-    const uint64_t tr_t0 = __builtin_amdgcn_s_memrealtime();
-    uint64_t tr_g[6] = {0, 0, 0, 0, 0, 0};
-    int tr_n = 0;
-#endif
 #pragma unroll
     for (int s = 0; s < 4; ++s) load(cur, 4 * s, blk[s]);
 
@@ -238,6 +233,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     const float rq = sgpr(1.0f / k.qdiv), rc = sgpr(1.0f / p.c);
     k.rerr = sgpr(1.0f / k.errdiv);
     k.fast_div = in_range && k.errdiv == 1536.0f;
+    k.shortcut_ok = shortcut_range(k.amax);
     // pseudo-quantize: the table also serves the dequantization (divisor c: the selection's for the adaptive
     // rules; the static rules make no selection, so their table is built with c)
     constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
@@ -247,9 +243,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, kt);
     __syncthreads();
 
-#ifdef FOS_TRACE
-    tr_g[tr_n++] = __builtin_amdgcn_s_memrealtime();  // setup done
-#endif
     // one quantised block (row `rstep` rows below the share's first, + li) to memory
     auto emit = [&](const TilesPos &t, uint32_t rstep, uint32_t c0, uint32_t c1, uint32_t sbyte, bool pred) {
         const int32_t row = t.row0 + (int32_t)rstep + li;
@@ -439,7 +432,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 SA = MAXRULE ? tile_max(SA) : tile_sum(SA);
                 SB = MAXRULE ? tile_max(SB) : tile_sum(SB);
                 // (IF4: one scale, so the two sums compare as they are)
-                if (IF4) cmp = shortcut_compare<FOS_RULE_MSE, true>(SA, 1.0f, SB, 1.0f);
+                if (!k.shortcut_ok) cmp = 0;
+                else if (IF4) cmp = shortcut_compare<FOS_RULE_MSE, true>(SA, 1.0f, SB, 1.0f);
                 else cmp = shortcut_compare<RULE, true>(SA, shortcut_weight<RULE>(A), SB, shortcut_weight<RULE>(B));
             }
             // an all-zero tile came out as zero codes under the zero scale byte
@@ -493,9 +487,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 #pragma nounroll
         for (uint32_t q = 0; q < 4; ++q) {
             sw |= process(cur, q, q == 3 ? nxt : cur, q == 3 ? 0u : q + 1) << (8 * q);
-#ifdef FOS_TRACE
-            if (tr_n < 6) tr_g[tr_n++] = __builtin_amdgcn_s_memrealtime();
-#endif
         }
         if (tiled) {
             // 16-byte unit of rows r, r + 32, r + 64, r + 96 and block columns 4 g .. 4 g + 3: word q =
@@ -512,15 +503,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         cur = nxt;
         tile = next;
     }
-#ifdef FOS_TRACE
-    if (lane == 0) {
-        // trace record behind the scale bytes: {start, end (100 MHz ticks), setup done, group ends...}
-        uint64_t *rec = reinterpret_cast<uint64_t *>(p.sf + p.rows_p * sf_cols) + (blockIdx.x * 4 + wave) * 8;
-        rec[0] = tr_t0;
-        rec[1] = __builtin_amdgcn_s_memrealtime();
-        for (int i = 0; i < 6; ++i) rec[2 + i] = tr_g[i];
-    }
-#endif
 }
 
 }  // namespace

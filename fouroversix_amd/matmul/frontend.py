@@ -14,6 +14,7 @@ from typing import Any
 
 import torch
 
+from fouroversix_amd import _native as nat
 from fouroversix_amd.quantize import QuantizationConfig, QuantizedTensor, quantize
 from fouroversix_amd.quantize import ops
 from fouroversix_amd.quantize.frontend import attach_known_amax, dequantize, dequantize_divisor
@@ -123,6 +124,27 @@ def _unit_alpha(device: torch.device) -> torch.Tensor:
     return one
 
 
+# Words that receive max|output| of a GEMM (emit_amax): the kernel folds into the word with an unsigned
+# atomic max, so it has to start at zero.  Outside a graph capture the words come from a zero-filled
+# block per (device, stream), one fresh word per call (a fill kernel per call would cost a decode-sized
+# GEMM a third of its time; the block's one fill is ordered before its words' uses by the stream); a
+# captured call gets a word of its own with its own fill, which replays with it.
+_AMAX_WORDS = 4096
+_AMAX_POOL: dict = {}
+
+
+def _fresh_amax_word(device: torch.device) -> torch.Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(1, dtype=torch.float32, device=device)
+    key = (device, nat.current_stream(device))
+    slot = _AMAX_POOL.get(key)
+    if slot is None or slot[1] == _AMAX_WORDS:
+        slot = _AMAX_POOL[key] = [torch.zeros(_AMAX_WORDS, dtype=torch.float32, device=device), 0]
+    word = slot[0][slot[1] : slot[1] + 1]
+    slot[1] += 1
+    return word
+
+
 def gemm_alpha(input: QuantizedTensor, other: QuantizedTensor) -> torch.Tensor:
     """``(amaxA * amaxB) / (qA sA qB sB adjA adjB)`` as a device f32[1] (reference
     matmul/cutlass/backend.py:86-98); one small kernel when both maxima are f32 GPU tensors."""
@@ -170,7 +192,7 @@ def quantized_matmul(
         and (out_dtype is DataType.bfloat16 or out_dtype is DataType.float16)
         and not torch.compiler.is_compiling()
     ):
-        d_amax = torch.zeros(1, dtype=torch.float32, device=ra[6]) if emit_amax else None
+        d_amax = _fresh_amax_word(ra[6]) if emit_amax else None
         out = ops.gemm_nvfp4_from_amax(
             ra[4], rb[0], ra[1], rb[1], ra[2], rb[2], ra[5] * rb[5],
             torch.bfloat16 if out_dtype is DataType.bfloat16 else torch.float16, d_amax, checked=True,

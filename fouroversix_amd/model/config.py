@@ -43,7 +43,7 @@ class ModuleQuantizationConfig:
     disable_fprop_quantization: bool = False
     disable_wgrad_quantization: bool = False
     dtype: DataType = DataType.nvfp4
-    emit_output_amax: bool = False  # (not in the reference) the forward GEMM records max|output| for the next layer's quantize
+    emit_output_amax: bool = True  # (not in the reference) the forward GEMM records max|output| for the next layer's quantize
     gradient_dtype: DataType | None = None
     gradient_round_style: RoundStyle = RoundStyle.stochastic
     gradient_scale_rule: ScaleRule | None = None

@@ -80,20 +80,36 @@ def _quantize_meta(x: torch.Tensor, config: QuantizationConfig) -> QuantizedTens
 
 # max|x| that a producer already has (the FP4 GEMM can record it while storing its output): kept
 # as an attribute of the tensor object together with the tensor's version counter, so that an
-# in-place write, or any operation that returns a new tensor, drops it.
+# in-place write, or any operation that returns a new tensor, drops it.  Only writes that torch
+# counts are seen: a write through ``x.data``, through a raw pointer (this library's own C entry
+# points, an ``out=`` kernel of another extension) leaves the counter, and with it the tag, as it was.
+# Tensors made under ``torch.inference_mode()`` have no version counter: they are never tagged and
+# ``quantize`` finds their maximum itself.
 _KNOWN_AMAX = "_fos_known_amax"
 
 
+def _version_or_none(x: torch.Tensor) -> int | None:
+    if x.is_inference():
+        return None
+    try:
+        return x._version
+    except RuntimeError:  # tensors that do not track a version counter
+        return None
+
+
 def attach_known_amax(x: torch.Tensor, amax: torch.Tensor) -> torch.Tensor:
-    """Record ``amax`` (device f32[1] = max|x|) on ``x`` for a later ``quantize(x)``."""
-    setattr(x, _KNOWN_AMAX, (amax, x._version))
+    """Record ``amax`` (device f32[1] = max|x|) on ``x`` for a later ``quantize(x)``; without effect
+    on tensors that have no version counter (inference tensors)."""
+    version = _version_or_none(x)
+    if version is not None:
+        setattr(x, _KNOWN_AMAX, (amax, version))
     return x
 
 
 def known_amax(x: torch.Tensor) -> torch.Tensor | None:
     """The maximum recorded by ``attach_known_amax`` if ``x`` has not been written since."""
     tag = getattr(x, _KNOWN_AMAX, None)
-    if tag is None or tag[1] != x._version or tag[0].device != x.device:
+    if tag is None or tag[0].device != x.device or tag[1] != _version_or_none(x):
         return None
     return tag[0]
 

@@ -234,10 +234,13 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
                            orig, (mp, np_), blocked)
 
 
-def selection_errors(x, *, dtype="nvfp4", scale_rule="mse", block_scale_2d=False, amax=None, threads=None) -> np.ndarray:
+def selection_errors(x, *, dtype="nvfp4", scale_rule="mse", block_scale_2d=False, amax=None, threads=None,
+                     round_style="nearest", seed=0, offset=0) -> np.ndarray:
     """f32 [M, N/16, 2]: the two errors the adaptive rule compared for every 1x16 block of an
-    unpadded-or-padded bf16 input (round to nearest), first the "6" / E2M1 candidate, second
-    the "4" / INT4 one; the second wins when strictly smaller."""
+    unpadded-or-padded bf16 input, first the "6" / E2M1 candidate, second the "4" / INT4 one; the
+    second wins when strictly smaller.  With a stochastic ``round_style`` the candidates are the
+    stochastically rounded ones of (seed, offset), and the width must already be a multiple of 64
+    (the dither is keyed by the block's index in the padded tensor)."""
     xb, x_type = input_bits(x)
     xp = np.ascontiguousarray(xb)
     m, n = xp.shape
@@ -247,8 +250,8 @@ def selection_errors(x, *, dtype="nvfp4", scale_rule="mse", block_scale_2d=False
     amax_in = None if amax is None else np.array([amax], dtype=np.float32)
     amax_out = np.zeros(1, dtype=np.float32)
     rc = lib().fos_oracle_quantize_errors(
-        _ptr(xp), x_type, m, n, DTYPE_IDS[dtype], RULE_IDS[scale_rule], 0, int(block_scale_2d), 0, 0,
-        _ptr(codes), _ptr(sf), _ptr(amax_out), None if amax_in is None else _ptr(amax_in),
+        _ptr(xp), x_type, m, n, DTYPE_IDS[dtype], RULE_IDS[scale_rule], ROUND_IDS[round_style], int(block_scale_2d),
+        seed, offset, _ptr(codes), _ptr(sf), _ptr(amax_out), None if amax_in is None else _ptr(amax_in),
         threads or default_threads(), _ptr(errors))
     assert rc == 0
     return errors

@@ -73,6 +73,7 @@ LLAMA_SHAPES = [(m, n, k) for m in (16, 128, 2048, 8192) for (n, k) in ((4096, 4
 
 @pytest.mark.parametrize(("m", "n", "k"), [(8192, 8192, 8192), *LLAMA_SHAPES,
                                            (16384, 4096, 4096), (16384, 1024, 4096),  # the decoder stack's token count, k/v projection
+                                           (16384, 14336, 4096), (16384, 4096, 14336),  # ... its gate / up and down projections
                                            (256, 384, 2368), (64, 14336, 4096), (96, 11008, 4096)])
 def test_gemm_full_size_sampled(oracle, m, n, k):
     """Headline shape, every Llama-3-8B linear shape (M in {16, 128, 2048, 8192}) and the
@@ -486,3 +487,75 @@ def test_linear_layers_hand_the_maximum_on():
             assert (known_amax(y) is not None) == emit
         outs.append(y)
     assert torch.equal(outs[0], outs[1])
+
+
+class _DecoderProjections(nn.Module):
+    """The seven linear projections of one Llama-3-8B decoder layer (grouped-query attention: 1024-wide
+    k / v), chained wherever a GEMM output can feed the next projection directly: o reads q's
+    output, gate / up read o's, down reads gate's.  No attention and no non-linearity, as in the
+    benchmark's layer stack."""
+
+    def __init__(self):
+        super().__init__()
+        mk = lambda i, o: nn.Linear(i, o, bias=False, dtype=torch.bfloat16)  # noqa: E731
+        self.q_proj, self.k_proj, self.v_proj, self.o_proj = mk(4096, 4096), mk(4096, 1024), mk(4096, 1024), mk(4096, 4096)
+        self.gate_proj, self.up_proj, self.down_proj = mk(4096, 14336), mk(4096, 14336), mk(14336, 4096)
+
+    def forward(self, x):
+        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        h = self.o_proj(q)
+        g, u = self.gate_proj(h), self.up_proj(h)
+        return {"q_proj": (x, q), "k_proj": (x, k), "v_proj": (x, v), "o_proj": (q, h), "gate_proj": (h, g),
+                "up_proj": (h, u), "down_proj": (g, self.down_proj(g))}
+
+
+def test_decoder_layer_at_16384_tokens_through_quantize_model(oracle):
+    """One decoder layer's projections at batch x seq = 8 x 2048 tokens through `quantize_model`
+    on an nn.Module (reference src/fouroversix/model/modules/linear.py:43-94, model/quantize.py:101-127):
+    weights 0.02 N(0,1) pre-quantized 4/6-MSE on 16 x 16 blocks, activations quantized on the fly
+    (4/6-MSE, 1 x 16).  Every projection's output is compared on 160 x 160 sampled entries with the
+    oracle's quantize of the same input and its fp64-accumulated product; the layer is run with the
+    GEMM-recorded maximum handed to the next quantize and without, and the two must agree bit for bit;
+    so must a run under torch.inference_mode(), where no maximum is handed on."""
+    from fouroversix_amd.quantize import known_amax
+
+    torch.manual_seed(11)
+    block = _DecoderProjections()
+    with torch.no_grad():
+        for lin in block.children():
+            lin.weight.copy_((0.02 * torch.randn(lin.weight.shape)).bfloat16())
+    weights = {name: lin.weight.detach().clone() for name, lin in block.named_children()}
+    block.cuda()
+    x = make_input("randn", (8, 2048, 4096), 71).cuda()
+    results = {}
+    for emit in (True, False):
+        model = _DecoderProjections().cuda()
+        model.load_state_dict(block.state_dict())
+        fos.quantize_model(model, fos.ModelQuantizationConfig(weight_scale_2d=True, emit_output_amax=emit))
+        for lin in model.children():
+            assert isinstance(lin, fos.FourOverSixLinear)
+            lin.quantize_weight_()
+        with torch.no_grad():
+            results[emit] = model(x)
+        for name, (_, out) in results[emit].items():
+            assert out.shape[:2] == (8, 2048)
+            assert (known_amax(out) is not None) == emit, name
+        if emit:
+            with torch.inference_mode():
+                inf = model(x)
+            for name, (_, out) in inf.items():
+                assert known_amax(out) is None and torch.equal(out, results[True][name][1]), name
+    for name in results[True]:
+        assert torch.equal(results[True][name][1], results[False][name][1]), f"{name}: recorded maximum changes the result"
+    g = torch.Generator("cpu").manual_seed(8)
+    for name, (inp, out) in results[True].items():
+        inp2, out2 = inp.reshape(-1, inp.shape[-1]), out.reshape(-1, out.shape[-1])
+        rows = torch.randperm(inp2.shape[0], generator=g)[:160].sort().values
+        cols = torch.randperm(out2.shape[1], generator=g)[:160].sort().values
+        # the oracle quantizes the whole activation (its maximum is the tensor's) and the sampled weight rows
+        # of the whole weight (16 x 16 tiles)
+        ra = oracle.quantize(inp2.cpu(), scale_rule="mse")
+        rw = oracle.quantize(weights[name], scale_rule="mse", block_scale_2d=True)
+        ref, _ = oracle.gemm_nvfp4(ra.values[rows.numpy()], ra.scale_rows[rows.numpy()], rw.values[cols.numpy()],
+                                   rw.scale_rows[cols.numpy()], oracle.gemm_alpha(ra, rw))
+        check(bits16(out2[rows.cuda()][:, cols.cuda()]), ref, oracle, name)

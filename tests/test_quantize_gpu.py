@@ -181,6 +181,7 @@ WEIGHT_CASES = [(shape, "weight", cfg)
     ((8192, 8192), "randn", dict(scale_rule="static_6")),
     *WEIGHT_CASES,                                                # Llama-3-8B weight shapes x {4/6-MSE, static_6, IF4}, 16 x 16 blocks
     ((16384, 4096), "randn", dict(scale_rule="mse")),             # the decoder stack's activations
+    ((16384, 14336), "randn", dict(scale_rule="mse")),            # ... the down projection's
     ((2048, 4096), "weight", dict(dtype="if4", scale_rule="mse")),
     # the other two adaptive rules through their certified shortcuts: 4 M blocks each, the closest calls among
     # them a few 1e-7 apart, plus the stochastic style on top
@@ -252,6 +253,31 @@ def test_extreme_ranges_take_the_operation_by_operation_path(oracle, scale, two_
     assert_same_quantization(q, oracle.quantize(x, dtype="if4", scale_rule="mse", block_scale_2d=two_d), f"scale {scale} if4")
 
 
+_FAR_CONFIGS = [dict(scale_rule="mse"), dict(scale_rule="mse", block_scale_2d=True), dict(scale_rule="mae"),
+                dict(scale_rule="mae", block_scale_2d=True), dict(scale_rule="abs_max", block_scale_2d=True),
+                dict(scale_rule="mse", round_style="stochastic"), dict(scale_rule="mse", round_style="stochastic", block_scale_2d=True),
+                dict(dtype="if4", scale_rule="mse"), dict(dtype="if4", scale_rule="mse", block_scale_2d=True)]
+
+
+@pytest.mark.parametrize("cfg", _FAR_CONFIGS, ids=lambda c: "-".join(str(v) for v in c.values()))
+@pytest.mark.parametrize("exponent", [-98, -90, -72, -66, -61, -59, -50, -41, -39, -30, 30, 39, 41, 59, 61, 90, 99])
+def test_tensor_maxima_far_from_one(oracle, exponent, cfg):
+    """The certified shortcuts model the reference's error sums with relative rounding errors, which holds
+    only while the reference's own fp32 squares and sums neither underflow nor overflow: a tensor of
+    values around 2^-70 has every squared error flushed to zero there, so every block ties and takes the
+    first candidate.  The kernels decide from their shortcuts for tensor maxima in [2^-40, 2^40] (with
+    the weights taken relative to the maximum's power of two) and evaluate exactly beyond.  Every
+    shortcut against the oracle, bit for bit, on both sides of the limits."""
+    x = (make_input("randn", (512, 1024), 14).float() * 2.0**exponent).bfloat16()
+    kw = {"kwargs": {"seed": 3}} if "round_style" in cfg else {}
+    okw = {"seed": 3} if "round_style" in cfg else {}
+    assert_same_quantization(hip_quantize(x, **cfg, **kw), oracle.quantize(x, **cfg, **okw), f"2^{exponent} {cfg}")
+    if cfg.get("dtype", "nvfp4") == "nvfp4" and "round_style" not in cfg:
+        r = fos.quantize(x.cuda(), fos.QuantizationConfig(pseudo_quantize=True, **cfg))
+        q = hip_quantize(x, **cfg)
+        assert torch.equal(r.view(torch.int16), fos.dequantize(q, dtype=torch.bfloat16).view(torch.int16))
+
+
 @pytest.mark.parametrize("two_d", [False, True], ids=["1d", "2d"])
 def test_if4_mse_fast_path_inputs(oracle, two_d):
     """IF4 with the MSE rule decides most blocks from sums in the scaled domain; inputs that
@@ -268,24 +294,55 @@ def test_if4_mse_fast_path_inputs(oracle, two_d):
     assert_same_quantization(q, oracle.quantize(x, dtype="if4", block_scale_2d=two_d, amax=given), "24-bit maximum")
 
 
+def _near_tie_cases(golden_dir):
+    d = np.load(os.path.join(golden_dir, "near_ties.npz"))
+    return d, sorted(k[:-2] for k in d.files if k.endswith(".x"))
+
+
 def test_near_ties_take_the_exact_decision(oracle, golden_dir):
     """Blocks and tiles whose two candidate errors differ by a few units in the last place (found
-    by a CPU search, tests/golden/make_near_ties.py): the kernels' certified shortcut must hand
-    every one of them to the exact evaluation.  4/6 and IF4, 1-D and 2-D, tensor maximum from the
-    data and a caller-supplied 24-bit maximum; also under the fused pseudo-quantize epilogue."""
-    d = np.load(os.path.join(golden_dir, "near_ties.npz"))
-    for case in sorted(k[:-2] for k in d.files if k.endswith(".x")):
+    by a CPU search, tests/golden/make_near_ties.py): the kernels' certified shortcuts must hand
+    every one of them to the exact evaluation.  4/6 under the MSE, MAE and abs-max rules and IF4,
+    1-D and 2-D, tensor maximum from the data and a caller-supplied 24-bit maximum, round to nearest
+    and the stochastic style (whose candidates are the stochastically rounded ones of the stored
+    seed); round to nearest also under the fused pseudo-quantize epilogue."""
+    d, cases = _near_tie_cases(golden_dir)
+    rules = set()
+    for case in cases:
         parts = case.split(".")
-        dtype, two_d, given = parts[0], parts[1] == "2d", len(parts) == 3
+        dtype, two_d, rule, style, given = parts[0], parts[1] == "2d", parts[2], parts[3], len(parts) == 5
+        rules.add((dtype, two_d, rule, style))
         x = torch.from_numpy(d[case + ".x"].view(np.int16).copy()).view(torch.bfloat16)
-        amax = float(d[case + ".amax"][0])
+        amax, seed = float(d[case + ".amax"][0]), int(d[case + ".seed"][0])
         kwargs = {"amax": torch.tensor(amax, device="cuda")} if given else {}
-        q = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype=dtype, scale_rule="mse", block_scale_2d=two_d, kwargs=kwargs))
-        ref = oracle.quantize(x, dtype=dtype, scale_rule="mse", block_scale_2d=two_d, amax=amax if given else None)
+        if style != "nearest":
+            kwargs["seed"] = seed
+        q = fos.quantize(x.cuda(), fos.QuantizationConfig(dtype=dtype, scale_rule=rule, round_style=style, block_scale_2d=two_d, kwargs=kwargs))
+        ref = oracle.quantize(x, dtype=dtype, scale_rule=rule, round_style=style, block_scale_2d=two_d, seed=seed, amax=amax if given else None)
         assert_same_quantization(q, ref, case)
-        if dtype == "nvfp4":
-            r = fos.quantize(x.cuda(), fos.QuantizationConfig(scale_rule="mse", block_scale_2d=two_d, pseudo_quantize=True, kwargs=kwargs))
+        if dtype == "nvfp4" and style == "nearest":
+            r = fos.quantize(x.cuda(), fos.QuantizationConfig(scale_rule=rule, block_scale_2d=two_d, pseudo_quantize=True, kwargs=kwargs))
             assert torch.equal(r.view(torch.int16), fos.dequantize(q, dtype=torch.bfloat16).view(torch.int16)), case
+    # every instantiation that decides from a shortcut has a case
+    for need in (("nvfp4", False, "mse", "nearest"), ("nvfp4", True, "mse", "nearest"), ("nvfp4", False, "mae", "nearest"),
+                 ("nvfp4", True, "mae", "nearest"), ("nvfp4", True, "abs_max", "nearest"), ("if4", False, "mse", "nearest"),
+                 ("if4", True, "mse", "nearest"), ("nvfp4", False, "mse", "stochastic"), ("nvfp4", False, "mae", "stochastic"),
+                 ("nvfp4", True, "mse", "stochastic")):
+        assert need in rules, need
+
+
+def test_near_ties_on_fp16_inputs(oracle, golden_dir):
+    """The same near-tie blocks handed over as fp16 tensors (every bf16 value of the fixture, at most 8
+    in magnitude, is an fp16 value too): the fp16 instantiation of the 1 x 16 streaming kernel decides
+    them as the oracle does on the fp16 input."""
+    d, cases = _near_tie_cases(golden_dir)
+    for case in cases:
+        parts = case.split(".")
+        if parts[0] != "nvfp4" or parts[1] != "1d" or parts[3] != "nearest" or len(parts) == 5:
+            continue
+        x = torch.from_numpy(d[case + ".x"].view(np.int16).copy()).view(torch.bfloat16).half()
+        q = fos.quantize(x.cuda(), fos.QuantizationConfig(scale_rule=parts[2]))
+        assert_same_quantization(q, oracle.quantize(x, scale_rule=parts[2]), case + " as fp16")
 
 
 def test_negative_zero_inputs(oracle):
