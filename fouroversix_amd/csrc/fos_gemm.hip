@@ -154,9 +154,7 @@ FOS_DEVICE void tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
 enum { kOutF16 = 0, kOutBF16 = 1, kOutPartial = 2 };
 
 template <int WAVES_M, int WAVES_N, int WM, int WN, int OUT>
-// (four wavefronts with eight MFMA tiles each: two workgroups per compute unit, so at most 256 registers)
-__global__ __launch_bounds__(64 * WAVES_M *WAVES_N) __attribute__((amdgpu_waves_per_eu(WAVES_M *WAVES_N == 4 && WM * WN == 8 ? 2 : 1)))
-void gemm_nvfp4_kernel(const GemmParams p) {
+__global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const GemmParams p) {
     constexpr bool OUT_BF16 = OUT == kOutBF16;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
@@ -1043,7 +1041,7 @@ static int launch_decode(GemmParams &p, int out_type, hipStream_t s) {
 
 // Which kernel runs a shape, and how K is split across workgroups (splits > 1 needs the
 // caller's workspace for splits * M * N FP32 partials).
-enum { kPlanBig, kPlanWide, kPlanSmall, kPlanSkinny, kPlanWide4 };
+enum { kPlanBig, kPlanWide, kPlanSmall, kPlanSkinny };
 struct GemmPlan {
     int kind, splits, ksteps_per_split;
     int narrow;  // M <= 16: workgroups of 16 instead of 32 rows of B
@@ -1074,15 +1072,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
             g.wide = 1;
             tiles = (N / 64) * (M > 64 ? 2 : 1);
         }
-    } else if ((M % 256 == 0) && (N % 256 == 0) && ((M / 256) * (N / 256) >= 256 || tile == 256) && tile != 128 && tile != 130) {
+    } else if ((M % 256 == 0) && (N % 256 == 0) && ((M / 256) * (N / 256) >= 256 || tile == 256) && tile != 128) {
         // 256 x 256 tiles once they give each of the 256 compute units a workgroup
         g.kind = kPlanBig;
-        g.splits = 1;
-        g.ksteps_per_split = (int)(K / BK);
-        return g;
-    } else if (tile == 130 && M % 128 == 0 && N % 256 == 0 && M >= 128) {
-        // experimental: 128 x 256 tiles on four wavefronts of 128 x 64, two workgroups per compute unit
-        g.kind = kPlanWide4;
         g.splits = 1;
         g.ksteps_per_split = (int)(K / BK);
         return g;
@@ -1185,7 +1177,6 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     switch (g.kind) {
         case kPlanBig: return launch_gemm<1, 8, 8, 1>(p, out_type, s);
         case kPlanWide: return launch_gemm<1, 8, 4, 1>(p, out_type, s);
-        case kPlanWide4: return launch_gemm<1, 4, 4, 2>(p, out_type, s);
         case kPlanSkinny:
             // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);

@@ -157,15 +157,17 @@ struct QuantConsts {
     // not -- and the divisor 1536; without both, undecided blocks take the generic form.
     bool exact_ok = false;
     // The certified shortcuts of the adaptive rules model the reference's error sums with relative
-    // rounding errors.  That holds while the reference's own fp32 arithmetic -- squares of residuals of
-    // the size of amax / 1536 times a block scale down to 2^-9, sums of up to 256 of them -- neither
-    // underflows nor overflows (a tensor of values around 2^-70 has all its squared errors flushed to
-    // zero or rounded as sub-normals there, and every block ties): tensor maxima in [2^-40, 2^40].
-    // Beyond, every block takes the exact evaluation.
+    // rounding errors.  That holds while the reference's own fp32 arithmetic stays in the normal range:
+    // its squared residuals are of the size of (amax / 1536 x block scale)^2 with block scales down to
+    // 2^-9, so for a tensor of values around 2^-70 every squared error is flushed to zero or rounded as a
+    // sub-normal (and every block ties), and sums of up to 256 squares of residuals up to amax / 4 overflow
+    // from amax = 2^62 on.  The shortcuts are used for tensor maxima in [2^-40, 2^60]: at the lower end what
+    // the reference loses to sub-normal squares (<= 256 x 2^-150) is 2^-12 of the smallest tolerance
+    // (2^-15 h^2 with h >= 2^-59.6).  Beyond, every block takes the exact evaluation.
     bool shortcut_ok = false;
 };
 
-FOS_DEVICE bool shortcut_range(float amax) { return amax >= 0x1p-40f && amax <= 0x1p40f; }
+FOS_DEVICE bool shortcut_range(float amax) { return amax >= 0x1p-40f && amax <= 0x1p60f; }
 
 // v / k.errdiv with IEEE rounding (the sign of a zero quotient may differ; callers subtract).
 FOS_DEVICE float div_errdiv(float v, const QuantConsts &k) {

@@ -334,6 +334,72 @@ FOS_DEVICE bool exact_pick_b_1d(const float *x, uint32_t a0, uint32_t a1, uint32
     return reduce_error<RULE, false>(eB) < reduce_error<RULE, false>(eA);
 }
 
+// The same, one undecided block at a time spread over the wavefront: lane (c, e) = (lane >> 4 & 1, lane & 15)
+// evaluates element e of candidate c, and the 16 errors of a candidate meet in torch.sum's order through
+// DPP moves inside its row of 16 lanes -- about 40 instructions per undecided block, where the per-lane
+// form above costs the wavefront its 300 whenever a single lane is undecided (one wavefront step in
+// twenty on N(0,1) data).  Every lane of the wavefront must call it (convergent control flow); `scratch`
+// = 16 words of LDS private to the wavefront.  Returns the decision in the lanes that asked.
+struct ExactRequest {
+    bool wanted = false;
+    uint32_t b0 = 0, b1 = 0, sB = 0;  // second candidate (the first is the provisional BlockOut)
+};
+
+template <int RULE, bool F16>
+FOS_DEVICE bool exact_pick_b_spread(bool wanted, const Block16 &blk, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1,
+                                    const FastLutEntry &A, const FastLutEntry &B, uint32_t *scratch) {
+    static_assert(RULE == FOS_RULE_MSE || RULE == FOS_RULE_MAE, "rules that sum their errors");
+    const int lane = threadIdx.x & 63;
+    const int e = lane & 15, c = (lane >> 4) & 1;
+    bool pickB = false;
+    uint64_t pending = __builtin_amdgcn_ballot_w64(wanted);
+    while (pending != 0) {
+        const int l = __builtin_ctzll(pending);
+        pending &= pending - 1;
+        if (lane == l) {
+            uint4 *dst = reinterpret_cast<uint4 *>(scratch);
+            dst[0] = make_uint4(blk.w[0], blk.w[1], blk.w[2], blk.w[3]);
+            dst[1] = make_uint4(blk.w[4], blk.w[5], blk.w[6], blk.w[7]);
+            dst[2] = make_uint4(a0, a1, b0, b1);
+            dst[3] = make_uint4(f2u(A.d1), A.delta, f2u(B.d1), B.delta);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const uint32_t xw = scratch[e >> 1];
+        float x;
+        if (F16) x = (float)__builtin_bit_cast(_Float16, (uint16_t)((e & 1) ? xw >> 16 : xw));
+        else x = (e & 1) ? u2f(xw & 0xffff0000u) : u2f(xw << 16);
+        const uint32_t cw = scratch[8 + 2 * c + (e >> 3)];
+        const float fq = unpack_fp4<0>(cw >> (4 * (e & 7))).x;
+        FastLutEntry E;
+        E.d1 = u2f(scratch[12 + 2 * c]);
+        E.delta = scratch[13 + 2 * c];
+        const float d = candidate_residual(fq, E, x);
+        const float err = RULE == FOS_RULE_MSE ? d * d : fabsf(d);
+        // p[i] = err[i] + err[i + 8] in lanes 0..7 of the row, then ((p0 + p1) + p2) + ... + p7 into lane 7
+        const float pr = err + dpp_move<kDppRowShl + 8>(0.0f, err);
+        float t = pr;
+#pragma unroll
+        for (int step = 0; step < 7; ++step) t = dpp_move<kDppRowShr + 1>(-0.0f, t) + pr;
+        const float EA = __shfl(t, 7), EB = __shfl(t, 23);
+        if (lane == l) pickB = EB < EA;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    return pickB;
+}
+
+// exact_pick_b_1d from the packed block (for callers that no longer hold the unpacked elements).
+template <int RULE, bool F16>
+FOS_DEVICE bool exact_pick_b_1d_packed(const Block16 &blk, uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, const FastLutEntry &A,
+                                       const FastLutEntry &B) {
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[i] = block_element<F16>(blk.w, i);
+    return exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
+}
+
 // Operation-by-operation form (sub-normal block scales, out-of-range tensors): the
 // arithmetic of quantize_block in fos_quantize_common.h, rolled.
 template <int RULE, bool TWO_D, bool F16 = false>
@@ -402,10 +468,13 @@ __device__ __attribute__((noinline)) BlockOut generic_block_sr(Block16 blk, Quan
 // and fq * s * amax stays exact with the 11 significant bits of an fp16 maximum (2 + 4 + 11 <= 24).
 // PRODUCT: the MSE shortcut in its product form (bf16 elements, 1x16 blocks, round to nearest; the table built
 // with make_lut_entry<true>).
-template <int RULE, bool TWO_D, bool SR, bool F16 = false, bool PRODUCT = false>
+// SPREAD: a block whose shortcut is inconclusive is not evaluated here; it comes back as the first candidate
+// with `req` filled in, for exact_pick_b_spread at a point where the whole wavefront is together.
+template <int RULE, bool TWO_D, bool SR, bool F16 = false, bool PRODUCT = false, bool SPREAD = false>
 FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantConsts &k, float enc, float rq,
                                               bool in_range, const FastLutEntry *lut, uint64_t seed, uint64_t offset,
-                                              uint64_t blkid) {
+                                              uint64_t blkid, ExactRequest *req = nullptr) {
+    static_assert(!SPREAD || (!TWO_D && (RULE == FOS_RULE_MSE || RULE == FOS_RULE_MAE)), "spread evaluation: 1x16 blocks, summing rules");
     static_assert(!F16 || (!TWO_D && !SR), "fp16 elements: 1x16 blocks, round to nearest");
     static_assert(!PRODUCT || (RULE == FOS_RULE_MSE && !TWO_D && !SR && !F16), "product form: MSE, 1x16, bf16, round to nearest");
     constexpr bool STATIC = (RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4);
@@ -490,7 +559,12 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                     if (SHORTCUT && TWO_D) tie = row16_max(tie ? 0.0f : 1.0f) == 0.0f;
                     if (tie) pickB = false;
                     else if (k.exact_ok) {
-                        if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
+                        if constexpr (SPREAD) {
+                            req->wanted = true;
+                            req->b0 = b0;
+                            req->b1 = b1;
+                            req->sB = s4;
+                        } else if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
                         else pickB = exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
                     } else return generic_block_sr<RULE, TWO_D>(blk, k, seed, offset, blkid);  // e.g. the unbiased style's divisor
                 }
@@ -562,7 +636,12 @@ FOS_DEVICE BlockOut quantize_block_nvfp4_fast(const Block16 &blk, const QuantCon
                 }
                 if (tie) pickB = false;
                 else if (k.exact_ok) {
-                    if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
+                    if constexpr (SPREAD) {
+                        req->wanted = true;
+                        req->b0 = b0;
+                        req->b1 = b1;
+                        req->sB = s4;
+                    } else if constexpr (TWO_D) pickB = exact_pick_b<RULE, TWO_D>(blk, a0, a1, b0, b1, A, B);
                     else pickB = exact_pick_b_1d<RULE>(x, a0, a1, b0, b1, A, B);
                 } else return generic_block<RULE, TWO_D, F16>(blk, k);
             }

@@ -153,6 +153,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     // per wavefront: 4 scale tiles x 128 bytes (pseudo-quantize: the 2 KiB of a step's output instead)
     __shared__ __attribute__((aligned(16))) uint32_t sf_stage[4][PSEUDO ? 512 : 128];
     __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
+    // undecided blocks are evaluated exactly one at a time, spread over the wavefront (whole tiles only: every
+    // lane takes part); per wavefront 16 words of staging
+    constexpr bool kSpread = FULL && !IF4 && (RULE == FOS_RULE_MSE || RULE == FOS_RULE_MAE);
+    __shared__ __attribute__((aligned(16))) uint32_t exact_stage[4][kSpread ? 16 : 4];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t sf_cols = p.cols_p >> 4;
@@ -261,8 +265,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         BlockOut o{0u, 0u, 0u};
         if (!padding_step) {
             if constexpr (IF4) o = quantize_block_if4_mse<false>(b, k, enc_fast, rq, in_range, lut);
-            else o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
-                                                                          (uint64_t)(row * sf_cols + t.cb));
+            else if constexpr (kSpread) {
+                ExactRequest req;
+                o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct, true>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                                                                                    (uint64_t)(row * sf_cols + t.cb), &req);
+                const uint64_t asking = __builtin_amdgcn_ballot_w64(req.wanted);
+                if (asking != 0) {
+                    // a few lanes (what data brings: one wavefront step in ten has one): one block at a time across the
+                    // wavefront; many lanes (a tensor outside the shortcuts' range: all of them): every lane its own
+                    bool pick_second = false;
+                    if (__builtin_popcountll(asking) <= 6)
+                        pick_second = exact_pick_b_spread<RULE, F16>(req.wanted, b, o.c0, o.c1, req.b0, req.b1, lut[o.s & 0x7fu],
+                                                                     lut[req.sB & 0x7fu], exact_stage[wave]);
+                    else if (req.wanted)
+                        pick_second = exact_pick_b_1d_packed<RULE, F16>(b, o.c0, o.c1, req.b0, req.b1, lut[o.s & 0x7fu], lut[req.sB & 0x7fu]);
+                    if (req.wanted && pick_second) o = BlockOut{req.b0, req.b1, req.sB};
+                }
+            } else o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                                                                                 (uint64_t)(row * sf_cols + t.cb));
         }
         if (PSEUDO) {
             uint32_t w[8];
