@@ -3,7 +3,7 @@
 
 The library is the only implementation: there is no CPU or eager fallback.  Loading
 fails loudly when the shared object is missing; build it with
-``python -m fouroversix_amd.build``.
+``python fouroversix_amd/build.py``.
 """
 
 from __future__ import annotations
@@ -35,6 +35,7 @@ EXPORTS = (
     "fos_gemm_nvfp4",
     "fos_gemm_nvfp4_amax",
     "fos_gemm_nvfp4_amax_out",
+    "fos_gemm_nvfp4_linear",
     "fos_gemm_mxfp4",
     "fos_gemm_alpha",
     "fos_padded_cols_for",
@@ -56,7 +57,7 @@ def lib() -> ctypes.CDLL:
     if not os.path.exists(LIB_PATH):
         msg = (
             f"{LIB_PATH} not found: the gfx950 library has not been built "
-            "(run `python -m fouroversix_amd.build`); there is no fallback path"
+            "(run `python fouroversix_amd/build.py`); there is no fallback path"
         )
         raise NativeLibraryError(msg)
     L = ctypes.CDLL(LIB_PATH)
@@ -91,6 +92,8 @@ def lib() -> ctypes.CDLL:
     L.fos_gemm_nvfp4_amax.restype = i32
     L.fos_gemm_nvfp4_amax_out.argtypes = [vp, vp, vp, vp, vp, vp, dbl, i64, i64, i64, vp, i32, i64, vp, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4_amax_out.restype = i32
+    L.fos_gemm_nvfp4_linear.argtypes = [vp, vp, vp, vp, vp, vp, dbl, i64, i64, i64, vp, i32, i64, vp, vp, vp, ctypes.c_size_t, vp]
+    L.fos_gemm_nvfp4_linear.restype = i32
     L.fos_gemm_alpha.argtypes = [vp, vp, dbl, vp, vp]
     L.fos_gemm_alpha.restype = i32
     L.fos_gemm_mxfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp]

@@ -1,7 +1,9 @@
 """Build the gfx950 shared library (``libfouroversix_hip.so``) with hipcc, and the PyTorch
 binding on top of its C ABI (``_C.so``: host C++ only, compiled with g++).
 
-    python -m fouroversix_amd.build [--force]
+    python fouroversix_amd/build.py [--force]
+
+(run as a script: importing the package needs the libraries this builds)
 
 hipcc cross-compiles for gfx950 without a GPU.  The flags matter for bit-exactness:
 no fp contraction (fused multiply-adds only where the source spells them), correctly

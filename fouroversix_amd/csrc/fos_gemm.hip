@@ -56,6 +56,7 @@ struct GemmParams {
     const float *amax_a, *amax_b;
     float inv_den;
     void *D;
+    const void *bias;          // optional: N values of the output type, added to the rounded product and rounded again
     float *d_amax;             // optional: max|D| as stored is folded into d_amax[0] (unsigned atomic max on the bits)
     int64_t M, N, K, ldd;
     int tiles_m, tiles_n;
@@ -71,28 +72,79 @@ FOS_DEVICE float load_alpha(const GemmParams &p) {
     return p.alpha ? *p.alpha : (*p.amax_a * *p.amax_b) * p.inv_den;
 }
 
-// max|D| for the caller that quantizes D next: `vmax` is the largest |alpha * acc| this lane
-// stored (0 for a lane that stored nothing).  Rounding to the output type is monotonic, so
-// the rounded maximum is the maximum of the rounded values.  At most one vector atomic per
-// wavefront on the unsigned image of the value (non-negative floats order like their bits);
+// One value of the result as stored: alpha * acc rounded to the output type (16 bits returned).
+template <bool OUT_BF16>
+FOS_DEVICE uint32_t round_out(float v) {
+    if (OUT_BF16) {
+        uint32_t u = f2u(v);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return u >> 16;
+    }
+    // (v is a product already rounded to fp32 -- the reference's epilogue multiplies in fp32, then converts -- and
+    // must stay one: left to itself the compiler folds the multiplication into the conversion, v_fma_mixlo_f16,
+    // which rounds the exact product once and differs from the two roundings in one output in 10^5)
+    asm("" : "+v"(v));
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
+}
+template <bool OUT_BF16>
+FOS_DEVICE float widen_out(uint32_t bits) {
+    if (OUT_BF16) return u2f(bits << 16);
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+
+// Four consecutive outputs (columns n .. n + 3, n % 4 == 0) from their scaled accumulators: rounded to the output
+// type, and with a bias rounded, added to bias[n ..] in fp32 and rounded again -- the two roundings of the
+// reference's `out + bias` on the GEMM's result (src/fouroversix/model/modules/linear.py:83-92).  The magnitude
+// bits of what goes into the last rounding are folded into `umax` as unsigned integers, which order finite
+// values, infinity and NaN (largest) alike: a NaN in the output ends up as the recorded maximum, as it does
+// in the reference's x.abs().max().
+template <bool OUT_BF16>
+FOS_DEVICE uint32_t finish_output(float f, bool with_bias, uint32_t bias16, uint32_t &umax) {
+    if (with_bias) f = widen_out<OUT_BF16>(round_out<OUT_BF16>(f)) + widen_out<OUT_BF16>(bias16);
+    const uint32_t mag = f2u(f) & 0x7fffffffu;
+    umax = mag > umax ? mag : umax;
+    return round_out<OUT_BF16>(f);
+}
+template <bool OUT_BF16>
+FOS_DEVICE uint2 pack_outputs(const float *v, const void *bias, int64_t n, uint32_t &umax) {
+    uint2 bw = make_uint2(0u, 0u);
+    if (bias) bw = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(bias) + n);
+    const uint32_t o0 = finish_output<OUT_BF16>(v[0], bias != nullptr, bw.x & 0xffffu, umax);
+    const uint32_t o1 = finish_output<OUT_BF16>(v[1], bias != nullptr, bw.x >> 16, umax);
+    const uint32_t o2 = finish_output<OUT_BF16>(v[2], bias != nullptr, bw.y & 0xffffu, umax);
+    const uint32_t o3 = finish_output<OUT_BF16>(v[3], bias != nullptr, bw.y >> 16, umax);
+    return make_uint2(o0 | (o1 << 16), o2 | (o3 << 16));
+}
+// ... two consecutive outputs (n % 2 == 0)
+template <bool OUT_BF16>
+FOS_DEVICE uint32_t pack_outputs2(float v0, float v1, const void *bias, int64_t n, uint32_t &umax) {
+    uint32_t bw = 0u;
+    if (bias) bw = *reinterpret_cast<const uint32_t *>(static_cast<const uint16_t *>(bias) + n);
+    const uint32_t o0 = finish_output<OUT_BF16>(v0, bias != nullptr, bw & 0xffffu, umax);
+    const uint32_t o1 = finish_output<OUT_BF16>(v1, bias != nullptr, bw >> 16, umax);
+    return o0 | (o1 << 16);
+}
+
+// max|D| for the caller that quantizes D next: `umax` holds the magnitude bits of the largest value this
+// lane stored, before its rounding to the output type (0 for a lane that stored nothing).  Rounding is
+// monotonic, so the rounded maximum is the maximum of the rounded values.  At most one vector atomic per
+// wavefront on the unsigned image of the value (non-negative floats order like their bits, NaN above all);
 // every lane of the wavefront must call it.
 template <bool OUT_BF16>
-FOS_DEVICE void fold_amax(float *d_amax, float vmax) {
-    float r;
-    if (OUT_BF16) {
-        uint32_t u = f2u(vmax);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        r = u2f(u & 0xffff0000u);
-    } else {
-        r = (float)(_Float16)vmax;
-    }
+FOS_DEVICE void fold_amax(float *d_amax, uint32_t umax) {
+    uint32_t r;
+    if (umax > 0x7f800000u) r = 0x7fc00000u;
+    else r = f2u(widen_out<OUT_BF16>(round_out<OUT_BF16>(u2f(umax))));
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) r = fmaxf(r, __shfl_xor(r, off));
+    for (int off = 32; off >= 1; off >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)r, off);
+        r = other > r ? other : r;
+    }
     // (the atomics of a launch all go to one address and are served one after the other: a
     // wavefront first looks whether its value would change anything -- only the first few do)
     if ((threadIdx.x & 63) == 0) {
         unsigned int *word = reinterpret_cast<unsigned int *>(d_amax);
-        if (f2u(r) > __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(word, f2u(r));
+        if (r > __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(word, r);
     }
 }
 
@@ -365,28 +417,18 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     __syncthreads();  // every wavefront is done reading the A buffers
     uint8_t *epi = reinterpret_cast<uint8_t *>(lds) + wave * 32 * kEpiPitch;
     constexpr int kLanesPerRow = kRowBytes / 16, kRowsPerPass = 64 / kLanesPerRow;
-    float vmax = 0.0f;
+    uint32_t umax = 0u;
 #pragma unroll
     for (int i = 0; i < WM; ++i) {
 #pragma unroll
         for (int j = 0; j < WN; ++j) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                uint16_t o[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float v = alpha * acc[i][j][4 * g + e];
-                    vmax = fmaxf(vmax, fabsf(v));
-                    if (OUT_BF16) {
-                        uint32_t u = f2u(v);
-                        u += 0x7fffu + ((u >> 16) & 1u);
-                        o[e] = (uint16_t)(u >> 16);
-                    } else {
-                        o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
-                    }
-                }
-                *reinterpret_cast<uint2 *>(epi + (lane & 31) * kEpiPitch + (j * 32 + 8 * g + 4 * (lane >> 5)) * 2) =
-                    make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
+                const float v[4] = {alpha * acc[i][j][4 * g], alpha * acc[i][j][4 * g + 1], alpha * acc[i][j][4 * g + 2],
+                                    alpha * acc[i][j][4 * g + 3]};
+                const int nl = j * 32 + 8 * g + 4 * (lane >> 5);  // column inside the wavefront's strip
+                *reinterpret_cast<uint2 *>(epi + (lane & 31) * kEpiPitch + nl * 2) =
+                    pack_outputs<OUT_BF16>(v, p.bias, n0 + wn * WN * 32 + nl, umax);
             }
         }
         // (LDS operations of one wavefront complete in order: its own writes are visible to its reads)
@@ -403,7 +445,7 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     }
-    if (p.d_amax) fold_amax<OUT_BF16>(p.d_amax, vmax);
+    if (p.d_amax) fold_amax<OUT_BF16>(p.d_amax, umax);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -720,17 +762,7 @@ __global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1
     constexpr int kGroups = R == 2 ? 1 : R / 4;
     float *P = OUT == kOutPartial ? p.partials + (int64_t)blockIdx.y * p.M * p.N : nullptr;
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
-    float vmax = 0.0f;
-    auto to16 = [&](float v) -> uint32_t {
-        v *= alpha;
-        vmax = fmaxf(vmax, fabsf(v));
-        if (OUT == kOutBF16) {
-            uint32_t u = f2u(v);
-            u += 0x7fffu + ((u >> 16) & 1u);
-            return u >> 16;
-        }
-        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)v);
-    };
+    uint32_t umax = 0u;
 #pragma unroll
     for (int c = 0; c < kGroups; ++c) {
         const int c4 = R == 2 ? (wave >> 1) : wave * (R / 4) + c;  // group of four columns: c4 = (i WN + t) 4 + g
@@ -739,17 +771,22 @@ __global__ __launch_bounds__(64 * skinny_waves(WN), (WN == 2 && MT == 2) ? 2 : 1
         if (m >= p.M) continue;
         const int64_t n = n128 + 32 * g + r0 + 8 * t + 4 * h + (R == 2 ? (wave & 1) * 2 : 0);
         if constexpr (R == 2) {
-            if (OUT == kOutPartial) *reinterpret_cast<float2 *>(P + (int64_t)m * p.N + n) = make_float2(mine[0], mine[1]);
-            else *reinterpret_cast<uint32_t *>(D + (int64_t)m * p.ldd + n) = to16(mine[0]) | (to16(mine[1]) << 16);
+            if (OUT == kOutPartial) {
+                *reinterpret_cast<float2 *>(P + (int64_t)m * p.N + n) = make_float2(mine[0], mine[1]);
+            } else {
+                *reinterpret_cast<uint32_t *>(D + (int64_t)m * p.ldd + n) =
+                    pack_outputs2<OUT == kOutBF16>(alpha * mine[0], alpha * mine[1], p.bias, n, umax);
+            }
         } else {
-            if (OUT == kOutPartial)
+            if (OUT == kOutPartial) {
                 *reinterpret_cast<float4 *>(P + (int64_t)m * p.N + n) = make_float4(mine[4 * c], mine[4 * c + 1], mine[4 * c + 2], mine[4 * c + 3]);
-            else
-                *reinterpret_cast<uint2 *>(D + (int64_t)m * p.ldd + n) =
-                    make_uint2(to16(mine[4 * c]) | (to16(mine[4 * c + 1]) << 16), to16(mine[4 * c + 2]) | (to16(mine[4 * c + 3]) << 16));
+            } else {
+                const float v[4] = {alpha * mine[4 * c], alpha * mine[4 * c + 1], alpha * mine[4 * c + 2], alpha * mine[4 * c + 3]};
+                *reinterpret_cast<uint2 *>(D + (int64_t)m * p.ldd + n) = pack_outputs<OUT == kOutBF16>(v, p.bias, n, umax);
+            }
         }
     }
-    if (OUT != kOutPartial && p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, vmax);
+    if (OUT != kOutPartial && p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, umax);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -911,27 +948,18 @@ __global__ __launch_bounds__(512) void gemm_nvfp4_decode_kernel(const GemmParams
         return;
     }
     uint16_t *D = reinterpret_cast<uint16_t *>(p.D);
-    float vmax = 0.0f;
+    uint32_t umax = 0u;
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-        uint16_t o[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float v = alpha * acc[b][e];
-            if (row_ok) vmax = fmaxf(vmax, fabsf(v));
-            if (OUT == kOutBF16) {
-                uint32_t u = f2u(v);
-                u += 0x7fffu + ((u >> 16) & 1u);
-                o[e] = (uint16_t)(u >> 16);
-            } else {
-                o[e] = __builtin_bit_cast(uint16_t, (_Float16)v);
-            }
+        const float v[4] = {alpha * acc[b][0], alpha * acc[b][1], alpha * acc[b][2], alpha * acc[b][3]};
+        uint32_t um = 0u;
+        const uint2 o = pack_outputs<OUT == kOutBF16>(v, p.bias, n_out + 32 * b, um);
+        if (row_ok) {
+            umax = um > umax ? um : umax;
+            *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n_out + 32 * b) = o;
         }
-        if (row_ok)
-            *reinterpret_cast<uint2 *>(D + (int64_t)c * p.ldd + n_out + 32 * b) =
-                make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
     }
-    if (p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, vmax);
+    if (p.d_amax) fold_amax<OUT == kOutBF16>(p.d_amax, umax);
 }
 
 // D = alpha * (sum of the split-K partial tiles, in split order), 4 consecutive n per thread.
@@ -951,24 +979,10 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
     }
     const float alpha = load_alpha(p);
     const float v[4] = {alpha * s.x, alpha * s.y, alpha * s.z, alpha * s.w};
-    uint16_t o[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        if (OUT_BF16) {
-            uint32_t u = f2u(v[e]);
-            u += 0x7fffu + ((u >> 16) & 1u);
-            o[e] = (uint16_t)(u >> 16);
-        } else {
-            o[e] = __builtin_bit_cast(uint16_t, (_Float16)v[e]);
-        }
-    }
-    if (mine)
-        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.D) + m * p.ldd + n) =
-            make_uint2(o[0] | ((uint32_t)o[1] << 16), o[2] | ((uint32_t)o[3] << 16));
-    if (p.d_amax) {
-        const float vmax = mine ? fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))) : 0.0f;
-        fold_amax<OUT_BF16>(p.d_amax, vmax);
-    }
+    uint32_t um = 0u;
+    const uint2 o = pack_outputs<OUT_BF16>(v, p.bias, n, um);
+    if (mine) *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.D) + m * p.ldd + n) = o;
+    if (p.d_amax) fold_amax<OUT_BF16>(p.d_amax, mine ? um : 0u);
 }
 
 template <int WAVES_M, int WAVES_N, int WM, int WN>
@@ -1143,10 +1157,10 @@ extern "C" size_t fos_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
 
 static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
                            const float *alpha, const float *amax_a, const float *amax_b, double denominator,
-                           int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, float *d_amax,
+                           int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, const void *bias, float *d_amax,
                            void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!A || !B || !sfA || !sfB || !D) return FOS_E_NULL_POINTER;
-    if ((uintptr_t)d_amax & 3) return FOS_E_BAD_ALIGNMENT;
+    if (((uintptr_t)d_amax & 3) || ((uintptr_t)bias & 7)) return FOS_E_BAD_ALIGNMENT;
     if (!alpha && (!amax_a || !amax_b)) return FOS_E_NULL_POINTER;
     if (!alpha && (((uintptr_t)amax_a & 3) || ((uintptr_t)amax_b & 3))) return FOS_E_BAD_ALIGNMENT;
     if (M <= 0 || N <= 0 || K <= 0 || (M > 128 && M % 128 != 0) || N % 128 != 0 || K % 64 != 0 || ldd < N) return FOS_E_BAD_SHAPE;
@@ -1157,7 +1171,7 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
         return FOS_E_BAD_ALIGNMENT;
     if ((M / 128) * (N / 128) > 0x7fffffffLL || K > (1LL << 22)) return FOS_E_BAD_SHAPE;  // a 256-row panel of packed codes stays below 2^31 bytes (32-bit buffer offsets)
     GemmParams p;
-    p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D; p.d_amax = d_amax;
+    p.A = A; p.B = B; p.sfA = sfA; p.sfB = sfB; p.alpha = alpha; p.D = D; p.bias = bias; p.d_amax = d_amax;
     p.amax_a = amax_a; p.amax_b = amax_b; p.inv_den = alpha ? 0.0f : (float)(1.0 / denominator);
     p.M = M; p.N = N; p.K = K; p.ldd = ldd;
     hipStream_t s = (hipStream_t)stream;
@@ -1198,7 +1212,7 @@ extern "C" int fos_gemm_nvfp4(const uint8_t *A, const uint8_t *B, const uint8_t 
                               void *D, int out_type, int64_t ldd,
                               void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!alpha) return FOS_E_NULL_POINTER;
-    return gemm_nvfp4_impl(A, B, sfA, sfB, alpha, nullptr, nullptr, 1.0, M, N, K, D, out_type, ldd, nullptr, workspace,
+    return gemm_nvfp4_impl(A, B, sfA, sfB, alpha, nullptr, nullptr, 1.0, M, N, K, D, out_type, ldd, nullptr, nullptr, workspace,
                            workspace_bytes, stream);
 }
 
@@ -1208,7 +1222,7 @@ extern "C" int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uin
                                    void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!amax_a || !amax_b) return FOS_E_NULL_POINTER;
     if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
-    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, nullptr, workspace,
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, nullptr, nullptr, workspace,
                            workspace_bytes, stream);
 }
 
@@ -1218,6 +1232,16 @@ extern "C" int fos_gemm_nvfp4_amax_out(const uint8_t *A, const uint8_t *B, const
                                        void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!amax_a || !amax_b || !d_amax) return FOS_E_NULL_POINTER;
     if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
-    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, d_amax, workspace,
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, nullptr, d_amax, workspace,
+                           workspace_bytes, stream);
+}
+
+extern "C" int fos_gemm_nvfp4_linear(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                                     const float *amax_a, const float *amax_b, double denominator,
+                                     int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, const void *bias,
+                                     float *d_amax, void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!amax_a || !amax_b) return FOS_E_NULL_POINTER;
+    if (!(denominator > 0.0)) return FOS_E_BAD_SHAPE;
+    return gemm_nvfp4_impl(A, B, sfA, sfB, nullptr, amax_a, amax_b, denominator, M, N, K, D, out_type, ldd, bias, d_amax, workspace,
                            workspace_bytes, stream);
 }

@@ -197,7 +197,7 @@ void check_gemm_operands(const Tensor &a, const Tensor &b, const Tensor &a_sf, c
 // One GEMM launch.  alpha, or (amax_a, amax_b, denominator) for the output scale formed in the kernel;
 // with the latter, d_amax (device f32[1], zero or an earlier maximum) receives max|out|.
 Tensor gemm_launch(const Tensor &a, const Tensor &b, const Tensor &a_sf, const Tensor &b_sf, const Tensor *alpha, const Tensor *amax_a,
-                   const Tensor *amax_b, double denominator, at::ScalarType out_dtype, const Tensor *d_amax) {
+                   const Tensor *amax_b, double denominator, at::ScalarType out_dtype, const Tensor *d_amax, const Tensor *bias = nullptr) {
     const int64_t m = a.size(0), n = b.size(0), k = a.size(1) * 2;
     Tensor out = at::empty({m, n}, a.options().dtype(out_dtype));
     const size_t ws_bytes = fos_gemm_workspace_bytes(m, n, k);
@@ -213,10 +213,16 @@ Tensor gemm_launch(const Tensor &a, const Tensor &b, const Tensor &a_sf, const T
     int rc;
     if (alpha) {
         rc = fos_gemm_nvfp4(A, B, sA, sB, alpha->data_ptr<float>(), m, n, k, out.data_ptr(), out_type, n, wsp, ws_bytes, stream);
-    } else if (d_amax) {
-        require_gpu(*d_amax, "d_amax");
-        rc = fos_gemm_nvfp4_amax_out(A, B, sA, sB, amax_a->data_ptr<float>(), amax_b->data_ptr<float>(), denominator, m, n, k,
-                                     out.data_ptr(), out_type, n, d_amax->data_ptr<float>(), wsp, ws_bytes, stream);
+    } else if (d_amax || bias) {
+        if (d_amax) require_gpu(*d_amax, "d_amax");
+        if (bias) {
+            require_gpu(*bias, "bias");
+            TORCH_CHECK(bias->scalar_type() == out_dtype && bias->dim() == 1 && bias->size(0) == n && bias->is_contiguous(),
+                        "gemm: bias must be a contiguous [N] tensor of the output type");
+        }
+        rc = fos_gemm_nvfp4_linear(A, B, sA, sB, amax_a->data_ptr<float>(), amax_b->data_ptr<float>(), denominator, m, n, k,
+                                   out.data_ptr(), out_type, n, bias ? bias->data_ptr() : nullptr,
+                                   d_amax ? d_amax->data_ptr<float>() : nullptr, wsp, ws_bytes, stream);
     } else {
         rc = fos_gemm_nvfp4_amax(A, B, sA, sB, amax_a->data_ptr<float>(), amax_b->data_ptr<float>(), denominator, m, n, k,
                                  out.data_ptr(), out_type, n, wsp, ws_bytes, stream);
@@ -241,8 +247,10 @@ Tensor gemm_nvfp4_fp16(const Tensor &a, const Tensor &b, const Tensor &a_sf, con
 // The NVFP4 GEMM with the output scale (amax_a * amax_b) * f32(1 / denominator) formed in the kernel: one launch
 // less than alpha + GEMM, same result.  `checked`: the operands are the members of two QuantizedTensors on
 // one GPU (the frontend has looked): only the shapes are compared.
+// `bias` ([N], output type): added to the rounded product and rounded again, as `out + bias` would.
 Tensor gemm_nvfp4_amax(const Tensor &a, const Tensor &b, const Tensor &a_sf, const Tensor &b_sf, const Tensor &amax_a, const Tensor &amax_b,
-                       double denominator, at::ScalarType out_dtype, const c10::optional<Tensor> &d_amax, bool checked) {
+                       double denominator, at::ScalarType out_dtype, const c10::optional<Tensor> &d_amax, bool checked,
+                       const c10::optional<Tensor> &bias) {
     if (checked) {
         TORCH_CHECK(a.size(1) == b.size(1), "Inner dims mismatch: ", a.size(1) * 2, " vs ", b.size(1) * 2);
     } else {
@@ -250,7 +258,8 @@ Tensor gemm_nvfp4_amax(const Tensor &a, const Tensor &b, const Tensor &a_sf, con
         const char *names[2] = {"amax_a", "amax_b"};
         check_gemm_operands(a, b, a_sf, b_sf, scales, 2, names);
     }
-    return gemm_launch(a, b, a_sf, b_sf, nullptr, &amax_a, &amax_b, denominator, out_dtype, d_amax.has_value() ? &*d_amax : nullptr);
+    return gemm_launch(a, b, a_sf, b_sf, nullptr, &amax_a, &amax_b, denominator, out_dtype, d_amax.has_value() ? &*d_amax : nullptr,
+                       bias.has_value() ? &*bias : nullptr);
 }
 
 // alpha[0] = (amax_a * amax_b) * f32(1 / denominator) on the device
@@ -318,7 +327,7 @@ TORCH_LIBRARY(fouroversix, m) {
     m.def("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");
     m.def(
         "gemm_nvfp4_amax(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor amax_a, Tensor amax_b, float denominator, "
-        "ScalarType out_dtype, Tensor(a!)? d_amax, bool checked=False) -> Tensor");
+        "ScalarType out_dtype, Tensor(a!)? d_amax, bool checked=False, Tensor? bias=None) -> Tensor");
     m.def(
         "dequantize(Tensor values, Tensor scale_factors, Tensor amax, int dtype, int sf_layout, float divisor, "
         "int rows, int cols, ScalarType out_dtype, bool f32_intermediate=False) -> Tensor");

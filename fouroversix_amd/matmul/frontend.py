@@ -171,8 +171,12 @@ def quantized_matmul(
 
     ``emit_amax=True`` (no counterpart in the reference) lets the NVFP4 GEMM record max|out| while
     it stores it and attaches it to the result (``known_amax``), so that a following
-    ``quantize(out)`` skips its own reduction pass over the tensor."""
+    ``quantize(out)`` skips its own reduction pass over the tensor.  ``bias=`` (a ``[N]`` tensor, no
+    counterpart either) returns ``out + bias``: the NVFP4 GEMM adds it in its epilogue with the two
+    roundings of that expression, and the recorded maximum is then that of the sum.  The tag is dropped
+    only by writes that torch counts (see ``attach_known_amax``)."""
     emit_amax = bool(kwargs.pop("emit_amax", False))
+    bias = kwargs.pop("bias", None)
     del kwargs
     if isinstance(input, torch.Tensor):
         input = quantize(input, input_config)
@@ -192,16 +196,28 @@ def quantized_matmul(
         and (out_dtype is DataType.bfloat16 or out_dtype is DataType.float16)
         and not torch.compiler.is_compiling()
     ):
-        d_amax = _fresh_amax_word(ra[6]) if emit_amax else None
+        torch_dtype = torch.bfloat16 if out_dtype is DataType.bfloat16 else torch.float16
+        fused_bias = (
+            bias is not None
+            and bias.dtype == torch_dtype
+            and bias.dim() == 1
+            and bias.shape[0] == rb[0].shape[0]  # (no row padding of the weight between the bias and the product)
+            and bias.device == ra[6]
+            and bias.is_contiguous()
+            and bias.data_ptr() % 8 == 0
+        )
+        d_amax = _fresh_amax_word(ra[6]) if emit_amax and (bias is None or fused_bias) else None
         out = ops.gemm_nvfp4_from_amax(
-            ra[4], rb[0], ra[1], rb[1], ra[2], rb[2], ra[5] * rb[5],
-            torch.bfloat16 if out_dtype is DataType.bfloat16 else torch.float16, d_amax, checked=True,
+            ra[4], rb[0], ra[1], rb[1], ra[2], rb[2], ra[5] * rb[5], torch_dtype, d_amax, True,
+            bias.detach() if fused_bias else None,
         )
         m, n = input.original_shape[0], other.original_shape[0]
         if out.shape[0] != m or out.shape[1] != n:
             out = out[:m, :n]  # (the padding is zeros: same maximum)
         if d_amax is not None:
             attach_known_amax(out, d_amax)
+        if bias is not None and not fused_bias:
+            out = out + bias
         return out
 
     if not is_supported(input, other, out_dtype=out_dtype):
@@ -213,7 +229,8 @@ def quantized_matmul(
                 dequantize(input, dtype=torch.float32), dequantize(other, dtype=torch.float32).T
             ).to(out_dtype.torch_dtype)
             out_shape = (input.original_shape[0], other.original_shape[0])
-            return out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
+            out = out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
+            return out if bias is None else out + bias
         if backend is None:
             msg = "No backend found that supports the given parameters"
         else:
@@ -228,7 +245,8 @@ def quantized_matmul(
             input.values, other.values, input.scale_factors, other.scale_factors, alpha,
             torch.bfloat16 if out_dtype == DataType.bfloat16 else torch.float16,
         )
-        return out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
+        out = out if tuple(out.shape) == out_shape else out[: out_shape[0], : out_shape[1]]
+        return out if bias is None else out + bias
 
     a_values = input.values
     m_orig = input.original_shape[0]
@@ -247,4 +265,4 @@ def quantized_matmul(
     out_shape = (input.original_shape[0], other.original_shape[0])
     if tuple(out.shape) != out_shape:
         out = out[: out_shape[0], : out_shape[1]]
-    return out
+    return out if bias is None else out + bias

@@ -50,18 +50,22 @@ def fp4_linear(
             amax_in = known_amax(input)
             if amax_in is not None and flat is not input:
                 attach_known_amax(flat, amax_in)
+            # (the bias goes into the GEMM's epilogue with the two roundings of `out + bias`; the recorded
+            # maximum is then that of the sum)
             out2d = quantized_matmul(
                 flat,
                 weight,
                 backend=config.matmul_backend,
                 input_config=config.get_activation_config(),
                 out_dtype=config.output_dtype,
-                emit_amax=config.emit_output_amax and bias is None,
+                emit_amax=config.emit_output_amax,
+                bias=bias,
             )
             out = out2d.reshape(*input.shape[:-1], weight.original_shape[0])
             amax_out = known_amax(out2d)
             if amax_out is not None and out is not out2d:
                 attach_known_amax(out, amax_out)
+            return out
     if bias is not None:
         out = out + bias
     return out

@@ -25,7 +25,7 @@ _EXT_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file_
 if not os.path.exists(_EXT_PATH):
     msg = (
         f"{_EXT_PATH} not found: the PyTorch binding has not been built "
-        "(run `python -m fouroversix_amd.build`); there is no fallback path"
+        "(run `python fouroversix_amd/build.py`); there is no fallback path"
     )
     raise nat.NativeLibraryError(msg)
 nat.lib()  # (the binding links against the C-ABI library next to it: fail with its message if that is missing)
@@ -96,12 +96,13 @@ def gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(a, b, a_sf, b_sf, alpha):
     return torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt.default(a, b, a_sf, b_sf, alpha)
 
 
-def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax=None, checked=False):
+def gemm_nvfp4_from_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax=None, checked=False, bias=None):
     """The NVFP4 GEMM with the output scale ``(amax_a * amax_b) * f32(1 / denominator)`` formed
     in the kernel (``fos_gemm_nvfp4_amax``): one launch less than alpha + GEMM, same result.
     ``d_amax`` (device f32[1] holding 0) additionally receives max|out|.  ``checked``: the operands are
-    the members of two QuantizedTensors on one GPU (the frontend has looked): only the shapes are compared."""
-    return _C.gemm_nvfp4_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax, checked)
+    the members of two QuantizedTensors on one GPU (the frontend has looked): only the shapes are compared.
+    ``bias`` ([N], output type) is added to the rounded product and the sum rounded again, as ``out + bias``."""
+    return _C.gemm_nvfp4_amax(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax, checked, bias)
 
 
 def gemm_alpha_into(amax_a, amax_b, denominator, alpha):
@@ -178,5 +179,5 @@ def _(x, transpose, rht):
 
 
 @torch.library.register_fake("fouroversix::gemm_nvfp4_amax")
-def _(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax, checked=False):
+def _(a, b, a_sf, b_sf, amax_a, amax_b, denominator, out_dtype, d_amax, checked=False, bias=None):
     return torch.empty(a.shape[0], b.shape[0], dtype=out_dtype, device=a.device)

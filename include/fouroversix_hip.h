@@ -203,7 +203,8 @@ int fos_gemm_nvfp4_amax(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, 
  * fos_gemm_nvfp4_amax that also folds max|D| -- of the values as stored, in the output type --
  * into d_amax[0] (device f32[1]): every wavefront does an unsigned atomic max on the value's
  * bits, so the caller sets d_amax[0] to 0 before the call (or leaves an earlier maximum there to
- * extend it).  The next layer's activation quantization can then take d_amax as its
+ * extend it).  A NaN among the outputs is recorded as NaN (its bits lie above every number's), as the
+ * reference's `x.abs().max()` would report it.  The next layer's activation quantization can then take d_amax as its
  * `amax` input (amax_is_input = 1) and skip its own pass over D.  No counterpart in the
  * reference, whose quantize op always reduces its input
  * (src/fouroversix/quantize/pytorch/reference.py:573-600).
@@ -212,6 +213,19 @@ int fos_gemm_nvfp4_amax_out(const uint8_t *A, const uint8_t *B, const uint8_t *s
                             const float *amax_a, const float *amax_b, double denominator,
                             int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, float *d_amax,
                             void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * The product of a linear layer in one launch: fos_gemm_nvfp4_amax_out with an optional bias (N values of
+ * the output type, 8-byte aligned, or NULL) and an optional d_amax (NULL: not recorded).  With a bias,
+ * D = RN(RN(alpha * acc) + bias[n]): the product rounded to the output type, then the sum rounded again --
+ * the two roundings of `out = quantized_matmul(...); out = out + bias` in the reference's layer
+ * (src/fouroversix/model/modules/linear.py:83-92) -- and d_amax receives max|D| of that sum, so that a layer
+ * with a bias hands its output maximum on like one without.
+ */
+int fos_gemm_nvfp4_linear(const uint8_t *A, const uint8_t *B, const uint8_t *sfA, const uint8_t *sfB,
+                          const float *amax_a, const float *amax_b, double denominator,
+                          int64_t M, int64_t N, int64_t K, void *D, int out_type, int64_t ldd, const void *bias,
+                          float *d_amax, void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
  * alpha[0] = (amax_a[0] * amax_b[0]) * f32(1 / denominator), in fp32 on the device: the

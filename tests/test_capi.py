@@ -13,12 +13,16 @@ HEADER = os.path.join(ROOT, "include", "fouroversix_hip.h")
 
 @pytest.fixture(scope="module")
 def native():
+    if not os.path.exists(os.path.join(ROOT, "fouroversix_amd", "libfouroversix_hip.so")):
+        # (the build script by path: importing the package needs the libraries it builds)
+        import importlib.util
+
+        spec = importlib.util.spec_from_file_location("fos_build", os.path.join(ROOT, "fouroversix_amd", "build.py"))
+        fos_build = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(fos_build)
+        fos_build.build()
     from fouroversix_amd import _native
 
-    if not os.path.exists(_native.LIB_PATH):
-        from fouroversix_amd.build import build
-
-        build()
     return _native
 
 

@@ -559,3 +559,43 @@ def test_decoder_layer_at_16384_tokens_through_quantize_model(oracle):
         ref, _ = oracle.gemm_nvfp4(ra.values[rows.numpy()], ra.scale_rows[rows.numpy()], rw.values[cols.numpy()],
                                    rw.scale_rows[cols.numpy()], oracle.gemm_alpha(ra, rw))
         check(bits16(out2[rows.cuda()][:, cols.cuda()]), ref, oracle, name)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize(("m", "n", "k"), [(16, 512, 1024), (5, 256, 2304), (48, 512, 2048), (100, 2048, 3328), (128, 1024, 8192),
+                                           (256, 384, 2368), (512, 512, 256), (2048, 1024, 512), (384, 256, 14336)])
+def test_bias_in_the_epilogue_equals_the_separate_addition(m, n, k, out_dtype):
+    """`quantized_matmul(..., bias=b)` = `quantized_matmul(...) + b` bit for bit (the product rounded to the
+    output type, the sum rounded again: reference src/fouroversix/model/modules/linear.py:83-92) in every
+    kernel of the plan -- 16-row, weight-streaming, tile and split-K reduction -- and the recorded maximum
+    is that of the sum."""
+    from fouroversix_amd.quantize import known_amax
+
+    a, b = make_input("randn", (m, k), 81).cuda(), make_input("weight", (n, k), 82).cuda()
+    qa, qb = fos.quantize(a), fos.quantize(b, fos.QuantizationConfig(block_scale_2d=True))
+    g = torch.Generator("cpu").manual_seed(83)
+    bias = (torch.randn(n, generator=g) * 0.3).to(out_dtype).cuda()
+    dt = fos.DataType.bfloat16 if out_dtype == torch.bfloat16 else fos.DataType.float16
+    plain = fos.quantized_matmul(qa, qb, out_dtype=dt)
+    fused = fos.quantized_matmul(qa, qb, out_dtype=dt, bias=bias, emit_amax=True)
+    assert torch.equal(fused, plain + bias)
+    amax = known_amax(fused)
+    assert amax is not None and float(amax) == float(fused.float().abs().max())
+    # a bias of another type, or on a weight whose rows were padded, is added separately: same values, no tag
+    other = fos.quantized_matmul(qa, qb, out_dtype=dt, bias=bias.float(), emit_amax=True)
+    assert torch.equal(other, plain + bias.float()) and known_amax(other) is None
+
+
+def test_recorded_maximum_of_an_output_with_nan_is_nan():
+    """The reference's `x.abs().max()` of a tensor that holds a NaN is NaN; the maximum the GEMM records
+    follows (the bits of a NaN lie above every number's in the unsigned comparison)."""
+    from fouroversix_amd.quantize import known_amax
+
+    a, b = make_input("randn", (256, 512), 84).cuda(), make_input("weight", (384, 512), 85).cuda()
+    qa, qb = fos.quantize(a), fos.quantize(b)
+    qa.amax = torch.full_like(qa.amax, float("nan"))  # alpha, and with it every output, is NaN
+    out = fos.quantized_matmul(qa, qb, emit_amax=True)
+    assert bool(torch.isnan(out).all())
+    assert bool(torch.isnan(known_amax(out)).all())
+    q = fos.quantize(out)
+    assert bool(torch.isnan(q.amax).all())
