@@ -230,6 +230,70 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const TransformPara
     write_partials<F16>(m, z, p.partials);
 }
 
+// fp32 input (the reference converts with `.float()` and multiplies by the fp32 matrix: a library matmul whose
+// summation order is not part of any interface, so the target is the product itself, to fp32 rounding).  One
+// thread per output group of 16: the butterfly in fp32 (four levels of additions: within 4 units in the last
+// place of the largest partial sum), fp32 out.  With transposition a wavefront's lanes take consecutive output
+// rows, i.e. consecutive columns of x, so that each of its 16 loads reads a contiguous run of one row of x.
+struct TransformParamsF32 {
+    const float *x;
+    int64_t rows, cols, ld;
+    float *y;
+    int64_t ldy;
+    uint32_t *partials;
+    int64_t out_rows, groups;  // output rows, groups of 16 per output row
+};
+
+template <bool TRANSPOSE, bool RHT>
+__global__ __launch_bounds__(kThreads) void transform_f32_kernel(const TransformParamsF32 p) {
+    __shared__ uint32_t smem[4];
+    uint32_t m = 0;
+    const int64_t n_units = p.out_rows * p.groups;
+    for (int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x; u < n_units; u += (int64_t)gridDim.x * kThreads) {
+        // transposed: consecutive units walk down the output rows (a column of groups at a time)
+        const int64_t r = TRANSPOSE ? u % p.out_rows : u / p.groups, g = TRANSPOSE ? u / p.out_rows : u % p.groups;
+        float v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int64_t c = g * 16 + i;  // column of y = (transposed) row of x
+            float e = 0.0f;
+            if (TRANSPOSE) { if (c < p.rows) e = p.x[c * p.ld + r]; }
+            else if (c < p.cols) e = p.x[r * p.ld + c];
+            v[i] = RHT && ((kRhtNegMask >> i) & 1u) ? -e : e;
+        }
+        if (RHT) {
+#pragma unroll
+            for (int len = 1; len < 16; len <<= 1) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if ((i & len) == 0) {
+                        const float a = v[i], b = v[i + len];
+                        v[i] = a + b;
+                        v[i + len] = a - b;
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = v[i] * 0.25f + 0.0f;
+        }
+        float4 *dst = reinterpret_cast<float4 *>(p.y + r * p.ldy + g * 16);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            dst[q] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t mag = f2u(v[4 * q + i]) & 0x7fffffffu;
+                m = mag > m ? mag : m;
+            }
+        }
+    }
+    m = block_max_u32(m, smem);
+    if (threadIdx.x == 0) {
+        p.partials[2 * blockIdx.x] = m;
+        p.partials[2 * blockIdx.x + 1] = 0u;
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void transform_amax_kernel(const uint32_t *__restrict__ partials, int n,
                                                                   float *__restrict__ amax) {
     __shared__ uint32_t smem[4];
@@ -248,12 +312,32 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
                              void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!x || !y || !amax) return FOS_E_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
-    if ((x_type != FOS_T_BF16 && x_type != FOS_T_F16) || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
+    if ((x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
     const bool f16 = x_type == FOS_T_F16;
     const int64_t out_cols = transpose ? rows : cols;
     // y is written in whole 16-element groups
     if (ldy < (out_cols + 15) / 16 * 16) return FOS_E_BAD_SHAPE;
     if (!workspace || workspace_bytes < fos_quantize_workspace_bytes(rows, cols)) return FOS_E_WORKSPACE;
+    if (x_type == FOS_T_F32) {
+        if (((uintptr_t)x & 3) || ((uintptr_t)y & 15) || (ldy % 4 != 0) || ((uintptr_t)workspace & 7) || ((uintptr_t)amax & 3))
+            return FOS_E_BAD_ALIGNMENT;
+        TransformParamsF32 q;
+        q.x = static_cast<const float *>(x);
+        q.rows = rows; q.cols = cols; q.ld = ld;
+        q.y = static_cast<float *>(y);
+        q.ldy = ldy;
+        q.partials = static_cast<uint32_t *>(workspace);
+        q.out_rows = transpose ? cols : rows;
+        q.groups = (out_cols + 15) / 16;
+        hipStream_t s32 = (hipStream_t)stream;
+        int64_t grid32 = (q.out_rows * q.groups + kThreads - 1) / kThreads;
+        if (grid32 > 1024) grid32 = 1024;  // pairs the workspace holds
+        if (transpose && rht) hipLaunchKernelGGL((transform_f32_kernel<true, true>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
+        else if (transpose) hipLaunchKernelGGL((transform_f32_kernel<true, false>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
+        else hipLaunchKernelGGL((transform_f32_kernel<false, true>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
+        hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s32, q.partials, (int)grid32, amax);
+        return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+    }
     if (((uintptr_t)x & 1) || ((uintptr_t)y & 15) || (ldy % 8 != 0) || ((uintptr_t)workspace & 7) || ((uintptr_t)amax & 3))
         return FOS_E_BAD_ALIGNMENT;
     TransformParams p;

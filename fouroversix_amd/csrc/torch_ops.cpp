@@ -132,8 +132,8 @@ Tensor pseudo_quantize(const Tensor &x, int64_t dtype, int64_t rule, int64_t rou
 
 // (y, amax): y = RHT(x^T) as the reference forms it before scaling, amax = max|y|
 std::tuple<Tensor, Tensor> transform(const Tensor &x_in, bool transpose, bool rht) {
-    TORCH_CHECK(x_in.dim() == 2 && (x_in.scalar_type() == at::kBFloat16 || x_in.scalar_type() == at::kHalf),
-                "transform: x must be a 2-D bfloat16 or float16 tensor");
+    TORCH_CHECK(x_in.dim() == 2 && (x_in.scalar_type() == at::kBFloat16 || x_in.scalar_type() == at::kHalf || x_in.scalar_type() == at::kFloat),
+                "transform: x must be a 2-D bfloat16, float16 or float32 tensor");
     require_gpu(x_in, "x");
     const Tensor x = x_in.stride(-1) == 1 ? x_in : x_in.contiguous();
     const int64_t rows = x.size(0), cols = x.size(1);

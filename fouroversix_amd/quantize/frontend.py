@@ -38,10 +38,6 @@ def unsupported_reason(x: torch.Tensor, config: QuantizationConfig) -> str | Non
         return f"input must live on the GPU, got {x.device}"
     if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         return f"input must be bfloat16, float16 or float32, got {x.dtype}"
-    if x.dtype == torch.float32 and (config.rht or config.transpose):
-        # (the reference's fp32 product with the Hadamard matrix is a library fp32 matmul, whose
-        # summation order is not fixed: there is nothing bit-exact to match)
-        return "rht and transpose take bfloat16 or float16 input, got float32"
     if config.dtype == DataType.mxfp4 and (config.block_scale_2d or config.round_style.is_stochastic):
         return "mxfp4 has kernels for 1x32 blocks with round-to-nearest only"
     if config.rht or config.transpose:

@@ -133,7 +133,7 @@ int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, i
  * Pre-transform of the training-side quantize options: y = x^T (transpose != 0) and / or
  * the 16-point random Hadamard transform of every group of 16 consecutive row elements
  * (rht != 0; fixed sign vector), written as a row-major matrix y of x's type (x_type
- * FOS_T_BF16 or FOS_T_F16; [cols, rows] when transposed, else [rows, cols]; leading dimension
+ * FOS_T_BF16, FOS_T_F16 or FOS_T_F32; [cols, rows] when transposed, else [rows, cols]; leading dimension
  * ldy), and amax[0] = max |y|.  Stands in
  * for the `x.T` / `x.reshape(-1, 16) @ had` / `abs().max()` steps of the reference
  * quantizer (src/fouroversix/quantize/pytorch/reference.py:567-578,
@@ -144,6 +144,9 @@ int fos_quantize_static(const void *x, int x_type, int64_t rows, int64_t cols, i
  * reference's zero padding, src/fouroversix/quantize/pytorch/backend.py:57-79), so with rht
  * the last group of a ragged width carries values in all 16 places.  x is read with 128-bit
  * loads when it is 16-byte aligned and ld a multiple of 8, element by element otherwise.
+ * FOS_T_F32 (ldy a multiple of 4): the reference's fp32 product with the Hadamard matrix is a library matmul
+ * whose summation order is not fixed; y equals the exact product to within four fp32 roundings of the
+ * largest partial sum of a group.
  * Same workspace as fos_quantize.
  */
 int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,

@@ -190,6 +190,17 @@ def transform(xb: np.ndarray, *, transpose=False, rht=False, x_type=0) -> np.nda
     (the reference pads to its block multiples before the transform,
     src/fouroversix/quantize/pytorch/backend.py:57-79), so with ``rht`` the result is a multiple
     of 16 wide."""
+    if x_type == 2:
+        # fp32 input: the reference's product is a library fp32 matmul (summation order not fixed); the target
+        # stated here is the exact product, formed in fp64 and rounded once to fp32
+        xf = np.asarray(xb, dtype=np.float32)
+        if transpose:
+            xf = np.ascontiguousarray(xf.T)
+        if rht:
+            if xf.shape[1] % 16:
+                xf = np.pad(xf, ((0, 0), (0, 16 - xf.shape[1] % 16)))
+            xf = (xf.astype(np.float64).reshape(-1, 16) @ rht_matrix().astype(np.float64)).astype(np.float32).reshape(xf.shape)
+        return xf
     xb = np.asarray(xb, dtype=np.uint16)
     if transpose:
         xb = np.ascontiguousarray(xb.T)
@@ -212,7 +223,6 @@ def quantize(x, *, dtype="nvfp4", scale_rule="mse", round_style="nearest",
     xb, x_type = input_bits(x)
     assert xb.ndim == 2
     if transpose or rht:
-        assert x_type in (0, 1), "transpose / rht: bf16 or fp16 input"
         xb = transform(xb, transpose=transpose, rht=rht, x_type=x_type)
     orig = tuple(int(v) for v in xb.shape)
     xp = np.ascontiguousarray(pad_bits(xb))

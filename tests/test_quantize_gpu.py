@@ -160,13 +160,41 @@ def test_fp32_and_fp16_inputs_other_paths(oracle):
         assert torch.equal(q2.values, q.values)
         assert fos.quantize(xt, fos.QuantizationConfig(dtype="mxfp4", scale_rule="static_6")).original_shape == (128, 128)
         for option in (dict(rht=True), dict(transpose=True)):
-            if t == torch.float32:
-                with pytest.raises(ValueError, match="bfloat16 or float16 input"):
-                    fos.quantize(xt, fos.QuantizationConfig(**option))
-            else:
-                assert fos.quantize(xt, fos.QuantizationConfig(**option)).original_shape == (128, 128)
+            assert fos.quantize(xt, fos.QuantizationConfig(**option)).original_shape == (128, 128)
     with pytest.raises(ValueError, match="bfloat16, float16 or float32"):
         fos.quantize(x.double().cuda())
+
+
+@pytest.mark.parametrize(("transpose", "rht"), [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("shape", [(256, 512), (100, 80), (130, 8)])
+def test_fp32_inputs_with_transpose_and_rht(oracle, shape, transpose, rht):
+    """fp32 tensors under the `transpose` / `rht` options (reference src/fouroversix/quantize/pytorch/reference.py:567-571:
+    `x.float()` times the fp32 Hadamard matrix, a library matmul whose summation order is not fixed).  Parity
+    with the reference is therefore to tolerance: the transformed tensor lies within 2^-21 |x| |H| of the exact
+    product (four fp32 roundings of partial sums; a plain transposition is exact), and the quantization of that
+    tensor is the oracle's, bit for bit."""
+    from fouroversix_amd.quantize import ops
+
+    g = torch.Generator("cpu").manual_seed(21)
+    x = torch.randn(*shape, generator=g) * torch.exp(torch.randn(shape[0], 1, generator=g))
+    y, amax = ops.transform(x.cuda(), transpose, rht)
+    y = y.cpu().numpy()
+    exact = oracle.transform(x.numpy(), transpose=transpose, rht=rht, x_type=2)
+    assert y.shape == exact.shape
+    if rht:
+        xt = x.numpy().T if transpose else x.numpy()
+        xt = np.pad(xt, ((0, 0), (0, -xt.shape[1] % 16)))
+        bound = np.repeat(np.abs(xt).astype(np.float64).reshape(-1, 16).sum(axis=1) * 0.25, 16).reshape(exact.shape) * 2.0**-21
+        assert (np.abs(y.astype(np.float64) - exact.astype(np.float64)) <= bound + 1e-45).all()
+    else:
+        assert np.array_equal(y, exact)
+    assert float(amax) == float(np.abs(y).max())
+    for cfg in (dict(scale_rule="mse"), dict(scale_rule="static_6", block_scale_2d=shape[0] % 16 == 0 and shape[1] % 16 == 0)):
+        q = fos.quantize(x.cuda(), fos.QuantizationConfig(transpose=transpose, rht=rht, **cfg))
+        ref = oracle.quantize(torch.from_numpy(y), **cfg)
+        assert q.original_shape == ((shape[1], shape[0]) if transpose else shape)
+        assert float(q.amax) == float(ref.amax)
+        assert np.array_equal(u8(q.values), ref.values) and np.array_equal(u8(q.scale_factors).reshape(-1), ref.scale_factors)
 
 
 WEIGHT_CASES = [(shape, "weight", cfg)
