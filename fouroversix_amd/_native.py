@@ -31,6 +31,8 @@ EXPORTS = (
     "fos_quantize",
     "fos_quantize_static",
     "fos_pseudo_quantize",
+    "fos_pseudo_quantize_keyed",
+    "fos_pseudo_quantize_is_fused",
     "fos_transform",
     "fos_gemm_nvfp4",
     "fos_gemm_nvfp4_amax",
@@ -84,6 +86,10 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize_static.restype = i32
     L.fos_pseudo_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i32, vp, sz, vp]
     L.fos_pseudo_quantize.restype = i32
+    L.fos_pseudo_quantize_keyed.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, vp, i64, vp, i32, vp, sz, vp]
+    L.fos_pseudo_quantize_keyed.restype = i32
+    L.fos_pseudo_quantize_is_fused.argtypes = [i32, i32, i32, i32, i32]
+    L.fos_pseudo_quantize_is_fused.restype = i32
     L.fos_transform.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, i64, vp, vp, sz, vp]
     L.fos_transform.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]

@@ -308,7 +308,7 @@ void dispatch_round(QuantParams &p, int round_style, bool two_d, bool aligned, h
             // inputs and inside the generic kernel's mapping otherwise
             if (two_d && aligned && !p.pseudo_out) launch_quantize_if4_mse_tiles(p, s);
             else if (two_d) launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, true>(p, aligned, s);
-            else if (aligned && !p.pseudo_out) launch_quantize_if4_mse_rows(p, s);
+            else if (aligned) launch_quantize_if4_mse_rows(p, s);
             else launch_quantize<true, DT, RULE, FOS_ROUND_NEAREST, false>(p, aligned, s);
         } else {
             dispatch_2d<DT, RULE, FOS_ROUND_NEAREST>(p, two_d, aligned, s);
@@ -364,6 +364,21 @@ static bool stream_is_capturing(hipStream_t s) {
     return status != hipStreamCaptureStatusNone;
 }
 
+// Which combinations the fused quantize -> dequantize kernels cover (alignment aside): NVFP4 with round to
+// nearest (bf16 with either block shape, fp16 with 1x16 blocks), NVFP4 with a stochastic style on bf16 and
+// 1x16 blocks (the unbiased style with the rules whose decision the streaming kernel makes), IF4 with the MSE
+// rule on bf16, round to nearest, 1x16 blocks.
+extern "C" int fos_pseudo_quantize_is_fused(int x_type, int dtype, int rule, int round_style, int block2d) {
+    const bool rtn = round_style == FOS_ROUND_NEAREST;
+    if (dtype == FOS_DTYPE_NVFP4 && rtn) return x_type == FOS_T_BF16 || (x_type == FOS_T_F16 && !block2d);
+    if (x_type != FOS_T_BF16 || block2d) return 0;
+    if (dtype == FOS_DTYPE_IF4) return rtn && rule == FOS_RULE_MSE;
+    if (dtype != FOS_DTYPE_NVFP4) return 0;
+    if (round_style == FOS_ROUND_STOCHASTIC) return 1;
+    return round_style == FOS_ROUND_STOCHASTIC_UNBIASED &&
+           (rule == FOS_RULE_MSE || rule == FOS_RULE_STATIC_6 || rule == FOS_RULE_STATIC_4);
+}
+
 // Shared body of fos_quantize and fos_pseudo_quantize (pseudo_out != null: bf16 round trip
 // instead of codes / scales).
 static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
@@ -386,7 +401,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     }
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if (x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) return FOS_E_UNSUPPORTED;
-    if (x_type != FOS_T_BF16 && pseudo_out) return FOS_E_UNSUPPORTED;  // the fused round trip reads bf16 only
+    if (pseudo_out && !fos_pseudo_quantize_is_fused(x_type, dtype, rule, round_style, block2d)) return FOS_E_UNSUPPORTED;
     if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;
     if (rule < FOS_RULE_STATIC_6 || rule > FOS_RULE_ABS_MAX) return FOS_E_UNSUPPORTED;
     if (round_style < FOS_ROUND_NEAREST || round_style > FOS_ROUND_STOCHASTIC_UNBIASED) return FOS_E_UNSUPPORTED;
@@ -407,11 +422,11 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     // elements or more (16 MiB rows) takes the element-wise kernel like an unaligned input.
     constexpr int64_t kMaxPitch = int64_t{1} << 23;
     // fp16 input has a streaming form for NVFP4 codes with 1x16 blocks and round to nearest
-    const bool f16_streams = x_type == FOS_T_F16 && dtype == FOS_DTYPE_NVFP4 && round_style == FOS_ROUND_NEAREST && !block2d && !pseudo_out;
+    const bool f16_streams = x_type == FOS_T_F16 && dtype == FOS_DTYPE_NVFP4 && round_style == FOS_ROUND_NEAREST && !block2d;
     const bool aligned = (x_type == FOS_T_BF16 || f16_streams) && (((uintptr_t)x & 15) == 0) && (ld % 8 == 0) && (cols % 16 == 0) && ld < kMaxPitch;
     if (pseudo_out) {
-        // only the NVFP4 round-to-nearest kernels have the fused epilogue
-        if (dtype != FOS_DTYPE_NVFP4 || round_style != FOS_ROUND_NEAREST || !aligned) return FOS_E_UNSUPPORTED;
+        // only the streaming kernels have the fused epilogue
+        if (!aligned) return FOS_E_UNSUPPORTED;
         if (ldo < cols || ldo >= kMaxPitch) return FOS_E_BAD_SHAPE;
         if (((uintptr_t)pseudo_out & 15) || (ldo % 8 != 0)) return FOS_E_BAD_ALIGNMENT;
     }
@@ -493,6 +508,15 @@ extern "C" int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int6
                                    void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     if (!out) return FOS_E_NULL_POINTER;
     return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, 0, 0, FOS_SF_LINEAR, nullptr, nullptr,
+                         amax, amax_is_input, workspace, workspace_bytes, stream, static_cast<uint16_t *>(out), ldo);
+}
+
+extern "C" int fos_pseudo_quantize_keyed(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                                         int dtype, int rule, int round_style, int block2d, uint64_t seed, uint64_t offset,
+                                         void *out, int64_t ldo, float *amax, int amax_is_input,
+                                         void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!out) return FOS_E_NULL_POINTER;
+    return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, seed, offset, FOS_SF_LINEAR, nullptr, nullptr,
                          amax, amax_is_input, workspace, workspace_bytes, stream, static_cast<uint16_t *>(out), ldo);
 }
 

@@ -750,6 +750,39 @@ FOS_DEVICE void dequant_block_bf16(const BlockOut &o, float amax, float c, float
     });
 }
 
+// ... for either format and 16-bit output type, operation by operation as dequantize_kernel does it (the
+// fp16 product value * scale is exact for E2M1 values and rounds for IF4's integer blocks, whose values are
+// fp16(6/7 * integer)).  `o.s` carries the integer-block flag in bit 7.
+template <bool IF4, bool OUT_F16, bool FASTDIV>
+FOS_DEVICE void dequant_block_any(const BlockOut &o, float amax, float c, float rc, uint32_t *w) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const float sf = e4m3_decode(o.s & 0x7fu);
+    const bool int_block = IF4 && (o.s & 0x80u);
+    const _Float16 s16 = (_Float16)sf;
+    static_for<0, 8>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        const uint32_t word = j < 4 ? o.c0 : o.c1;
+        float2_t f = unpack_fp4<(j & 3)>(word) * sf;
+        if (int_block) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int iv = ((int)(word << (28 - 8 * (j & 3) - 4 * e))) >> 28;  // the nibble, sign-extended
+                f[e] = (float)((_Float16)((float)iv * (float)(6.0 / 7.0)) * s16);
+            }
+        }
+        float2_t q;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float t = f[e] * amax;
+            if (FASTDIV) q[e] = u2f((f2u(div_const(t, c, rc)) & 0x7fffffffu) | (f2u(t) & 0x80000000u));
+            else q[e] = t / c;
+        }
+        if (OUT_F16) w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, f16x2_t));
+        else w[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(q, bf16x2_t));
+    });
+}
+
 // The same through the per-scale table when fq * s * amax is exact (a maximum of <= 8 significant bits, no
 // sub-normal results): RN(fq * g / c) with g = s * amax is fq * RN(g / c) for fq in {.5, 1, 2, 4} and
 // (fq / 1.5) * RN(1.5 g / c) for fq in {1.5, 3, 6} (1.5 g is exact), i.e. (power of two) x (table value):

@@ -147,7 +147,7 @@ template <int RULE, bool FULL, bool PSEUDO, bool SR, bool IF4 = false, bool F16 
 // (the stochastic instantiations hold two sets of scaled values and the Philox state: with 128
 // registers they spilled -- 30 MB of scratch traffic per launch at 8192 x 8192 -- and the launch
 // grid of three workgroups per compute unit leaves 168; the IF4 instantiation spilled as well)
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR || IF4) ? 3 : 4))) void quantize_nvfp4_rows_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR || IF4) ? 3 : 4, (SR || IF4) ? 3 : 8))) void quantize_nvfp4_rows_kernel(
     const QuantParams p) {
     __shared__ uint32_t red[4];
     // per wavefront: 4 scale tiles x 128 bytes (pseudo-quantize: the 2 KiB of a step's output instead)
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         t.x_off = (FULL || t.cb * 16 < p.cols) ? x_lane : 0x80000000u;
         return t;
     };
-    auto load = [&](const RowsTile &t, int g, Block16 &b) {
+    auto load = [&](const RowsTile &t, int g, Block16 &b) __attribute__((always_inline)) {
         const BufferRsrc rx = make_rsrc(reinterpret_cast<const void *>(uniform64(t.x_base)), __builtin_amdgcn_readfirstlane(t.x_bytes));
         u32x4 lo, hi;
         if (FULL) {
@@ -250,13 +250,15 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
     QuantConsts kt = k;
     if (PSEUDO && kStaticRule) kt.errdiv = p.c;
-    const bool deq_lut = PSEUDO && in_range && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
+    // (the 3-operation division is exact for these divisors only; the unbiased stochastic style rescales them)
+    const bool fast_c = p.c == 1536.0f || p.c == 1792.0f || p.c == 2688.0f;
+    const bool deq_lut = PSEUDO && in_range && fast_c && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
     // the MSE decision in its product form (bf16 elements, round to nearest)
     constexpr bool kProduct = RULE == FOS_RULE_MSE && !SR && !IF4 && !F16;
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry<kProduct>(threadIdx.x, kt);
     __syncthreads();
 
-    auto process = [&](const RowsTile &t, int g, const Block16 &b) {
+    auto process = [&](const RowsTile &t, int g, const Block16 &b) __attribute__((always_inline)) {
         if (!FULL && t.cb >= sf_cols) return;  // past the padded width
         const int64_t row = t.row_base + step_row(g) + rl;
         // a step that lies wholly in the row padding (decode-sized inputs: most steps) only
@@ -286,9 +288,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         }
         if (PSEUDO) {
             uint32_t w[8];
-            if (deq_lut) dequant_block_bf16_lut(o, lut[o.s & 0x7fu], w);
-            else if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
-            else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
+            if constexpr (IF4 || F16) {
+                if (in_range && fast_c) dequant_block_any<IF4, F16, true>(o, k.amax, p.c, rc, w);
+                else dequant_block_any<IF4, F16, false>(o, k.amax, p.c, rc, w);
+            } else {
+                if (deq_lut) dequant_block_bf16_lut(o, lut[o.s & 0x7fu], w);
+                else if (in_range && fast_c) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+                else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
+            }
             const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
             if constexpr (FULL) {
                 // A lane's 32 bytes would leave as two stores of 16, each instruction covering half of every
@@ -333,8 +340,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
         const uint32_t next = tile + gridDim.x;
         const bool has_next = next < n_tiles;
         const RowsTile nxt = open_tile(has_next ? next : tile, has_next);  // without a next tile: loads of nothing
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
+        auto step = [&](int g) __attribute__((always_inline)) {
             // in its last tile a wavefront gives way, step by step, to those that are further behind
             if (!has_next && (g & 1) == 0) {
                 if (g == 0) __builtin_amdgcn_s_setprio(3);
@@ -345,6 +351,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
             if (g + 3 < 8) load(cur, g + 3, ring[(g + 3) & 3]);
             else load(nxt, g + 3 - 8, ring[(g + 3) & 3]);
             process(cur, g, ring[g & 3]);
+        };
+        if constexpr (PSEUDO && SR) {
+            // (the largest instantiations: beyond the size up to which the unroll pragma is honoured, and a loop
+            // that stays a loop indexes the ring of input registers at run time; unrolled by construction)
+            static_for<0, 8>(step);
+        } else {
+#pragma unroll
+            for (int g = 0; g < 8; ++g) step(g);
         }
         if (tiled) {
             // the wavefront's own 4 x 128 bytes: written above by its lanes, read back here in
@@ -389,12 +403,12 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
         p.tile_map = kMapRowMajor;
         if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
         const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
-        if constexpr (!PSEUDO && !SR) {
+        if constexpr (!SR) {
             if (p.x_type == FOS_T_F16) {
                 if (full)
-                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, true, PSEUDO, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
                 else
-                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+                    hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, PSEUDO, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
                 return;
             }
         }
@@ -406,16 +420,18 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
     }
     if constexpr (!SR) {
         launch_quantize_nvfp4_tiles<RULE, PSEUDO>(p, s);
-        return;
+    } else if constexpr (PSEUDO) {
+        return;  // rejected by the entry point: the fused round trip of the stochastic styles is for 1x16 blocks
+    } else {
+        p.tiles_x = (int)(p.cols_p / 64);
+        const int64_t n_tiles = (p.rows_p / 128) * p.tiles_x;
+        // Persistent grid: a few workgroups per compute unit (256 CUs), fewer when the tensor
+        // is small.  FOS_QUANT_GRID overrides the count for tuning runs.
+        int64_t grid = 256 * 6;
+        if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
+        if (grid > n_tiles) grid = n_tiles;
+        hipLaunchKernelGGL((quantize_nvfp4_tile_kernel<RULE, true, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     }
-    p.tiles_x = (int)(p.cols_p / 64);
-    const int64_t n_tiles = (p.rows_p / 128) * p.tiles_x;
-    // Persistent grid: a few workgroups per compute unit (256 CUs), fewer when the tensor
-    // is small.  FOS_QUANT_GRID overrides the count for tuning runs.
-    int64_t grid = 256 * 6;
-    if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
-    if (grid > n_tiles) grid = n_tiles;
-    hipLaunchKernelGGL((quantize_nvfp4_tile_kernel<RULE, true, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
 template <bool PSEUDO, bool SR>
@@ -441,17 +457,23 @@ void launch_quantize_if4_mse_rows(QuantParams &p, hipStream_t s) {
     if (grid > n) grid = n;
     p.tile_map = kMapRowMajor;
     if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
-    if (p.rows % 128 == 0 && p.cols % 256 == 0)
+    const bool full = p.rows % 128 == 0 && p.cols % 256 == 0;
+    if (p.pseudo_out) {
+        if (full) hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, true, true, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        else hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, false, true, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    } else if (full) {
         hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, true, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
-    else
+    } else {
         hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<FOS_RULE_MSE, false, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+    }
 }
 
 // `sr`: a stochastic style on an aligned input.  The fast exact evaluation is tied to the
 // selection divisor 1536; with the unbiased style's rescaled divisor an inconclusive
 // shortcut falls back to the operation-by-operation form.
 void launch_quantize_nvfp4_fast(QuantParams &p, int rule, bool two_d, bool aligned, bool sr, hipStream_t s) {
-    if (sr) by_rule<false, true>(p, rule, two_d, aligned, s);
+    if (sr && p.pseudo_out) by_rule<true, true>(p, rule, two_d, aligned, s);
+    else if (sr) by_rule<false, true>(p, rule, two_d, aligned, s);
     else if (p.pseudo_out) by_rule<true, false>(p, rule, two_d, aligned, s);
     else by_rule<false, false>(p, rule, two_d, aligned, s);
 }

@@ -106,15 +106,18 @@ std::tuple<Tensor, Tensor, Tensor> quantize_ex(const Tensor &x, int64_t dtype, i
 }
 
 // True when the library has a fused quantize -> dequantize kernel for this call.
-bool pseudo_quantize_is_fused(const Tensor &x, int64_t dtype, int64_t round_style) {
-    return dtype == FOS_DTYPE_NVFP4 && round_style == FOS_ROUND_NEAREST && x.dim() == 2 && x.scalar_type() == at::kBFloat16 &&
+bool pseudo_quantize_is_fused(const Tensor &x, int64_t dtype, int64_t rule, int64_t round_style, bool is_2d) {
+    if (x.dim() != 2 || (x.scalar_type() != at::kBFloat16 && x.scalar_type() != at::kHalf)) return false;
+    return fos_pseudo_quantize_is_fused(x.scalar_type() == at::kHalf ? FOS_T_F16 : FOS_T_BF16, (int)dtype, (int)rule, (int)round_style,
+                                        is_2d ? 1 : 0) &&
            x.numel() > 0 && x.stride(-1) == 1 && x.size(1) % 16 == 0 && x.stride(0) % 8 == 0 &&
            x.stride(0) < (int64_t(1) << 23)  // (the streaming kernels' 32-bit tile offsets)
            && reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0;
 }
 
-Tensor pseudo_quantize(const Tensor &x, int64_t dtype, int64_t rule, int64_t round_style, bool is_2d, const c10::optional<Tensor> &amax) {
-    TORCH_CHECK(pseudo_quantize_is_fused(x, dtype, round_style),
+Tensor pseudo_quantize(const Tensor &x, int64_t dtype, int64_t rule, int64_t round_style, bool is_2d, const c10::optional<Tensor> &amax,
+                       int64_t seed, int64_t offset) {
+    TORCH_CHECK(pseudo_quantize_is_fused(x, dtype, rule, round_style, is_2d),
                 "pseudo_quantize: no fused kernel for these arguments (quantize, then dequantize)");
     require_gpu(x, "x");
     const int64_t rows = x.size(0), cols = x.size(1);
@@ -123,9 +126,9 @@ Tensor pseudo_quantize(const Tensor &x, int64_t dtype, int64_t rule, int64_t rou
     const DeviceGuard guard(x.device());
     const fos_stream_t stream = current_stream(x);
     Tensor ws = quantize_workspace(x, stream);
-    check(fos_pseudo_quantize(x.data_ptr(), FOS_T_BF16, rows, cols, x.stride(0), (int)dtype, (int)rule, (int)round_style, is_2d ? 1 : 0,
-                              out.data_ptr(), cols, amax_buf.data_ptr<float>(), amax.has_value() ? 1 : 0, ws.data_ptr(),
-                              (size_t)ws.numel(), stream),
+    check(fos_pseudo_quantize_keyed(x.data_ptr(), x.scalar_type() == at::kHalf ? FOS_T_F16 : FOS_T_BF16, rows, cols, x.stride(0), (int)dtype,
+                                    (int)rule, (int)round_style, is_2d ? 1 : 0, (uint64_t)seed, (uint64_t)offset, out.data_ptr(), cols,
+                                    amax_buf.data_ptr<float>(), amax.has_value() ? 1 : 0, ws.data_ptr(), (size_t)ws.numel(), stream),
           "fouroversix::pseudo_quantize");
     return out;
 }
@@ -320,7 +323,7 @@ TORCH_LIBRARY(fouroversix, m) {
     m.def(
         "quantize_ex(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, int seed, int offset, "
         "int sf_layout, Tensor? amax) -> (Tensor, Tensor, Tensor)");
-    m.def("pseudo_quantize(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, Tensor? amax) -> Tensor");
+    m.def("pseudo_quantize(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, Tensor? amax, int seed=0, int offset=0) -> Tensor");
     m.def("transform(Tensor x, bool transpose, bool rht) -> (Tensor, Tensor)");
     m.def("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");
     m.def("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");

@@ -153,17 +153,6 @@ def quantize(
         q.original_shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
         return q
 
-    if config.pseudo_quantize:
-        # one fused kernel where the library has it, else the two-step round trip
-        # (QuantizeBackendBase.pseudo_quantize, src/fouroversix/quantize/backend.py:213-234)
-        fmt, style = NATIVE_FORMAT_IDS[config.dtype.value], config.round_style.native_id
-        if ops.pseudo_quantize_is_fused(x, fmt, style):
-            return ops.pseudo_quantize(
-                x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax", known_amax(x))
-            )
-        plain = QuantizationConfig(**{**config.__dict__, "pseudo_quantize": False})
-        return dequantize(quantize(x, plain), dtype=x.dtype)
-
     if config.round_style.is_stochastic and "seed" not in config.kwargs:
         if x.is_cuda and torch.cuda.is_current_stream_capturing():
             # the seed is a launch argument: a graph replays the one drawn now, every time
@@ -177,6 +166,20 @@ def quantize(
         seed = int(config.kwargs.get("seed", config.kwargs.get("rbits", 0)))
         seed = max(seed, 0)
     offset = int(config.kwargs.get("offset", 0))
+
+    if config.pseudo_quantize:
+        # one fused kernel where the library has it, else the two-step round trip
+        # (QuantizeBackendBase.pseudo_quantize, src/fouroversix/quantize/backend.py:213-234)
+        fmt, style = NATIVE_FORMAT_IDS[config.dtype.value], config.round_style.native_id
+        if ops.pseudo_quantize_is_fused(x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d):
+            return ops.pseudo_quantize(
+                x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax", known_amax(x)), seed, offset
+            )
+        plain = QuantizationConfig(
+            **{**config.__dict__, "pseudo_quantize": False, "kwargs": {**config.kwargs, "seed": seed, "offset": offset}}
+        )
+        return dequantize(quantize(x, plain), dtype=x.dtype)
+
     linear = config.dtype in _LINEAR_SCALE_FORMATS
 
     x_rows = x if x.stride(-1) == 1 else x.contiguous()

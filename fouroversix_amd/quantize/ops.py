@@ -43,9 +43,9 @@ def _direct(t: torch.Tensor) -> bool:
     return type(t) is torch.Tensor and t.device.type == "cuda" and not torch.compiler.is_compiling()
 
 
-def pseudo_quantize_is_fused(x: torch.Tensor, dtype: int, round_style: int) -> bool:
+def pseudo_quantize_is_fused(x: torch.Tensor, dtype: int, selection_rule: int, round_style: int, is_2d: bool) -> bool:
     """True when the library has a fused quantize->dequantize kernel for this call."""
-    return _C.pseudo_quantize_is_fused(x, dtype, round_style)
+    return _C.pseudo_quantize_is_fused(x, dtype, selection_rule, round_style, is_2d)
 
 
 def transform_unsupported_reason(x: torch.Tensor, transpose: bool, rht: bool) -> str | None:
@@ -77,11 +77,13 @@ def transform(x, transpose, rht):
     return torch.ops.fouroversix.transform.default(x, transpose, rht)
 
 
-def pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax=None):
-    """Fused quantize -> dequantize (bf16 in, bf16 out); see ``pseudo_quantize_is_fused``."""
+def pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax=None, seed=0, offset=0):
+    """Fused quantize -> dequantize (out has x's type); see ``pseudo_quantize_is_fused``.  ``seed`` /
+    ``offset`` key the dither of the stochastic styles, as in ``quantize_ex``."""
+    seed, offset = seed & 0x7FFFFFFFFFFFFFFF, offset & 0x7FFFFFFFFFFFFFFF
     if _direct(x):
-        return _C.pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax)
-    return torch.ops.fouroversix.pseudo_quantize.default(x, dtype, selection_rule, round_style, is_2d, amax)
+        return _C.pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax, seed, offset)
+    return torch.ops.fouroversix.pseudo_quantize.default(x, dtype, selection_rule, round_style, is_2d, amax, seed, offset)
 
 
 def gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(a, b, a_sf, b_sf, alpha):
@@ -147,7 +149,7 @@ def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, ama
 
 
 @torch.library.register_fake("fouroversix::pseudo_quantize")
-def _(x, dtype, selection_rule, round_style, is_2d, amax):
+def _(x, dtype, selection_rule, round_style, is_2d, amax, seed=0, offset=0):
     return torch.empty_like(x, memory_format=torch.contiguous_format)
 
 

@@ -158,15 +158,35 @@ int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t
  * the values fos_dequantize would return for fos_quantize's result, without materialising
  * codes or scales.  Stands in for QuantizeBackendBase.pseudo_quantize
  * (src/fouroversix/quantize/backend.py:213-234; fused Triton kernel
- * src/fouroversix/kernels/triton/ops.py:212-374).  Arguments as fos_quantize.  Fused
- * kernels exist for FOS_T_BF16 input, FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST, x and out 16-byte aligned,
- * ld and ldo multiples of 8 and cols a multiple of 16; anything else returns
+ * src/fouroversix/kernels/triton/ops.py:212-374).  Arguments as fos_quantize; out has x's element
+ * type.  Fused kernels exist for the combinations fos_pseudo_quantize_is_fused names, with x and out
+ * 16-byte aligned, ld and ldo multiples of 8 and cols a multiple of 16; anything else returns
  * FOS_E_UNSUPPORTED (compose fos_quantize and fos_dequantize instead).
  */
 int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
                         int dtype, int rule, int round_style, int block2d,
                         void *out, int64_t ldo, float *amax, int amax_is_input,
                         void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * fos_pseudo_quantize with the dither key of the stochastic rounding styles (seed, offset as in
+ * fos_quantize; fos_pseudo_quantize uses 0, 0): the output is bit for bit what fos_dequantize returns for
+ * fos_quantize's result under the same key.  The reference's fused kernel draws its random bits inside
+ * the kernel (src/fouroversix/kernels/triton/ops.py:212-374); here the caller holds the key.
+ */
+int fos_pseudo_quantize_keyed(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                              int dtype, int rule, int round_style, int block2d, uint64_t seed, uint64_t offset,
+                              void *out, int64_t ldo, float *amax, int amax_is_input,
+                              void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
+ * 1 when a fused kernel exists for this element type (FOS_T_*), format, selection rule, rounding style and
+ * block shape (alignment aside), else 0: FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST on bf16 (either block
+ * shape) and fp16 (1x16 blocks); FOS_DTYPE_NVFP4 with FOS_ROUND_STOCHASTIC on bf16 and 1x16 blocks (the
+ * unbiased style with the MSE and static rules); FOS_DTYPE_IF4 with FOS_RULE_MSE on bf16, round to nearest,
+ * 1x16 blocks.  Pure host function.
+ */
+int fos_pseudo_quantize_is_fused(int x_type, int dtype, int rule, int round_style, int block2d);
 
 /*
  * D[M, N] = alpha * sum_k (A[m,k] * sfA[m,k/16]) * (B[n,k] * sfB[n,k/16]), FP32
