@@ -365,14 +365,14 @@ static bool stream_is_capturing(hipStream_t s) {
 }
 
 // Which combinations the fused quantize -> dequantize kernels cover (alignment aside): NVFP4 with round to
-// nearest (bf16 with either block shape, fp16 with 1x16 blocks), NVFP4 with a stochastic style on bf16 and
-// 1x16 blocks (the unbiased style with the rules whose decision the streaming kernel makes), IF4 with the MSE
+// nearest (bf16 with either block shape, fp16 with 1x16 blocks), NVFP4 with a stochastic style on bf16
+// (the unbiased style with the rules whose decision the streaming kernels make), IF4 with the MSE
 // rule on bf16, round to nearest, 1x16 blocks.
 extern "C" int fos_pseudo_quantize_is_fused(int x_type, int dtype, int rule, int round_style, int block2d) {
     const bool rtn = round_style == FOS_ROUND_NEAREST;
     if (dtype == FOS_DTYPE_NVFP4 && rtn) return x_type == FOS_T_BF16 || (x_type == FOS_T_F16 && !block2d);
-    if (x_type != FOS_T_BF16 || block2d) return 0;
-    if (dtype == FOS_DTYPE_IF4) return rtn && rule == FOS_RULE_MSE;
+    if (x_type != FOS_T_BF16) return 0;
+    if (dtype == FOS_DTYPE_IF4) return rtn && rule == FOS_RULE_MSE && !block2d;
     if (dtype != FOS_DTYPE_NVFP4) return 0;
     if (round_style == FOS_ROUND_STOCHASTIC) return 1;
     return round_style == FOS_ROUND_STOCHASTIC_UNBIASED &&

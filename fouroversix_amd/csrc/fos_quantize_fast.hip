@@ -1,16 +1,12 @@
-// Pass 2 for NVFP4 with round-to-nearest or plain stochastic rounding, around the fast
-// block formulation of fos_quantize_fast.h.  Two lane mappings:
-//
-//  * 1x16 blocks (quantize_nvfp4_rows_kernel): a wavefront covers 4 rows x 16 blocks,
-//    i.e. 512 contiguous bytes per row.  Measured on MI355X, a wavefront that touches 16
-//    rows x 128 bytes streams at ~4.1 TB/s while 4 rows x 512 bytes reaches ~6 TB/s, so the
-//    row-contiguous mapping is what the HBM-bound path uses.  A 256-thread workgroup
-//    covers 128 rows x 256 columns in eight steps of 16 rows (the next step's loads are
-//    issued before the current step is processed), stages the 4 complete 128x4 scale
-//    tiles in LDS and writes them as one contiguous 2 KiB run.
-//  * 16x16 tiles (quantize_nvfp4_tile_kernel): the 16 rows of a tile must lie along one DPP
-//    row for the tile reductions, so a wavefront covers 16 rows x 4 blocks; persistent
-//    workgroups walk over 128 x 64 tiles with the next tile prefetched.
+// Pass 2 for NVFP4 with round-to-nearest or a stochastic rounding style and 1x16 blocks, around the fast
+// block formulation of fos_quantize_fast.h (quantize_nvfp4_rows_kernel): a wavefront covers 4 rows x 16
+// blocks, i.e. 512 contiguous bytes per row.  Measured on MI355X, a wavefront that touches 16
+// rows x 128 bytes streams at ~4.1 TB/s while 4 rows x 512 bytes reaches ~6 TB/s, so the
+// row-contiguous mapping is what the HBM-bound path uses.  A 256-thread workgroup
+// covers 128 rows x 256 columns in eight steps of 16 rows (the next step's loads are
+// issued before the current step is processed), stages the 4 complete 128x4 scale
+// tiles in LDS and writes them as one contiguous 2 KiB run.  16x16 tiles have the same mapping in
+// fos_quantize_tiles.hip; the dispatch by rule, block shape and style is at the end of this file.
 #include <cstdlib>
 
 #include "fos_buffer.h"
@@ -18,103 +14,6 @@
 #include "fos_tuning.h"
 
 namespace fos {
-
-struct TileRegs {
-    Block16 b[2];
-};
-
-FOS_DEVICE void load_tile(const QuantParams &p, uint32_t tile, int lane, int wave, TileRegs &t) {
-    const int64_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - (uint32_t)tile_y * (uint32_t)p.tiles_x;
-    const int64_t c0 = (tile_x * 4 + (lane >> 4)) * 16;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int64_t r = tile_y * 128 + h * 64 + wave * 16 + (lane & 15);
-        if (r < p.rows && c0 < p.cols) {
-            const uint4 *src = reinterpret_cast<const uint4 *>(p.x + r * p.ld + c0);
-            const uint4 lo = src[0], hi = src[1];
-            t.b[h].w[0] = lo.x; t.b[h].w[1] = lo.y; t.b[h].w[2] = lo.z; t.b[h].w[3] = lo.w;
-            t.b[h].w[4] = hi.x; t.b[h].w[5] = hi.y; t.b[h].w[6] = hi.z; t.b[h].w[7] = hi.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) t.b[h].w[i] = 0;
-        }
-    }
-}
-
-template <int RULE, bool TWO_D, bool PSEUDO, bool SR>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_tile_kernel(const QuantParams p) {
-    __shared__ uint32_t red[4];
-    __shared__ uint32_t sf_tile[2][128];
-    __shared__ __attribute__((aligned(16))) FastLutEntry lut[128];
-
-    const uint32_t amax_bits = reduce_partials(p, red);
-    QuantConsts k;
-    k.amax = u2f(amax_bits);
-    k.enc = p.c / k.amax;
-    k.dec = 1.0f / (p.c / k.amax);
-    k.qdiv = p.qdiv;
-    k.errdiv = p.errdiv;
-    k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
-    k.shortcut_ok = shortcut_range(k.amax);
-    if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
-    const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
-    const float enc_fast = in_range ? k.enc : 0.0f;
-    const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
-    if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, k);
-    __syncthreads();
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t sf_cols = p.cols_p >> 4;
-    const uint32_t n_tiles = (uint32_t)(p.rows_p >> 7) * (uint32_t)p.tiles_x;
-    const bool tiled = !PSEUDO && p.sf_layout == FOS_SF_TILED_128X4;
-
-    auto process = [&](uint32_t tile, const TileRegs &t, uint32_t *stage) {
-        const int64_t tile_y = tile / (uint32_t)p.tiles_x, tile_x = tile - (uint32_t)tile_y * (uint32_t)p.tiles_x;
-        const int64_t cb = tile_x * 4 + (lane >> 4);
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int rr = h * 64 + wave * 16 + (lane & 15);
-            const int64_t r = tile_y * 128 + rr;
-            const BlockOut o = quantize_block_nvfp4_fast<RULE, TWO_D, SR>(t.b[h], k, enc_fast, rq, in_range, lut,
-                                                                          p.seed, p.offset, (uint64_t)(r * sf_cols + cb));
-            if (PSEUDO) {
-                uint32_t w[8];
-                if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
-                else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
-                if (r < p.rows && cb * 16 < p.cols) {
-                    uint4 *d = reinterpret_cast<uint4 *>(p.pseudo_out + r * p.ldo + cb * 16);
-                    d[0] = make_uint4(w[0], w[1], w[2], w[3]);
-                    d[1] = make_uint4(w[4], w[5], w[6], w[7]);
-                }
-                continue;
-            }
-            *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(o.c0, o.c1);
-            if (tiled) reinterpret_cast<uint8_t *>(stage)[(rr & 31) * 16 + (rr >> 5) * 4 + (lane >> 4)] = (uint8_t)o.s;
-            else p.sf[r * sf_cols + cb] = (uint8_t)o.s;
-        }
-        if (tiled) {
-            __syncthreads();
-            if (threadIdx.x < 128)
-                reinterpret_cast<uint32_t *>(p.sf + (tile_y * (sf_cols >> 2) + tile_x) * 512)[threadIdx.x] = stage[threadIdx.x];
-        }
-    };
-
-    // two tiles per trip so that the prefetch registers alternate without copies
-    TileRegs ta, tb;
-    uint32_t tile = blockIdx.x;
-    const uint32_t step = gridDim.x;
-    if (tile < n_tiles) load_tile(p, tile, lane, wave, ta);
-    while (tile < n_tiles) {
-        if (tile + step < n_tiles) load_tile(p, tile + step, lane, wave, tb);
-        process(tile, ta, sf_tile[0]);
-        tile += step;
-        if (tile >= n_tiles) break;
-        if (tile + step < n_tiles) load_tile(p, tile + step, lane, wave, ta);
-        process(tile, tb, sf_tile[1]);
-        tile += step;
-    }
-}
-
 
 // 1x16 blocks, row-contiguous mapping.  Workgroup tile: 128 rows x 256 columns, walked in
 // eight steps; in a step a wavefront covers 4 rows x 16 blocks (lane -> block column lane & 15
@@ -378,8 +277,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     }
 }
 
-// 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): round to nearest, every rule.
-template <int RULE, bool PSEUDO>
+// 16x16 tiles on the row-contiguous mapping (fos_quantize_tiles.hip): every rule and rounding style.
+template <int RULE, bool PSEUDO, bool SR>
 void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s);
 
 template <int RULE, bool PSEUDO, bool SR>
@@ -418,20 +317,7 @@ static void by_dim(QuantParams &p, bool two_d, bool aligned, hipStream_t s) {
             hipLaunchKernelGGL((quantize_nvfp4_rows_kernel<RULE, false, PSEUDO, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         return;
     }
-    if constexpr (!SR) {
-        launch_quantize_nvfp4_tiles<RULE, PSEUDO>(p, s);
-    } else if constexpr (PSEUDO) {
-        return;  // rejected by the entry point: the fused round trip of the stochastic styles is for 1x16 blocks
-    } else {
-        p.tiles_x = (int)(p.cols_p / 64);
-        const int64_t n_tiles = (p.rows_p / 128) * p.tiles_x;
-        // Persistent grid: a few workgroups per compute unit (256 CUs), fewer when the tensor
-        // is small.  FOS_QUANT_GRID overrides the count for tuning runs.
-        int64_t grid = 256 * 6;
-        if (const int forced = tuning().quant_grid) grid = forced > 0 ? forced : grid;
-        if (grid > n_tiles) grid = n_tiles;
-        hipLaunchKernelGGL((quantize_nvfp4_tile_kernel<RULE, true, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
-    }
+    launch_quantize_nvfp4_tiles<RULE, PSEUDO, SR>(p, s);
 }
 
 template <bool PSEUDO, bool SR>

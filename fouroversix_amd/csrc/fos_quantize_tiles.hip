@@ -1,4 +1,4 @@
-// Pass 2 for NVFP4 with 16x16 scale tiles (block_scale_2d), round to nearest, rules static_6 /
+// Pass 2 for NVFP4 with 16x16 scale tiles (block_scale_2d), round to nearest or a stochastic style, rules static_6 /
 // static_4 and 4/6 with the MSE, MAE or abs-max rule, on the row-contiguous lane mapping of the 1x16 kernel: a wavefront
 // touches 4 rows x 512 contiguous bytes per step.
 //
@@ -17,7 +17,7 @@
 // A tile whose certified shortcut is inconclusive, whose scale byte is zero or sub-normal in a
 // way the hardware convert cannot follow, or a tensor whose maximum is outside the fast range
 // takes the operation-by-operation form, one tile at a time spread over the whole wavefront
-// (slow_tile in the kernel).
+// (slow_tile in the kernel; slow_tile_sr for the stochastic styles, whose dither is keyed per row of a tile).
 #include "fos_buffer.h"
 #include "fos_quantize_kernel.h"
 #include "fos_tuning.h"
@@ -85,6 +85,41 @@ FOS_DEVICE void block_candidates(const Block16 &blk, float invA, float invB, uin
     });
 }
 
+// ... with a stochastic style: the hardware's dithered convert on the scaled values, one Philox call per block
+// keyed by `blkid` = row * (cols_p / 16) + block column (the second candidate reads the words exchanged pairwise),
+// as in the 1x16 path.
+template <int RULE>
+FOS_DEVICE void block_candidates_sr(const Block16 &blk, float invA, float invB, uint64_t seed, uint64_t offset, uint64_t blkid,
+                                    uint32_t &a0, uint32_t &a1, uint32_t &b0, uint32_t &b1, float &SA, float &SB) {
+    float xs[16];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        xs[2 * j] = scaled(u2f(blk.w[j] << 16), invA);
+        xs[2 * j + 1] = scaled(u2f(blk.w[j] & 0xffff0000u), invA);
+    }
+    const Philox4 pA = block_philox(seed, offset, blkid);
+    sr_pack16(xs, pA, a0, a1);
+    b0 = b1 = 0;
+    if (RULE != FOS_RULE_STATIC_6) {
+        static_for<0, 8>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const float2_t fa = unpack_fp4<(j & 3)>(j < 4 ? a0 : a1);
+            accumulate_scaled<RULE>(fa.x - xs[2 * j], fa.y - xs[2 * j + 1], SA);
+        });
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            xs[2 * j] = scaled(u2f(blk.w[j] << 16), invB);
+            xs[2 * j + 1] = scaled(u2f(blk.w[j] & 0xffff0000u), invB);
+        }
+        sr_pack16(xs, second_candidate_words(pA), b0, b1);
+        static_for<0, 8>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const float2_t fb = unpack_fp4<(j & 3)>(j < 4 ? b0 : b1);
+            accumulate_scaled<RULE>(fb.x - xs[2 * j], fb.y - xs[2 * j + 1], SB);
+        });
+    }
+}
+
 // IF4: the E2M1 candidate ("a") and the INT4 candidate ("b") of one block on their common scale,
 // with the sums of squared residuals in the scaled domain (quantize_block_if4_mse, for a tile).
 FOS_DEVICE void block_candidates_if4(const Block16 &blk, float inv, uint32_t &a0, uint32_t &a1, uint32_t &b0, uint32_t &b1,
@@ -128,9 +163,12 @@ FOS_DEVICE uint32_t quad_bytes(uint32_t l0, uint32_t l1, uint32_t l2, uint32_t l
 
 // IF4: the IF4 format with its MSE rule (both candidates on one scale; the chosen one is flagged in
 // bit 7 of the scale byte) instead of NVFP4.
-template <int RULE, bool FULL, bool PSEUDO, bool IF4 = false>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void quantize_nvfp4_tiles_kernel(
+// SR: a stochastic rounding style (NVFP4); its two sets of scaled values and the Philox state take the
+// registers of three wavefronts per SIMD.
+template <int RULE, bool FULL, bool PSEUDO, bool IF4 = false, bool SR = false>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3 : 4, SR ? 3 : 8))) void quantize_nvfp4_tiles_kernel(
     const QuantParams p) {
+    static_assert(!(SR && IF4), "stochastic styles: NVFP4");
     constexpr bool STATIC = RULE == FOS_RULE_STATIC_6;
     constexpr bool ADAPTIVE = !STATIC;            // 4/6 with the MSE, MAE or abs-max rule
     constexpr bool MAXRULE = RULE == FOS_RULE_ABS_MAX;  // the error is the largest term, not the sum
@@ -239,7 +277,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
     QuantConsts kt = k;
     if (PSEUDO && kStaticRule) kt.errdiv = p.c;
-    const bool deq_lut = PSEUDO && in_range && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
+    // (the 3-operation division is exact for these divisors only; the unbiased stochastic style rescales them)
+    const bool fast_c = p.c == 1536.0f || p.c == 1792.0f || p.c == 2688.0f;
+    const bool deq_lut = PSEUDO && in_range && fast_c && (amax_bits & 0xffffu) == 0 && kt.errdiv == p.c;
     if (threadIdx.x < 128) lut[threadIdx.x] = make_lut_entry(threadIdx.x, kt);
     __syncthreads();
 
@@ -250,7 +290,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             uint32_t w[8];
             const BlockOut o{c0, c1, sbyte};
             if (deq_lut) dequant_block_bf16_lut(o, lut[sbyte & 0x7fu], w);
-            else if (in_range) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
+            else if (in_range && fast_c) dequant_block_bf16<true>(o, k.amax, p.c, rc, w);
             else dequant_block_bf16<false>(o, k.amax, p.c, rc, w);
             if (pred && (FULL || (row < rows32 && t.cb < cols16))) {
                 const u32x4 d0 = {w[0], w[1], w[2], w[3]}, d1 = {w[4], w[5], w[6], w[7]};
@@ -391,6 +431,52 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         return s_out;
     };
 
+    // The same for the stochastic styles: lane & 15 = row of the tile, which the lane quantizes as one block of
+    // the tile with the operation-by-operation block function (its tile reductions run along the 16 lanes of a
+    // DPP row; the four DPP rows compute the same tile and the first one writes).  The dither is keyed per
+    // row of the tile, as everywhere.
+    auto slow_tile_sr = [&](const TilesPos &t, uint32_t q, uint32_t tl) -> uint32_t {
+        const BufferRsrc rx = make_rsrc(reinterpret_cast<const void *>(uniform64(t.x_base)), __builtin_amdgcn_readfirstlane(t.x_bytes));
+        const int32_t cb_tile = __builtin_amdgcn_readfirstlane(t.cb - lb) + (int32_t)tl;
+        const uint32_t gbase = (FULL || cb_tile < cols16) ? 32u * q * x_row + tl * 32u : 0x80000000u;
+        const uint32_t r = lane & 15;
+        const u32x4 lo = __builtin_amdgcn_raw_buffer_load_b128(rx, gbase + r * x_row, 0, 0);
+        const u32x4 hi = __builtin_amdgcn_raw_buffer_load_b128(rx, gbase + r * x_row + 16u, 0, 0);
+        const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        float x[16];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            x[2 * j] = u2f(w[j] << 16);
+            x[2 * j + 1] = u2f(w[j] & 0xffff0000u);
+        }
+        const uint32_t rstep = 32u * q + r;
+        const int32_t row = t.row0 + (int32_t)rstep;
+        uint32_t codes[2], sbyte;
+        quantize_block_f32<FOS_DTYPE_NVFP4, RULE, FOS_ROUND_STOCHASTIC, true>(x, k, p.seed, p.offset,
+                                                                              (uint64_t)((int64_t)row * sf_cols + cb_tile), codes, sbyte);
+        if (PSEUDO) {
+            uint32_t d[8];
+            dequant_block_bf16<false>(BlockOut{codes[0], codes[1], sbyte}, k.amax, p.c, rc, d);
+            if (lane < 16 && (FULL || (row < rows32 && cb_tile < cols16))) {
+                const u32x4 d0 = {d[0], d[1], d[2], d[3]}, d1 = {d[4], d[5], d[6], d[7]};
+                const BufferRsrc rout = make_rsrc(reinterpret_cast<const void *>(uniform64(t.out_base)), 0xffffffffu);
+                __builtin_amdgcn_raw_buffer_store_b128(d0, rout, rstep * o_row + tl * 32u, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(d1, rout, rstep * o_row + tl * 32u + 16u, 0, 0);
+            }
+            return sbyte;
+        }
+        if (lane < 16) {
+            const u32x2 c01 = {codes[0], codes[1]};
+            const BufferRsrc rcodes = make_rsrc(reinterpret_cast<const void *>(uniform64(t.codes_base)), 0xffffffffu);
+            __builtin_amdgcn_raw_buffer_store_b64(c01, rcodes, rstep * c_row + tl * 8u, 0, 0);
+            if (!tiled) {
+                const BufferRsrc rsf = make_rsrc(reinterpret_cast<const void *>(uniform64((uint64_t)(p.sf + (int64_t)t.row0 * sf_cols))), 0xffffffffu);
+                __builtin_amdgcn_raw_buffer_store_b8((uint8_t)sbyte, rsf, rstep * (uint32_t)sf_cols + (uint32_t)cb_tile, 0, 0);
+            }
+        }
+        return sbyte;
+    };
+
     // one group: four blocks per lane in, codes (or dequantised values) out; returns the scale byte
     auto process = [&](const TilesPos &t, uint32_t q, const TilesPos &nt, uint32_t nq) -> uint32_t {
         const int32_t grow = t.row0 + 32 * (int32_t)q;  // first row of the group (wave-uniform)
@@ -408,7 +494,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 for (int j = 0; j < 8; ++j)
                     bmax = fmaxf(fmaxf(fabsf(u2f(blk[s].w[j] << 16)), fabsf(u2f(blk[s].w[j]))), bmax);
             bmax = tile_max(u2f(f2u(bmax) & 0xffff0000u));
-            const float s_hp6 = div_const(bmax, k.qdiv, rq) * enc_fast;
+            // (the 3-operation division is exact for the divisors 6 and 4; the unbiased stochastic style rescales them)
+            float bq;
+            if (SR && k.qdiv != 6.0f && k.qdiv != 4.0f) bq = bmax / k.qdiv;
+            else bq = div_const(bmax, k.qdiv, rq);
+            const float s_hp6 = bq * enc_fast;
             const float s_hp4 = s_hp6 * 1.5f;
             const uint32_t pk = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s_hp6, s_hp4, 0, false);
             const uint32_t s6 = pk & 0xffu, s4 = (pk >> 8) & 0xffu;
@@ -417,13 +507,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
             if (ADAPTIVE && !IF4) B = lut[s4];
             // the hardware convert saturates at 6 where the reference's unclamped rounding gives 8:
             // that needs a sub-normal scale byte rounded down by more than 7/6; a zero scale byte
-            // of a non-zero tile has no scaled domain
-            const bool fast_ok = s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f);
+            // of a non-zero tile has no scaled domain.  (The stochastic styles clamp to 6 in the
+            // reference as well: only the zero scale byte is left out there.)
+            const bool fast_ok = SR ? s6 != 0u : (s6 >= 8u || (s6 != 0u && bmax * A.inv < 7.0f));
             uint32_t cB[4][2];
             float SA = 0.0f, SB = 0.0f;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 if constexpr (IF4) block_candidates_if4(blk[s], A.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
+                else if constexpr (SR)
+                    block_candidates_sr<RULE>(blk[s], A.inv, B.inv, p.seed, p.offset, (uint64_t)((int64_t)(grow + 4 * s + li) * sf_cols + t.cb),
+                                              oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 else block_candidates<RULE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 load(nt, 32 * nq + 4 * s, blk[s]);
             }
@@ -472,7 +566,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
         uint64_t pending = __builtin_amdgcn_ballot_w64(need_slow);
         while (pending != 0) {
             const uint32_t tl = (uint32_t)__builtin_ctzll(pending) & 15u;
-            const uint32_t sP = slow_tile(t, q, tl);
+            uint32_t sP;
+            if constexpr (SR) sP = slow_tile_sr(t, q, tl);
+            else sP = slow_tile(t, q, tl);
             if ((uint32_t)lb == tl) os = sP;
             pending &= ~(0x0001000100010001ull << tl);
         }
@@ -507,7 +603,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
 
 }  // namespace
 
-template <int RULE, bool PSEUDO>
+template <int RULE, bool PSEUDO, bool SR>
 void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s) {
     p.tiles_x = (int)((p.cols_p + 511) / 512);
     const int64_t n = (p.rows_p / 128) * p.tiles_x;
@@ -521,9 +617,9 @@ void launch_quantize_nvfp4_tiles(QuantParams &p, hipStream_t s) {
     if (const int forced = tuning().quant_map) p.tile_map = forced - 1;
     const bool full = p.rows % 128 == 0 && p.cols % 512 == 0;
     if (full)
-        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, true, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, true, PSEUDO, false, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     else
-        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, false, PSEUDO>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
+        hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<RULE, false, PSEUDO, false, SR>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
 // IF4 with the MSE rule, round to nearest, 16x16 tiles, aligned input.
@@ -541,13 +637,21 @@ void launch_quantize_if4_mse_tiles(QuantParams &p, hipStream_t s) {
         hipLaunchKernelGGL((quantize_nvfp4_tiles_kernel<FOS_RULE_MSE, false, false, true>), dim3((unsigned)grid), dim3(kThreads), 0, s, p);
 }
 
-template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, false>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, true>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, false>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, true>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, false>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, true>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, false>(QuantParams &, hipStream_t);
-template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, false, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, true, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, false, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_STATIC_6, true, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, false, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, true, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, false, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MSE, true, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, false, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, true, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, false, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_MAE, true, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, false, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, true, false>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, false, true>(QuantParams &, hipStream_t);
+template void launch_quantize_nvfp4_tiles<FOS_RULE_ABS_MAX, true, true>(QuantParams &, hipStream_t);
 
 }  // namespace fos

@@ -182,7 +182,7 @@ int fos_pseudo_quantize_keyed(const void *x, int x_type, int64_t rows, int64_t c
 /*
  * 1 when a fused kernel exists for this element type (FOS_T_*), format, selection rule, rounding style and
  * block shape (alignment aside), else 0: FOS_DTYPE_NVFP4 with FOS_ROUND_NEAREST on bf16 (either block
- * shape) and fp16 (1x16 blocks); FOS_DTYPE_NVFP4 with FOS_ROUND_STOCHASTIC on bf16 and 1x16 blocks (the
+ * shape) and fp16 (1x16 blocks); FOS_DTYPE_NVFP4 with FOS_ROUND_STOCHASTIC on bf16, either block shape (the
  * unbiased style with the MSE and static rules); FOS_DTYPE_IF4 with FOS_RULE_MSE on bf16, round to nearest,
  * 1x16 blocks.  Pure host function.
  */

@@ -601,6 +601,20 @@ def test_stochastic_rounding_bit_exact_with_oracle_key(oracle, dtype, rule, two_
     assert (u8(q2.values) != u8(q.values)).mean() > 0.05
 
 
+@pytest.mark.parametrize("rule", ["static_6", "static_4", "mse", "mae", "abs_max"])
+@pytest.mark.parametrize("style", ["stochastic", "stochastic_unbiased"])
+def test_stochastic_rounding_on_tiles_bit_exact(oracle, rule, style):
+    """16x16 tiles with a stochastic style on the streaming kernel: whole and ragged workgroup tiles, data whose
+    tiles tie or come close (outlier channels, blocks spanning six decades), every rule; the dither is keyed per
+    row of a tile, so a tile sent through the operation-by-operation path must draw the same bits."""
+    for kind, shape, seed in (("randn", (256, 1024), 31), ("outlier", (384, 528), 32), ("tiny_blocks", (128, 512), 33),
+                              ("weight", (1024, 2048), 34)):
+        x = make_input(kind, shape, seed)
+        kw = dict(scale_rule=rule, block_scale_2d=True, round_style=style)
+        q = hip_quantize(x, kwargs={"seed": 1234 + seed, "offset": 2}, **kw)
+        assert_same_quantization(q, oracle.quantize(x, seed=1234 + seed, offset=2, **kw), f"{kind} {shape} {kw}")
+
+
 @pytest.mark.parametrize("style", ["stochastic", "stochastic_unbiased"])
 def test_stochastic_rounding_edge_cases_bit_exact(oracle, style):
     """The stochastic styles on the inputs that steer the kernels off their main path:
@@ -803,6 +817,27 @@ def test_fused_round_trip_of_the_other_formats_and_styles(fmt, rule, style, dtyp
     r = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True, **kw))
     e = fos.dequantize(fos.quantize(x, cfg), dtype=x.dtype)
     assert r.dtype == dtype and r.shape == x.shape
+    assert torch.equal(r.view(torch.int16), e.view(torch.int16))
+
+
+@pytest.mark.parametrize("rule", ["static_6", "static_4", "mse", "mae", "abs_max"])
+@pytest.mark.parametrize("style", ["stochastic", "stochastic_unbiased"])
+@pytest.mark.parametrize(("shape", "scale"), [((256, 512), 1.0), ((200, 208), 1.0), ((128, 1024), 2.0**-30), ((2048, 2048), 1.0)])
+def test_fused_round_trip_of_the_stochastic_styles_on_tiles(rule, style, shape, scale):
+    """... and with 16x16 tiles (the unbiased style's MAE and abs-max rules take the two-step path)."""
+    from fouroversix_amd.quantize import ops
+
+    x = (make_input("outlier", shape, 23).float() * scale).bfloat16()
+    x[0, :16] = -x[0, :16].abs()
+    x[1, 3] = -0.0
+    x[16:32] = 0
+    x = x.cuda()
+    kw = dict(scale_rule=rule, round_style=style, block_scale_2d=True, kwargs={"seed": 78, "offset": 1})
+    cfg = fos.QuantizationConfig(**kw)
+    fused = ops.pseudo_quantize_is_fused(x, 0, cfg.scale_rule.cuda_id, cfg.round_style.native_id, True)
+    assert fused == (style == "stochastic" or rule in ("static_6", "static_4", "mse"))
+    r = fos.quantize(x, fos.QuantizationConfig(pseudo_quantize=True, **kw))
+    e = fos.dequantize(fos.quantize(x, cfg), dtype=x.dtype)
     assert torch.equal(r.view(torch.int16), e.view(torch.int16))
 
 
