@@ -260,11 +260,17 @@ def extras(dev, steps: int) -> dict:
                      ("quantize_mse_rht", dict(scale_rule="mse", rht=True)),
                      ("quantize_mse_transpose_rht", dict(scale_rule="mse", rht=True, transpose=True)),
                      ("quantize_mse_stochastic", dict(scale_rule="mse", round_style="stochastic", kwargs={"seed": 1})),
+                     ("quantize_mse_2d_stochastic", dict(scale_rule="mse", round_style="stochastic", block_scale_2d=True, kwargs={"seed": 1})),
+                     ("pseudo_quantize_mse_stochastic", dict(scale_rule="mse", round_style="stochastic", pseudo_quantize=True, kwargs={"seed": 1})),
                      ("quantize_if4_mse", dict(dtype="if4", scale_rule="mse")),
+                     ("pseudo_quantize_if4_mse", dict(dtype="if4", scale_rule="mse", pseudo_quantize=True)),
                      ("quantize_mxfp4_static_6", dict(dtype="mxfp4", scale_rule="static_6"))):
         cfg = fos.QuantizationConfig(**kw)
         out[f"{name}_8192x8192_us"] = us(lambda: fos.quantize(nxt(), cfg))
-    del xs
+    xh = xs[0].half()
+    cfg = fos.QuantizationConfig(scale_rule="mse", pseudo_quantize=True)
+    out["pseudo_quantize_mse_fp16_8192x8192_us"] = us(lambda: fos.quantize(xh, cfg))
+    del xs, xh
     mse = fos.QuantizationConfig(scale_rule="mse")
     for m, nn, k in ((16, 4096, 4096), (16, 14336, 4096), (16, 4096, 14336), (128, 4096, 4096), (128, 14336, 4096),
                      (128, 4096, 14336), (2048, 14336, 4096), (2048, 4096, 4096), (2048, 4096, 14336)):

@@ -30,6 +30,7 @@ EXPORTS = (
     "fos_amax",
     "fos_quantize",
     "fos_quantize_static",
+    "fos_quantize_devkey",
     "fos_pseudo_quantize",
     "fos_pseudo_quantize_keyed",
     "fos_pseudo_quantize_is_fused",
@@ -84,6 +85,8 @@ def lib() -> ctypes.CDLL:
     L.fos_quantize.restype = i32
     L.fos_quantize_static.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, i32, vp, vp, vp, i32, vp]
     L.fos_quantize_static.restype = i32
+    L.fos_quantize_devkey.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i32, vp, vp, vp, i32, vp, sz, vp]
+    L.fos_quantize_devkey.restype = i32
     L.fos_pseudo_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, vp, i64, vp, i32, vp, sz, vp]
     L.fos_pseudo_quantize.restype = i32
     L.fos_pseudo_quantize_keyed.argtypes = [vp, i32, i64, i64, i64, i32, i32, i32, i32, u64, u64, vp, i64, vp, i32, vp, sz, vp]

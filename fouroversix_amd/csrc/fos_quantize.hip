@@ -386,8 +386,9 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
                          uint64_t seed, uint64_t offset, int sf_layout,
                          uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
                          void *workspace, size_t workspace_bytes, fos_stream_t stream,
-                         uint16_t *pseudo_out, int64_t ldo) {
+                         uint16_t *pseudo_out, int64_t ldo, const uint64_t *key = nullptr) {
     if (!x || !amax || (!pseudo_out && (!codes || !sf))) return FOS_E_NULL_POINTER;
+    if ((uintptr_t)key & 7) return FOS_E_BAD_ALIGNMENT;
     if (dtype == FOS_DTYPE_MXFP4) {
         // one streaming kernel; no tensor maximum, no workspace
         if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
@@ -444,6 +445,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     p.rows_p = rows_p; p.cols_p = cols_p;
     p.codes = codes; p.sf = sf;
     p.seed = seed; p.offset = offset;
+    p.key = key;
     p.sf_layout = sf_layout;
 
     if (amax_is_input) {
@@ -500,6 +502,17 @@ extern "C" int fos_quantize(const void *x, int x_type, int64_t rows, int64_t col
                             void *workspace, size_t workspace_bytes, fos_stream_t stream) {
     return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, seed, offset, sf_layout, codes, sf,
                          amax, amax_is_input, workspace, workspace_bytes, stream, nullptr, 0);
+}
+
+extern "C" int fos_quantize_devkey(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                                   int dtype, int rule, int round_style, int block2d,
+                                   const uint64_t *key, int sf_layout,
+                                   uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                                   void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!key) return FOS_E_NULL_POINTER;
+    if (dtype == FOS_DTYPE_MXFP4) return FOS_E_UNSUPPORTED;  // (no stochastic style there)
+    return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, 0, 0, sf_layout, codes, sf,
+                         amax, amax_is_input, workspace, workspace_bytes, stream, nullptr, 0, key);
 }
 
 extern "C" int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,

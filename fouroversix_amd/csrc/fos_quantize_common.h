@@ -28,7 +28,8 @@ struct QuantParams {
     int n_partials;              // number of pairs; 0 = `partials` points at a caller-supplied f32 amax;
                                  // -1 = no pass 1 ran: pass 2 scans the (small, contiguous, aligned) input itself
     float *amax_out;             // written by workgroup 0 when not null
-    uint64_t seed, offset;
+    uint64_t seed, offset;       // dither key of the stochastic styles ...
+    const uint64_t *key = nullptr;  // ... or, when not null, where the kernels read {seed, offset} from (device memory)
     int sf_layout;
     int tiles_x;                 // workgroup tiles along the columns
     int tile_map = 0;            // TileMap: which tile the n-th unit of work is

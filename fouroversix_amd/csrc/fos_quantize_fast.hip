@@ -141,6 +141,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
     k.exact_ok = k.errdiv == 1536.0f && (amax_bits & (F16 ? 0x1fffu : 0xffffu)) == 0;
     k.shortcut_ok = shortcut_range(k.amax);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
+    // dither key: launch arguments, or read from device memory (a captured launch whose key the caller advances)
+    uint64_t key_seed = p.seed, key_offset = p.offset;
+    if (SR && p.key) {
+        key_seed = uniform64(p.key[0]);
+        key_offset = uniform64(p.key[1]);
+    }
     const bool in_range = k.amax >= 0x1p-100f && k.amax <= 0x1p100f;
     const float enc_fast = in_range ? k.enc : 0.0f;
     const float rq = 1.0f / k.qdiv, rc = 1.0f / p.c;
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
             if constexpr (IF4) o = quantize_block_if4_mse<false>(b, k, enc_fast, rq, in_range, lut);
             else if constexpr (kSpread) {
                 ExactRequest req;
-                o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct, true>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+                o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct, true>(b, k, enc_fast, rq, in_range, lut, key_seed, key_offset,
                                                                                     (uint64_t)(row * sf_cols + t.cb), &req);
                 const uint64_t asking = __builtin_amdgcn_ballot_w64(req.wanted);
                 if (asking != 0) {
@@ -182,7 +188,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu((SR ||
                         pick_second = exact_pick_b_1d_packed<RULE, F16>(b, o.c0, o.c1, req.b0, req.b1, lut[o.s & 0x7fu], lut[req.sB & 0x7fu]);
                     if (req.wanted && pick_second) o = BlockOut{req.b0, req.b1, req.sB};
                 }
-            } else o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct>(b, k, enc_fast, rq, in_range, lut, p.seed, p.offset,
+            } else o = quantize_block_nvfp4_fast<RULE, false, SR, F16, kProduct>(b, k, enc_fast, rq, in_range, lut, key_seed, key_offset,
                                                                                  (uint64_t)(row * sf_cols + t.cb));
         }
         if (PSEUDO) {

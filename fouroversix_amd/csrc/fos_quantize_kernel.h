@@ -33,6 +33,12 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
     k.exact_ok = k.errdiv == 1536.0f && (amax_bits & 0xffffu) == 0;
     k.shortcut_ok = shortcut_range(k.amax);
     if (blockIdx.x == 0 && threadIdx.x == 0 && p.amax_out) *p.amax_out = k.amax;
+    // dither key: launch arguments, or read from device memory (a captured launch whose key the caller advances)
+    uint64_t key_seed = p.seed, key_offset = p.offset;
+    if (ROUND != FOS_ROUND_NEAREST && p.key) {
+        key_seed = p.key[0];
+        key_offset = p.key[1];
+    }
 
     // The fast formulation assumes that no intermediate leaves the normal fp32 range,
     // which holds for 2^-100 <= amax <= 2^100; other tensors use the fallback throughout.
@@ -111,10 +117,10 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const QuantParams p)
             codes[1] = o.c1;
             sbyte = o.s;
         } else if (TYPED)
-            quantize_block_f32<DT, RULE, ROUND, TWO_D>(xf[it], k, p.seed, p.offset, (uint64_t)(r * sf_cols + cb), codes,
+            quantize_block_f32<DT, RULE, ROUND, TWO_D>(xf[it], k, key_seed, key_offset, (uint64_t)(r * sf_cols + cb), codes,
                                                        sbyte);
         else
-            quantize_block<DT, RULE, ROUND, TWO_D>(w[it], k, p.seed, p.offset, (uint64_t)(r * sf_cols + cb), codes,
+            quantize_block<DT, RULE, ROUND, TWO_D>(w[it], k, key_seed, key_offset, (uint64_t)(r * sf_cols + cb), codes,
                                                    sbyte);
         *reinterpret_cast<uint2 *>(p.codes + r * (p.cols_p >> 1) + cb * 8) = make_uint2(codes[0], codes[1]);
         if (p.sf_layout == FOS_SF_TILED_128X4) {

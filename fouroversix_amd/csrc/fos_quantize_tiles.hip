@@ -272,6 +272,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3
     k.rerr = sgpr(1.0f / k.errdiv);
     k.fast_div = in_range && k.errdiv == 1536.0f;
     k.shortcut_ok = shortcut_range(k.amax);
+    // dither key: launch arguments, or read from device memory (a captured launch whose key the caller advances)
+    uint64_t key_seed = p.seed, key_offset = p.offset;
+    if (SR && p.key) {
+        key_seed = uniform64(p.key[0]);
+        key_offset = uniform64(p.key[1]);
+    }
     // pseudo-quantize: the table also serves the dequantization (divisor c: the selection's for the adaptive
     // rules; the static rules make no selection, so their table is built with c)
     constexpr bool kStaticRule = RULE == FOS_RULE_STATIC_6 || RULE == FOS_RULE_STATIC_4;
@@ -452,7 +458,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3
         const uint32_t rstep = 32u * q + r;
         const int32_t row = t.row0 + (int32_t)rstep;
         uint32_t codes[2], sbyte;
-        quantize_block_f32<FOS_DTYPE_NVFP4, RULE, FOS_ROUND_STOCHASTIC, true>(x, k, p.seed, p.offset,
+        quantize_block_f32<FOS_DTYPE_NVFP4, RULE, FOS_ROUND_STOCHASTIC, true>(x, k, key_seed, key_offset,
                                                                               (uint64_t)((int64_t)row * sf_cols + cb_tile), codes, sbyte);
         if (PSEUDO) {
             uint32_t d[8];
@@ -516,7 +522,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(SR ? 3
             for (int s = 0; s < 4; ++s) {
                 if constexpr (IF4) block_candidates_if4(blk[s], A.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 else if constexpr (SR)
-                    block_candidates_sr<RULE>(blk[s], A.inv, B.inv, p.seed, p.offset, (uint64_t)((int64_t)(grow + 4 * s + li) * sf_cols + t.cb),
+                    block_candidates_sr<RULE>(blk[s], A.inv, B.inv, key_seed, key_offset, (uint64_t)((int64_t)(grow + 4 * s + li) * sf_cols + t.cb),
                                               oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 else block_candidates<RULE>(blk[s], A.inv, B.inv, oc[s][0], oc[s][1], cB[s][0], cB[s][1], SA, SB);
                 load(nt, 32 * nq + 4 * s, blk[s]);

@@ -75,9 +75,11 @@ Tensor amax_buffer(const c10::optional<Tensor> &amax, const Tensor &x) {
     return at::empty({1}, x.options().dtype(at::kFloat));
 }
 
-// quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax?) -> (values, scale_factors, amax)
+// quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax?, key?) -> (values, scale_factors, amax)
+// key: int64[2] on x's device holding {seed, offset}, read by the kernels when they run (seed / offset are then ignored)
 std::tuple<Tensor, Tensor, Tensor> quantize_ex(const Tensor &x, int64_t dtype, int64_t rule, int64_t round_style, bool is_2d,
-                                               int64_t seed, int64_t offset, int64_t sf_layout, const c10::optional<Tensor> &amax) {
+                                               int64_t seed, int64_t offset, int64_t sf_layout, const c10::optional<Tensor> &amax,
+                                               const c10::optional<Tensor> &key) {
     TORCH_CHECK(x.dim() == 2, "quantize: x must be 2-D");
     const int xt = type_id(x.scalar_type(), "quantize: x");
     TORCH_CHECK(x.stride(-1) == 1, "quantize: x must be contiguous on the last dim");
@@ -97,6 +99,16 @@ std::tuple<Tensor, Tensor, Tensor> quantize_ex(const Tensor &x, int64_t dtype, i
     const DeviceGuard guard(x.device());
     const fos_stream_t stream = current_stream(x);
     Tensor ws = quantize_workspace(x, stream);
+    if (key.has_value()) {
+        TORCH_CHECK(key->scalar_type() == at::kLong && key->numel() == 2 && key->is_contiguous() && key->device() == x.device(),
+                    "quantize: key must be a contiguous int64[2] tensor on x's device");
+        check(fos_quantize_devkey(x.data_ptr(), xt, rows, cols, x.stride(0), (int)dtype, (int)rule, (int)round_style, is_2d ? 1 : 0,
+                                  reinterpret_cast<const uint64_t *>(key->data_ptr<int64_t>()), (int)sf_layout, values.data_ptr<uint8_t>(),
+                                  static_cast<uint8_t *>(sf.data_ptr()), amax_buf.data_ptr<float>(), amax.has_value() ? 1 : 0,
+                                  ws.data_ptr(), (size_t)ws.numel(), stream),
+              "fouroversix::quantize");
+        return {values, sf, amax_buf};
+    }
     check(fos_quantize(x.data_ptr(), xt, rows, cols, x.stride(0), (int)dtype, (int)rule, (int)round_style, is_2d ? 1 : 0,
                        (uint64_t)seed, (uint64_t)offset, (int)sf_layout, values.data_ptr<uint8_t>(),
                        static_cast<uint8_t *>(sf.data_ptr()), amax_buf.data_ptr<float>(), amax.has_value() ? 1 : 0,
@@ -167,9 +179,9 @@ std::tuple<Tensor, Tensor, Tensor> quantize_ref(const Tensor &x, bool is_nvfp4, 
     const int64_t seed = rbits < 0 ? 0 : rbits;
     if (is_rht || is_transpose) {
         auto [y, amax] = transform(x, is_transpose, is_rht);
-        return quantize_ex(y, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, amax);
+        return quantize_ex(y, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, amax, c10::nullopt);
     }
-    return quantize_ex(x, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, c10::nullopt);
+    return quantize_ex(x, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, c10::nullopt, c10::nullopt);
 }
 
 // Operand checks of the reference's GEMM op (csrc/include/element_traits.hpp:122-170, csrc/fp4_gemm.cu:105-107).
@@ -322,7 +334,7 @@ TORCH_LIBRARY(fouroversix, m) {
         "int selection_rule, int rbits) -> (Tensor, Tensor, Tensor)");
     m.def(
         "quantize_ex(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, int seed, int offset, "
-        "int sf_layout, Tensor? amax) -> (Tensor, Tensor, Tensor)");
+        "int sf_layout, Tensor? amax, Tensor? key=None) -> (Tensor, Tensor, Tensor)");
     m.def("pseudo_quantize(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, Tensor? amax, int seed=0, int offset=0) -> Tensor");
     m.def("transform(Tensor x, bool transpose, bool rht) -> (Tensor, Tensor)");
     m.def("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");

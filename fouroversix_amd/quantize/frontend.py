@@ -118,7 +118,9 @@ def quantize(
 
     With no config: NVFP4, 1x16 blocks, round-to-nearest, 4/6 selection by block MSE.
     ``config.kwargs`` may carry ``seed`` / ``offset`` (ints) keying the dither of the
-    stochastic rounding styles (default: drawn from torch's global generator) and
+    stochastic rounding styles (default: drawn from torch's global generator), or ``key``
+    (an int64[2] tensor {seed, offset} on x's device, read when the kernels run: a call
+    recorded into a graph rounds with whatever the tensor holds at each replay), and
     ``amax`` (a tensor) to skip the tensor-wide maximum pass.
     """
     if config is None:
@@ -153,12 +155,15 @@ def quantize(
         q.original_shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
         return q
 
-    if config.round_style.is_stochastic and "seed" not in config.kwargs:
+    key = config.kwargs.get("key") if config.round_style.is_stochastic else None
+    if key is not None:
+        seed = 0  # (the kernels read {seed, offset} from the tensor when they run)
+    elif config.round_style.is_stochastic and "seed" not in config.kwargs:
         if x.is_cuda and torch.cuda.is_current_stream_capturing():
             # the seed is a launch argument: a graph replays the one drawn now, every time
             warnings.warn(
-                "stochastic rounding captured into a graph without kwargs['seed'] / kwargs['offset']: every replay "
-                "will round with the same random bits",
+                "stochastic rounding captured into a graph without kwargs['key'] (an int64[2] device tensor holding seed "
+                "and offset, which the captured code can advance): every replay will round with the same random bits",
                 stacklevel=2,
             )
         seed = int(torch.randint(0, 2**62, (1,)).item())
@@ -171,7 +176,7 @@ def quantize(
         # one fused kernel where the library has it, else the two-step round trip
         # (QuantizeBackendBase.pseudo_quantize, src/fouroversix/quantize/backend.py:213-234)
         fmt, style = NATIVE_FORMAT_IDS[config.dtype.value], config.round_style.native_id
-        if ops.pseudo_quantize_is_fused(x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d):
+        if key is None and ops.pseudo_quantize_is_fused(x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d):
             return ops.pseudo_quantize(
                 x, fmt, config.scale_rule.cuda_id, style, config.block_scale_2d, config.kwargs.get("amax", known_amax(x)), seed, offset
             )
@@ -193,6 +198,7 @@ def quantize(
         offset,
         nat.SF_LINEAR if linear else nat.SF_TILED,
         None if config.dtype == DataType.mxfp4 else config.kwargs.get("amax", known_amax(x)),  # mxfp4 has no tensor scale
+        key,
     )
     return QuantizedTensor.from_kernel(
         values,

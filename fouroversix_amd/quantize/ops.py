@@ -60,13 +60,14 @@ def quantize(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, r
     )
 
 
-def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax=None):
-    """Extended quantize: ``(values, scale_factors, amax)``."""
+def quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax=None, key=None):
+    """Extended quantize: ``(values, scale_factors, amax)``.  ``key``: int64[2] device tensor {seed, offset}
+    that the kernels read when they run, in place of the two integers (for launches recorded into a graph)."""
     seed, offset = seed & 0x7FFFFFFFFFFFFFFF, offset & 0x7FFFFFFFFFFFFFFF
     if _direct(x):
-        return _C.quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax)
+        return _C.quantize_ex(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax, key)
     return torch.ops.fouroversix.quantize_ex.default(
-        x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax
+        x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax, key
     )
 
 
@@ -144,7 +145,7 @@ def _(x, is_nvfp4, is_rtn, is_rht, is_2d, is_transpose, selection_rule, rbits):
 
 
 @torch.library.register_fake("fouroversix::quantize_ex")
-def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax):
+def _(x, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout, amax, key=None):
     return _fake_quantize_shapes(x, dtype)
 
 

@@ -154,6 +154,20 @@ int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t
                   void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * fos_quantize with the dither key of the stochastic styles read by the kernels from device memory:
+ * key[0] = seed, key[1] = offset (8-byte aligned, read when the kernels run).  For launches recorded into a
+ * HIP graph, whose scalar arguments are frozen at capture: the caller advances key[1] between replays (a
+ * small kernel of its own, recorded with the rest) and every replay rounds with fresh bits.  Same results
+ * as fos_quantize called with the values the key holds.  No counterpart in the reference, whose kernels take
+ * their random bits as launch arguments (src/fouroversix/csrc/quantize/fp4_quant.cu:134-136).
+ */
+int fos_quantize_devkey(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                        int dtype, int rule, int round_style, int block2d,
+                        const uint64_t *key, int sf_layout,
+                        uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
+                        void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * Fused quantize -> dequantize round trip: out[rows, cols] (bf16, leading dimension ldo) =
  * the values fos_dequantize would return for fos_quantize's result, without materialising
  * codes or scales.  Stands in for QuantizeBackendBase.pseudo_quantize

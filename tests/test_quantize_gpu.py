@@ -486,6 +486,60 @@ def test_two_pass_quantize_replays_in_a_hip_graph():
         assert float(static_q.amax) == float(eager.amax), f"replay {i}"
 
 
+@pytest.mark.parametrize(("shape", "cfg"), [
+    ((256, 512), dict(scale_rule="mse")), ((256, 512), dict(scale_rule="mse", block_scale_2d=True)),
+    ((100, 80), dict(scale_rule="mae", block_scale_2d=True)), ((128, 256), dict(scale_rule="static_6", round_style="stochastic_unbiased")),
+    ((128, 256), dict(dtype="if4", scale_rule="mse")), ((128, 264), dict(scale_rule="abs_max", round_style="stochastic_unbiased")),
+])
+def test_dither_key_read_from_device_memory(shape, cfg):
+    """kwargs['key'] (int64[2] on the device: seed, offset) gives the bytes of the same two integers passed as
+    launch arguments, on every kernel that rounds stochastically (streaming 1x16 and 16x16, element-wise)."""
+    kw = {"round_style": "stochastic", **cfg}
+    x = make_input("randn", shape, 60).cuda()
+    key = torch.tensor([2**40 + 99, 3], dtype=torch.int64, device="cuda")
+    for src in (x, x.float()):
+        q = fos.quantize(src, fos.QuantizationConfig(**kw, kwargs={"key": key}))
+        ref = fos.quantize(src, fos.QuantizationConfig(**kw, kwargs={"seed": 2**40 + 99, "offset": 3}))
+        assert torch.equal(q.values, ref.values) and torch.equal(q.scale_factors.view(torch.uint8), ref.scale_factors.view(torch.uint8))
+    p = fos.quantize(x, fos.QuantizationConfig(**kw, pseudo_quantize=True, kwargs={"key": key}))
+    ref = fos.quantize(x, fos.QuantizationConfig(**kw, kwargs={"seed": 2**40 + 99, "offset": 3}))
+    assert torch.equal(p, fos.dequantize(ref, dtype=x.dtype))
+    with pytest.raises(RuntimeError, match="key"):
+        fos.quantize(x, fos.QuantizationConfig(**kw, kwargs={"key": key.int()}))
+
+
+def test_captured_stochastic_rounding_advances_its_key():
+    """A stochastic quantize recorded into a HIP graph together with an increment of its key's offset rounds
+    with fresh bits on every replay: replay i equals the eager call with offset i (a launch argument would
+    freeze the bits drawn at capture)."""
+    cfg = dict(scale_rule="mse", round_style="stochastic")
+    x = make_input("randn", (512, 1024), 61).cuda()
+    key = torch.tensor([7, 0], dtype=torch.int64, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fos.quantize(x, fos.QuantizationConfig(**cfg, kwargs={"key": key}))
+            key[1:].add_(1)
+    torch.cuda.current_stream().wait_stream(side)
+    key.copy_(torch.tensor([7, 0], dtype=torch.int64))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_q = fos.quantize(x, fos.QuantizationConfig(**cfg, kwargs={"key": key}))
+        key[1:].add_(1)
+    seen = []
+    for i in range(4):
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = fos.quantize(x, fos.QuantizationConfig(**cfg, kwargs={"seed": 7, "offset": i}))
+        torch.cuda.synchronize()
+        assert torch.equal(static_q.values, eager.values), f"replay {i}"
+        assert torch.equal(static_q.scale_factors.view(torch.uint8), eager.scale_factors.view(torch.uint8)), f"replay {i}"
+        seen.append(static_q.values.clone())
+    assert not torch.equal(seen[0], seen[1])
+    assert int(key[1]) == 4
+
+
 @pytest.mark.parametrize("shape", [(16, 4096), (4, 4096), (16, 1024), (1, 8192), (16, 4064)])
 def test_decode_sized_quantize_eager_and_captured(oracle, shape):
     """Decode-sized inputs take one launch (every workgroup scans the tensor for its maximum) up to
