@@ -49,6 +49,48 @@ def test_static_entry_point_matches_fos_quantize_on_two_calls_in_a_row():
         assert np.array_equal(got[1], want[1]), "scales differ"
 
 
+def test_static_entry_point_leaves_device_memory_alone_and_replays_in_a_graph():
+    """What the entry point is for: the free device memory is the same before and after a call (nothing is
+    allocated once the first call has looked the scratch array up), and a call recorded into a HIP graph
+    -- where an allocation would fail -- gives fos_quantize's bytes on every replay, on new contents."""
+    dev = torch.device("cuda:0")
+    L = nat.lib()
+    g = torch.Generator("cpu").manual_seed(12)
+    x = torch.randn(1024, 2048, generator=g).bfloat16().to(dev)  # 4 MiB: two launches (tensor maximum, then codes)
+    rows, cols = x.shape
+    codes = torch.empty(rows, cols // 2, dtype=torch.uint8, device=dev)
+    sf = torch.empty(rows * cols // 16, dtype=torch.uint8, device=dev)
+    amax = torch.empty(1, dtype=torch.float32, device=dev)
+    workspace = torch.empty(L.fos_quantize_workspace_bytes(rows, cols), dtype=torch.uint8, device=dev)
+
+    def static_call(stream):
+        rc = L.fos_quantize_static(x.data_ptr(), nat.T_BF16, rows, cols, cols, 0, MSE, 0, 0, 0, 0, nat.SF_TILED,
+                                   codes.data_ptr(), sf.data_ptr(), amax.data_ptr(), 0, stream)
+        assert rc == 0, L.fos_error_string(rc)
+
+    static_call(torch.cuda.current_stream(dev).cuda_stream)  # (looks the scratch array up)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    static_call(torch.cuda.current_stream(dev).cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_call(torch.cuda.current_stream(dev).cuda_stream)
+    for i in range(2):
+        xi = (float(i + 2) * torch.randn(rows, cols, generator=g)).bfloat16().to(dev)
+        x.copy_(xi)
+        codes.fill_(0xAB)
+        sf.fill_(0xCD)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _call("plain", xi, MSE, 0, nat.SF_TILED, workspace)
+        assert float(amax) == want[2] == float(xi.abs().max())
+        assert np.array_equal(codes.cpu().numpy(), want[0]), f"replay {i}: codes differ"
+        assert np.array_equal(sf.cpu().numpy(), want[1]), f"replay {i}: scales differ"
+
+
 def test_static_entry_point_argument_checks():
     L = nat.lib()
     dev = torch.device("cuda:0")
