@@ -21,6 +21,7 @@ void load_tuning() {
     g_tuning.quant_grid = env_int("FOS_QUANT_GRID");
     g_tuning.amax_grid = env_int("FOS_AMAX_GRID");
     g_tuning.quant_map = env_int("FOS_QUANT_MAP");
+    g_tuning.quant_passes = env_int("FOS_QUANT_PASSES");
     g_tuning.amax_units = env_int("FOS_AMAX_UNITS");
 }
 }  // namespace

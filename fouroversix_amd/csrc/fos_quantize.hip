@@ -464,6 +464,8 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
         p.amax_out = amax;
     }
 
+    if (tuning().quant_passes == 1) return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;  // timing runs: pass 1 alone
+
     // (qmax, smax): static_6 (6,448); static_4 (4,448); adaptive NVFP4 (6,256); IF4 (6,448).
     const double adj = round_style == FOS_ROUND_STOCHASTIC_UNBIASED ? 16.0 / 17.0 : 1.0;
     const double qmax = rule == FOS_RULE_STATIC_4 ? 4.0 : 6.0;

@@ -16,6 +16,7 @@ struct Tuning {
     std::atomic<int> amax_grid{0};    // FOS_AMAX_GRID
     std::atomic<int> amax_units{0};   // FOS_AMAX_UNITS: -1 = flat pass 1 also ahead of a streaming pass 2
     std::atomic<int> quant_map{0};    // FOS_QUANT_MAP: tile order of the streaming quantize kernels (1 + TileMap)
+    std::atomic<int> quant_passes{0};  // FOS_QUANT_PASSES: 1 = fos_quantize stops after the tensor-maximum pass (timing runs: what pass 2 adds to a step)
 };
 
 const Tuning &tuning();
