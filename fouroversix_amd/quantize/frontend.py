@@ -98,14 +98,15 @@ def attach_known_amax(x: torch.Tensor, amax: torch.Tensor) -> torch.Tensor:
     on tensors that have no version counter (inference tensors)."""
     version = _version_or_none(x)
     if version is not None:
-        setattr(x, _KNOWN_AMAX, (amax, version))
+        # (address and shape as well: a tag copied along with the object's attributes onto other storage is not believed)
+        setattr(x, _KNOWN_AMAX, (amax, version, x.data_ptr(), x.shape))
     return x
 
 
 def known_amax(x: torch.Tensor) -> torch.Tensor | None:
     """The maximum recorded by ``attach_known_amax`` if ``x`` has not been written since."""
     tag = getattr(x, _KNOWN_AMAX, None)
-    if tag is None or tag[0].device != x.device or tag[1] != _version_or_none(x):
+    if tag is None or tag[0].device != x.device or tag[1] != _version_or_none(x) or tag[2] != x.data_ptr() or tag[3] != x.shape:
         return None
     return tag[0]
 
