@@ -486,6 +486,38 @@ def test_two_pass_quantize_replays_in_a_hip_graph():
         assert float(static_q.amax) == float(eager.amax), f"replay {i}"
 
 
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_configurations_match_the_oracle(oracle, seed):
+    """120 configurations per seed drawn over shape (whole and ragged workgroup tiles, single rows), format, rule,
+    rounding style, block shape, input type, input kind and tensor scale: codes, scales and maximum are the
+    oracle's, and a fused round trip equals dequantize(quantize(x)) bit for bit."""
+    import random
+
+    rng = random.Random(seed)
+    for it in range(120):
+        rows = rng.choice([1, 16, 37, 100, 128, 130, 256, 384, 512, 777])
+        cols = rng.choice([16, 48, 80, 256, 272, 512, 528, 1024, 1040, 2048])
+        fmt = rng.choice(["nvfp4", "nvfp4", "nvfp4", "if4"])
+        rule = rng.choice(["mse", "mae", "abs_max"] + ([] if fmt == "if4" else ["static_6", "static_4"]))
+        kw = dict(dtype=fmt, scale_rule=rule, round_style=rng.choice(["nearest", "stochastic", "stochastic", "stochastic_unbiased"]),
+                  block_scale_2d=rng.random() < 0.5)
+        kind = rng.choice(["randn", "outlier", "tiny_blocks", "weight", "rand01"])
+        if kind == "tiny_blocks" and cols % 16:
+            kind = "randn"
+        scale = rng.choice([1.0, 1.0, 2.0**-20, 2.0**30, 2.0**-50, 3e4])
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        x = make_input(kind, (rows, cols), 1000 * seed + it).float() * scale
+        x = (x.clamp(-6e4, 6e4) if dtype == torch.float16 else x).to(dtype)
+        key = dict(seed=rng.randrange(2**40), offset=rng.randrange(100))
+        what = f"case {it}: {rows}x{cols} {kw} {kind} x {scale} {dtype} {key}"
+        q = fos.quantize(x.cuda(), fos.QuantizationConfig(**kw, kwargs=key))
+        assert_same_quantization(q, oracle.quantize(x, **key, **kw), what)
+        if rng.random() < 0.3:
+            p = fos.quantize(x.cuda(), fos.QuantizationConfig(**kw, pseudo_quantize=True, kwargs=key))
+            bits = torch.int32 if dtype == torch.float32 else torch.int16
+            assert torch.equal(p.view(bits), fos.dequantize(q, dtype=dtype).view(bits)), what
+
+
 @pytest.mark.parametrize(("shape", "cfg"), [
     ((256, 512), dict(scale_rule="mse")), ((256, 512), dict(scale_rule="mse", block_scale_2d=True)),
     ((100, 80), dict(scale_rule="mae", block_scale_2d=True)), ((128, 256), dict(scale_rule="static_6", round_style="stochastic_unbiased")),
