@@ -35,6 +35,7 @@ EXPORTS = (
     "fos_pseudo_quantize_keyed",
     "fos_pseudo_quantize_is_fused",
     "fos_transform",
+    "fos_transform_quantize",
     "fos_gemm_nvfp4",
     "fos_gemm_nvfp4_amax",
     "fos_gemm_nvfp4_amax_out",
@@ -95,6 +96,8 @@ def lib() -> ctypes.CDLL:
     L.fos_pseudo_quantize_is_fused.restype = i32
     L.fos_transform.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, i64, vp, vp, sz, vp]
     L.fos_transform.restype = i32
+    L.fos_transform_quantize.argtypes = [vp, i32, i64, i64, i64, i32, i32, vp, i64, i32, i32, i32, i32, u64, u64, i32, vp, vp, vp, vp, sz, vp]
+    L.fos_transform_quantize.restype = i32
     L.fos_gemm_nvfp4.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]
     L.fos_gemm_nvfp4.restype = i32
     L.fos_gemm_nvfp4_amax.argtypes = [vp, vp, vp, vp, vp, vp, dbl, i64, i64, i64, vp, i32, i64, vp, ctypes.c_size_t, vp]

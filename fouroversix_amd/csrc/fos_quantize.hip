@@ -386,7 +386,7 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
                          uint64_t seed, uint64_t offset, int sf_layout,
                          uint8_t *codes, uint8_t *sf, float *amax, int amax_is_input,
                          void *workspace, size_t workspace_bytes, fos_stream_t stream,
-                         uint16_t *pseudo_out, int64_t ldo, const uint64_t *key = nullptr) {
+                         uint16_t *pseudo_out, int64_t ldo, const uint64_t *key = nullptr, int ready_partials = 0) {
     if (!x || !amax || (!pseudo_out && (!codes || !sf))) return FOS_E_NULL_POINTER;
     if ((uintptr_t)key & 7) return FOS_E_BAD_ALIGNMENT;
     if (dtype == FOS_DTYPE_MXFP4) {
@@ -448,7 +448,12 @@ static int quantize_impl(const void *x, int x_type, int64_t rows, int64_t cols, 
     p.key = key;
     p.sf_layout = sf_layout;
 
-    if (amax_is_input) {
+    if (ready_partials > 0) {
+        // the producer of x (fos_transform) has left its per-workgroup maxima in the workspace
+        p.partials = partials;
+        p.n_partials = ready_partials;
+        p.amax_out = amax;
+    } else if (amax_is_input) {
         p.partials = (const uint32_t *)amax;
         p.n_partials = 0;
         p.amax_out = nullptr;
@@ -515,6 +520,29 @@ extern "C" int fos_quantize_devkey(const void *x, int x_type, int64_t rows, int6
     if (dtype == FOS_DTYPE_MXFP4) return FOS_E_UNSUPPORTED;  // (no stochastic style there)
     return quantize_impl(x, x_type, rows, cols, ld, dtype, rule, round_style, block2d, 0, 0, sf_layout, codes, sf,
                          amax, amax_is_input, workspace, workspace_bytes, stream, nullptr, 0, key);
+}
+
+namespace fos {
+int transform_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, int transpose, int rht, void *y, int64_t ldy,
+                   float *amax, int *n_partials, void *workspace, size_t workspace_bytes, fos_stream_t stream);
+}
+
+extern "C" int fos_transform_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                                      int transpose, int rht, void *y, int64_t ldy,
+                                      int dtype, int rule, int round_style, int block2d,
+                                      uint64_t seed, uint64_t offset, int sf_layout,
+                                      uint8_t *codes, uint8_t *sf, float *amax,
+                                      void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!amax || !codes || !sf) return FOS_E_NULL_POINTER;
+    if (dtype != FOS_DTYPE_NVFP4 && dtype != FOS_DTYPE_IF4) return FOS_E_UNSUPPORTED;  // (MXFP4 has no tensor maximum to hand over)
+    int n = 0;
+    const int rc = fos::transform_impl(x, x_type, rows, cols, ld, transpose, rht, y, ldy, nullptr, &n, workspace, workspace_bytes, stream);
+    if (rc != FOS_OK) return rc;
+    const int64_t out_rows = transpose ? cols : rows, out_cols = transpose ? rows : cols;
+    // with rht a ragged last group of 16 holds values in all its places: the padded width is what gets quantized
+    const int64_t q_cols = rht ? (out_cols + 15) / 16 * 16 : out_cols;
+    return quantize_impl(y, x_type, out_rows, q_cols, ldy, dtype, rule, round_style, block2d, seed, offset, sf_layout, codes, sf,
+                         amax, 0, workspace, workspace_bytes, stream, nullptr, 0, nullptr, n);
 }
 
 extern "C" int fos_pseudo_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,

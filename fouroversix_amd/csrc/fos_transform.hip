@@ -305,12 +305,18 @@ __global__ __launch_bounds__(kThreads) void transform_amax_kernel(const uint32_t
 
 }  // namespace fos
 
+namespace fos {
+int transform_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld, int transpose, int rht, void *y, int64_t ldy,
+                   float *amax, int *n_partials, void *workspace, size_t workspace_bytes, fos_stream_t stream);
+}
 using namespace fos;
 
-extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
-                             int transpose, int rht, void *y, int64_t ldy, float *amax,
-                             void *workspace, size_t workspace_bytes, fos_stream_t stream) {
-    if (!x || !y || !amax) return FOS_E_NULL_POINTER;
+// Body of fos_transform.  `amax` null: the reduction kernel is left out and *n_partials tells how many
+// {maximum, reserved} pairs the transform left in the workspace (for a pass 2 that reduces them itself).
+int fos::transform_impl(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                        int transpose, int rht, void *y, int64_t ldy, float *amax, int *n_partials,
+                        void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!x || !y || (!amax && !n_partials)) return FOS_E_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || ld < cols) return FOS_E_BAD_SHAPE;
     if ((x_type != FOS_T_BF16 && x_type != FOS_T_F16 && x_type != FOS_T_F32) || (!transpose && !rht)) return FOS_E_UNSUPPORTED;
     const bool f16 = x_type == FOS_T_F16;
@@ -335,7 +341,8 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
         if (transpose && rht) hipLaunchKernelGGL((transform_f32_kernel<true, true>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
         else if (transpose) hipLaunchKernelGGL((transform_f32_kernel<true, false>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
         else hipLaunchKernelGGL((transform_f32_kernel<false, true>), dim3((unsigned)grid32), dim3(kThreads), 0, s32, q);
-        hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s32, q.partials, (int)grid32, amax);
+        if (n_partials) *n_partials = (int)grid32;
+        if (amax) hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s32, q.partials, (int)grid32, amax);
         return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
     }
     if (((uintptr_t)x & 1) || ((uintptr_t)y & 15) || (ldy % 8 != 0) || ((uintptr_t)workspace & 7) || ((uintptr_t)amax & 3))
@@ -366,6 +373,14 @@ extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t co
         if (f16) hipLaunchKernelGGL(rht_rows_kernel<true>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
         else hipLaunchKernelGGL(rht_rows_kernel<false>, dim3((unsigned)grid), dim3(kThreads), 0, s, p);
     }
-    hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s, p.partials, (int)grid, amax);
+    if (n_partials) *n_partials = (int)grid;
+    if (amax) hipLaunchKernelGGL(transform_amax_kernel, dim3(1), dim3(kThreads), 0, s, p.partials, (int)grid, amax);
     return hipGetLastError() == hipSuccess ? FOS_OK : FOS_E_LAUNCH;
+}
+
+extern "C" int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                             int transpose, int rht, void *y, int64_t ldy, float *amax,
+                             void *workspace, size_t workspace_bytes, fos_stream_t stream) {
+    if (!amax) return FOS_E_NULL_POINTER;
+    return transform_impl(x, x_type, rows, cols, ld, transpose, rht, y, ldy, amax, nullptr, workspace, workspace_bytes, stream);
 }

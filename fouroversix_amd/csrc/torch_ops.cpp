@@ -168,6 +168,35 @@ std::tuple<Tensor, Tensor> transform(const Tensor &x_in, bool transpose, bool rh
     return {y, amax};
 }
 
+// transform, then quantize_ex of its result, in one call into the library (one small kernel and one dispatch less):
+// (values, scale_factors, amax) of the transformed tensor
+std::tuple<Tensor, Tensor, Tensor> transform_quantize(const Tensor &x_in, bool transpose, bool rht, int64_t dtype, int64_t rule,
+                                                      int64_t round_style, bool is_2d, int64_t seed, int64_t offset, int64_t sf_layout) {
+    TORCH_CHECK(x_in.dim() == 2 && (x_in.scalar_type() == at::kBFloat16 || x_in.scalar_type() == at::kHalf || x_in.scalar_type() == at::kFloat),
+                "transform_quantize: x must be a 2-D bfloat16, float16 or float32 tensor");
+    TORCH_CHECK(x_in.numel() > 0 && (transpose || rht), "transform_quantize: a non-empty tensor and at least one of transpose / rht");
+    require_gpu(x_in, "x");
+    const Tensor x = x_in.stride(-1) == 1 ? x_in : x_in.contiguous();
+    const int64_t rows = x.size(0), cols = x.size(1);
+    const int64_t out_rows = transpose ? cols : rows, out_cols = transpose ? rows : cols;
+    const int64_t width = (out_cols + 15) / 16 * 16;
+    Tensor y = at::empty({out_rows, width}, x.options());
+    const auto [rows_p, cols_p] = padded(out_rows, rht ? width : out_cols, dtype);
+    const auto bytes = x.options().dtype(at::kByte);
+    Tensor values = at::empty({rows_p, cols_p / 2}, bytes);
+    Tensor sf = at::empty({rows_p * cols_p / 16}, x.options().dtype(at::kFloat8_e4m3fn));
+    Tensor amax = at::empty({1}, x.options().dtype(at::kFloat));
+    const DeviceGuard guard(x.device());
+    const fos_stream_t stream = current_stream(x);
+    Tensor ws = quantize_workspace(x, stream);
+    check(fos_transform_quantize(x.data_ptr(), type_id(x.scalar_type(), "transform_quantize: x"), rows, cols, x.stride(0), transpose ? 1 : 0,
+                                 rht ? 1 : 0, y.data_ptr(), y.stride(0), (int)dtype, (int)rule, (int)round_style, is_2d ? 1 : 0,
+                                 (uint64_t)seed, (uint64_t)offset, (int)sf_layout, values.data_ptr<uint8_t>(),
+                                 static_cast<uint8_t *>(sf.data_ptr()), amax.data_ptr<float>(), ws.data_ptr(), (size_t)ws.numel(), stream),
+          "fouroversix::transform_quantize");
+    return {values, sf, amax};
+}
+
 // The reference's schema (csrc/bindings.cpp:28): NVFP4 only; `rbits` seeds the stochastic style.
 std::tuple<Tensor, Tensor, Tensor> quantize_ref(const Tensor &x, bool is_nvfp4, bool is_rtn, bool is_rht, bool is_2d, bool is_transpose,
                                                 int64_t selection_rule, int64_t rbits) {
@@ -177,10 +206,8 @@ std::tuple<Tensor, Tensor, Tensor> quantize_ref(const Tensor &x, bool is_nvfp4, 
     TORCH_CHECK(x.scalar_type() == at::kHalf || x.scalar_type() == at::kBFloat16, "quantize: x must be bfloat16 or float16, got ",
                 x.scalar_type());
     const int64_t seed = rbits < 0 ? 0 : rbits;
-    if (is_rht || is_transpose) {
-        auto [y, amax] = transform(x, is_transpose, is_rht);
-        return quantize_ex(y, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, amax, c10::nullopt);
-    }
+    if (is_rht || is_transpose)
+        return transform_quantize(x, is_transpose, is_rht, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4);
     return quantize_ex(x, FOS_DTYPE_NVFP4, selection_rule, is_rtn ? 0 : 1, is_2d, seed, 0, FOS_SF_TILED_128X4, c10::nullopt, c10::nullopt);
 }
 
@@ -337,6 +364,9 @@ TORCH_LIBRARY(fouroversix, m) {
         "int sf_layout, Tensor? amax, Tensor? key=None) -> (Tensor, Tensor, Tensor)");
     m.def("pseudo_quantize(Tensor x, int dtype, int selection_rule, int round_style, bool is_2d, Tensor? amax, int seed=0, int offset=0) -> Tensor");
     m.def("transform(Tensor x, bool transpose, bool rht) -> (Tensor, Tensor)");
+    m.def(
+        "transform_quantize(Tensor x, bool transpose, bool rht, int dtype, int selection_rule, int round_style, bool is_2d, "
+        "int seed, int offset, int sf_layout) -> (Tensor, Tensor, Tensor)");
     m.def("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");
     m.def("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");
     m.def("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt(Tensor A, Tensor B, Tensor A_sf, Tensor B_sf, Tensor alpha) -> Tensor");
@@ -353,6 +383,7 @@ TORCH_LIBRARY_IMPL(fouroversix, CUDA, m) {
     m.impl("quantize_ex", &quantize_ex);
     m.impl("pseudo_quantize", &pseudo_quantize);
     m.impl("transform", &transform);
+    m.impl("transform_quantize", &transform_quantize);
     m.impl("gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt", &gemm_nvfp4_bf16);
     m.impl("gemm_nvfp4nvfp4_accum_fp32_out_fp16_tnt", &gemm_nvfp4_fp16);
     m.impl("gemm_mxfp4mxfp4_accum_fp32_out_bf16_tnt", &gemm_mxfp4_bf16);
@@ -366,6 +397,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pseudo_quantize", &pseudo_quantize);
     m.def("pseudo_quantize_is_fused", &pseudo_quantize_is_fused);
     m.def("transform", &transform);
+    m.def("transform_quantize", &transform_quantize);
     m.def("gemm_nvfp4", &gemm_nvfp4);
     m.def("gemm_nvfp4_amax", &gemm_nvfp4_amax);
     m.def("gemm_alpha", &gemm_alpha);

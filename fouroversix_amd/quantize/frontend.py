@@ -138,24 +138,6 @@ def quantize(
             msg = f"Backend {config.backend} does not support the given parameters ({reason})"
         raise ValueError(msg)
 
-    if config.transpose or config.rht:
-        # x.T and / or the random Hadamard transform first (reference
-        # quantize/pytorch/reference.py:567-571), as one pass that also yields the tensor
-        # maximum; the rest is the plain path on the transformed tensor
-        if "amax" in config.kwargs:
-            msg = "kwargs['amax'] cannot be combined with transpose / rht (the maximum is that of the transformed tensor)"
-            raise ValueError(msg)
-        y, amax = ops.transform(x, config.transpose, config.rht)
-        plain = QuantizationConfig(
-            **{**config.__dict__, "transpose": False, "rht": False, "kwargs": {**config.kwargs, "amax": amax}}
-        )
-        q = quantize(y, plain)
-        # the logical shape is that of x (transposed); a ragged width that the Hadamard transform
-        # filled up to a multiple of 16 keeps its codes in the padding, as in the reference
-        # (src/fouroversix/quantize/pytorch/backend.py:57-79,110-121)
-        q.original_shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
-        return q
-
     key = config.kwargs.get("key") if config.round_style.is_stochastic else None
     if key is not None:
         seed = 0  # (the kernels read {seed, offset} from the tensor when they run)
@@ -172,6 +154,57 @@ def quantize(
         seed = int(config.kwargs.get("seed", config.kwargs.get("rbits", 0)))
         seed = max(seed, 0)
     offset = int(config.kwargs.get("offset", 0))
+
+    if config.transpose or config.rht:
+        # x.T and / or the random Hadamard transform first (reference
+        # quantize/pytorch/reference.py:567-571), as one pass that also yields the tensor
+        # maximum; the rest is the plain path on the transformed tensor
+        if "amax" in config.kwargs:
+            msg = "kwargs['amax'] cannot be combined with transpose / rht (the maximum is that of the transformed tensor)"
+            raise ValueError(msg)
+        # the logical shape is that of x (transposed); a ragged width that the Hadamard transform
+        # filled up to a multiple of 16 keeps its codes in the padding, as in the reference
+        # (src/fouroversix/quantize/pytorch/backend.py:57-79,110-121)
+        logical_shape = (x.shape[1], x.shape[0]) if config.transpose else tuple(x.shape)
+        if not config.pseudo_quantize and key is None and config.dtype != DataType.mxfp4:
+            # both steps in one call into the library (pass 2 reduces the transform's partial maxima itself)
+            linear = config.dtype in _LINEAR_SCALE_FORMATS
+            values, scale_factors, amax = ops.transform_quantize(
+                x,
+                config.transpose,
+                config.rht,
+                NATIVE_FORMAT_IDS[config.dtype.value],
+                config.scale_rule.cuda_id,
+                config.round_style.native_id,
+                config.block_scale_2d,
+                seed,
+                offset,
+                nat.SF_LINEAR if linear else nat.SF_TILED,
+            )
+            return QuantizedTensor.from_kernel(
+                values,
+                scale_factors,
+                amax.reshape(()),
+                config.dtype,
+                logical_shape,
+                config.scale_rule,
+                config.round_style,
+                (values.shape[0], values.shape[1] * config.dtype.quantized_value_type.packing_factor),
+                not linear,
+            )
+        y, amax = ops.transform(x, config.transpose, config.rht)
+        plain = QuantizationConfig(
+            **{
+                **config.__dict__,
+                "transpose": False,
+                "rht": False,
+                "kwargs": {**config.kwargs, "amax": amax, "seed": seed, "offset": offset},
+            }
+        )
+        q = quantize(y, plain)
+        if isinstance(q, QuantizedTensor):
+            q.original_shape = logical_shape
+        return q
 
     if config.pseudo_quantize:
         # one fused kernel where the library has it, else the two-step round trip

@@ -78,6 +78,17 @@ def transform(x, transpose, rht):
     return torch.ops.fouroversix.transform.default(x, transpose, rht)
 
 
+def transform_quantize(x, transpose, rht, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout):
+    """``transform`` and ``quantize_ex`` of its result in one call into the library: ``(values, scale_factors,
+    amax)`` of the transformed tensor (NVFP4 / IF4)."""
+    seed, offset = seed & 0x7FFFFFFFFFFFFFFF, offset & 0x7FFFFFFFFFFFFFFF
+    if _direct(x):
+        return _C.transform_quantize(x, transpose, rht, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout)
+    return torch.ops.fouroversix.transform_quantize.default(
+        x, transpose, rht, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout
+    )
+
+
 def pseudo_quantize(x, dtype, selection_rule, round_style, is_2d, amax=None, seed=0, offset=0):
     """Fused quantize -> dequantize (out has x's type); see ``pseudo_quantize_is_fused``.  ``seed`` /
     ``offset`` key the dither of the stochastic styles, as in ``quantize_ex``."""
@@ -179,6 +190,13 @@ def _(x, transpose, rht):
     rows, cols = (x.shape[1], x.shape[0]) if transpose else (x.shape[0], x.shape[1])
     width = -(-cols // 16) * 16 if rht else cols
     return torch.empty(rows, width, dtype=x.dtype, device=x.device), torch.empty(1, dtype=torch.float32, device=x.device)
+
+
+@torch.library.register_fake("fouroversix::transform_quantize")
+def _(x, transpose, rht, dtype, selection_rule, round_style, is_2d, seed, offset, sf_layout):
+    rows, cols = (x.shape[1], x.shape[0]) if transpose else (x.shape[0], x.shape[1])
+    width = -(-cols // 16) * 16 if rht else cols
+    return _fake_quantize_shapes(torch.empty(rows, width, dtype=x.dtype, device=x.device), dtype)
 
 
 @torch.library.register_fake("fouroversix::gemm_nvfp4_amax")

@@ -154,6 +154,22 @@ int fos_transform(const void *x, int x_type, int64_t rows, int64_t cols, int64_t
                   void *workspace, size_t workspace_bytes, fos_stream_t stream);
 
 /*
+ * fos_transform followed by fos_quantize of its result, without the small kernel that reduces the
+ * transform's per-workgroup maxima to one number in between: the quantizer's second pass reduces them
+ * itself, as it does behind its own first pass.  y [out_rows, ldy] receives the transformed tensor (the
+ * caller may discard it); codes / sf / amax are those of fos_quantize(y, ...) -- rows = cols of x when
+ * transposing, width rounded up to 16 with rht -- byte for byte.  One workspace serves both steps.
+ * FOS_DTYPE_NVFP4 and FOS_DTYPE_IF4.  Stands in for the transpose / rht options of
+ * quantize_to_fp4 (src/fouroversix/quantize/pytorch/reference.py:567-578) in one call.
+ */
+int fos_transform_quantize(const void *x, int x_type, int64_t rows, int64_t cols, int64_t ld,
+                           int transpose, int rht, void *y, int64_t ldy,
+                           int dtype, int rule, int round_style, int block2d,
+                           uint64_t seed, uint64_t offset, int sf_layout,
+                           uint8_t *codes, uint8_t *sf, float *amax,
+                           void *workspace, size_t workspace_bytes, fos_stream_t stream);
+
+/*
  * fos_quantize with the dither key of the stochastic styles read by the kernels from device memory:
  * key[0] = seed, key[1] = offset (8-byte aligned, read when the kernels run).  For launches recorded into a
  * HIP graph, whose scalar arguments are frozen at capture: the caller advances key[1] between replays (a

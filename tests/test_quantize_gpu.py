@@ -1072,6 +1072,25 @@ def test_fp16_transform_matches_reference_vectors_and_oracle(oracle, golden_dir)
             assert_same_quantization(q, ref, f"fp16 {shape} transpose={transpose} rht={rht}")
 
 
+@pytest.mark.parametrize(("shape", "dtype"), [((512, 1024), torch.bfloat16), ((100, 200), torch.bfloat16), ((256, 384), torch.float16),
+                                              ((130, 272), torch.float32)])
+@pytest.mark.parametrize(("transpose", "rht"), [(True, False), (False, True), (True, True)])
+def test_transform_and_quantize_in_one_call_equals_the_two_calls(shape, dtype, transpose, rht):
+    """fos_transform_quantize (the frontend's path for the transpose / rht options) leaves out the kernel that
+    reduces the transform's partial maxima; its bytes are those of transform, then quantize with that maximum."""
+    from fouroversix_amd import _native as nat
+    from fouroversix_amd.quantize import ops
+
+    x = (make_input("outlier", shape, 41).float() * 1.37).to(dtype).cuda()
+    for fmt, rule, style, two_d in ((0, 3, 0, False), (0, 0, 1, False), (1, 3, 0, False)) + (((0, 3, 0, True),) if shape[0] % 16 == 0 else ()):
+        y, amax = ops.transform(x, transpose, rht)
+        layout = nat.SF_LINEAR if fmt == 1 else nat.SF_TILED
+        want = ops.quantize_ex(y, fmt, rule, style, two_d, 5, 2, layout, amax)
+        got = ops.transform_quantize(x, transpose, rht, fmt, rule, style, two_d, 5, 2, layout)
+        for g, w, name in zip(got, want, ("values", "scales", "amax")):
+            assert torch.equal(g.view(torch.uint8), w.view(torch.uint8)), f"{name} fmt {fmt} rule {rule} style {style} 2d {two_d}"
+
+
 def test_transform_reads_unaligned_rows():
     """x whose rows start at odd element offsets takes the element-wise loads."""
     from fouroversix_amd.quantize import ops
