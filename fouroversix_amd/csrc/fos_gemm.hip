@@ -28,7 +28,7 @@
 // 256 x 128 tile of 8 wavefronts of 128 x 32 in two rows lost to it wherever 256 x 256 tiles
 // are too few to fill the chip), with bit-identical outputs.  The 128 x 128 tile serves
 // shapes that are not multiples of 256 or too small to fill the chip otherwise, and a 128 x 256
-// tile (the template with BM = 128 and eight wavefronts: half of the threads stage A) those
+// tile (the template with BM = 128 and eight wavefronts: every thread stages a quarter row of A) those
 // that it covers with one workgroup per compute unit.
 // Workgroups are numbered so that the tiles resident on one XCD (blockIdx % 8) form a
 // compact block of the output, which keeps their A/B panels in that XCD's L2.
@@ -205,13 +205,16 @@ FOS_DEVICE void tile_of(int bid, int tiles_m, int tiles_n, int &tm, int &tn) {
 // output row and can be stored as 8 bytes.
 enum { kOutF16 = 0, kOutBF16 = 1, kOutPartial = 2 };
 
-template <int WAVES_M, int WAVES_N, int WM, int WN, int OUT>
+// QUARTER (4 * BM == threads): every thread stages a quarter row of A (16 codes) instead of the first 2 * BM threads
+// half a row each, so that all wavefronts carry the same conversion work.
+template <int WAVES_M, int WAVES_N, int WM, int WN, int OUT, bool QUARTER = false>
 __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const GemmParams p) {
     constexpr bool OUT_BF16 = OUT == kOutBF16;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
     static_assert(2 * BM <= kThreadsG, "one thread per half row of A (wavefronts beyond the first 2 * BM threads stage nothing)");
-    constexpr bool kAllStage = 2 * BM == kThreadsG;
+    static_assert(!QUARTER || 4 * BM == kThreadsG, "quarter rows: four threads per row of A");
+    constexpr bool kAllStage = QUARTER || 2 * BM == kThreadsG;
     extern __shared__ __attribute__((aligned(16))) _Float16 lds[];
     _Float16 *lds_a[2] = {lds, lds + BM * kPitch};
 
@@ -225,13 +228,14 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     // global -> register staging: 32 codes (16 bytes) of one row of each operand, through
     // buffer loads (wave-uniform base + per-thread 32-bit offset + scalar K offset), which
     // keeps 64-bit address arithmetic out of the loop
-    const int ld_row = tid >> 1, ld_half = tid & 1;
+    // (QUARTER: ld_half counts quarter rows, 0..3)
+    const int ld_row = QUARTER ? tid >> 2 : tid >> 1, ld_half = QUARTER ? tid & 3 : tid & 1;
     const bool stager = __builtin_amdgcn_readfirstlane(tid) < 2 * BM;  // wavefront-uniform
     const BufferRsrc ra = make_rsrc(p.A + m0 * kbytes, (uint32_t)(BM * kbytes));
     const BufferRsrc rb = make_rsrc(p.B + n0 * kbytes, (uint32_t)(BN * kbytes));
     const BufferRsrc rsa = make_rsrc(p.sfA + (m0 >> 7) * sf_groups * 512, (uint32_t)((BM >> 7) * sf_groups * 512));
     const BufferRsrc rsb = make_rsrc(p.sfB + (n0 >> 7) * sf_groups * 512, (uint32_t)((BN >> 7) * sf_groups * 512));
-    const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_half * 16);
+    const uint32_t q_off = (uint32_t)(ld_row * kbytes + ld_half * (QUARTER ? 8 : 16));
     const uint32_t s_off = (uint32_t)((ld_row >> 7) * sf_groups * 512 + (ld_row & 31) * 16 + ((ld_row & 127) >> 5) * 4);
     // this lane's B rows: row (lane & 31) of tile j of the wavefront's columns, K half lane >> 5
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -252,7 +256,12 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     typedef Staged<WN> StagedT;
     auto fetch = [&](int64_t ks, StagedT &s) {
         const uint32_t kq = (uint32_t)(ks0 + ks) * 32u, ksf = (uint32_t)(ks0 + ks) * 512u;
-        if (kAllStage || stager) {
+        if constexpr (QUARTER) {
+            const uint2 w = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(ra, (int)q_off, (int)kq, 0));
+            s.qa.x = w.x;
+            s.qa.y = w.y;
+            s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
+        } else if (kAllStage || stager) {
             s.qa = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra, (int)q_off, (int)kq, 0));
             s.sa = __builtin_amdgcn_raw_buffer_load_b32(rsa, (int)s_off, (int)ksf, 0);
         }
@@ -264,6 +273,16 @@ __global__ __launch_bounds__(64 * WAVES_M *WAVES_N) void gemm_nvfp4_kernel(const
     };
     // quarter q (0..3) of the staged A data -> 8 halfs in LDS buffer `buf`
     auto stage_quarter = [&](const StagedT &s, int buf, int q) {
+        if constexpr (QUARTER) {
+            // the thread's 16 codes are one block: its two words go out in the first and the third slice of a step
+            if (q & 1) return;
+            const uint32_t wq = q == 0 ? s.qa.x : s.qa.y;
+            const half2_t s2 = e4m3x2_to_half2(s.sa >> (8 * ld_half));
+            const half2_t sq = __builtin_shufflevector(s2, s2, 0, 0);
+            half8_t *dq = reinterpret_cast<half8_t *>(lds_a[buf] + ld_row * kPitch + ld_half * 16);
+            dq[q >> 1] = dequant8(wq, sq);
+            return;
+        }
         if (!kAllStage && !stager) return;
         const uint32_t wa = q == 0 ? s.qa.x : q == 1 ? s.qa.y : q == 2 ? s.qa.z : s.qa.w;
         // this thread's two block scales: bytes 2*ld_half, 2*ld_half + 1
@@ -985,7 +1004,7 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
     if (p.d_amax) fold_amax<OUT_BF16>(p.d_amax, mine ? um : 0u);
 }
 
-template <int WAVES_M, int WAVES_N, int WM, int WN>
+template <int WAVES_M, int WAVES_N, int WM, int WN, bool QUARTER = false>
 static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
     constexpr int BM = WAVES_M * WM * 32, BN = WAVES_N * WN * 32;
     constexpr int kThreadsG = 64 * WAVES_M * WAVES_N;
@@ -993,9 +1012,9 @@ static int launch_gemm(GemmParams &p, int out_type, hipStream_t s) {
     p.tiles_m = (int)(p.M / BM);
     p.tiles_n = (int)(p.N / BN);
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.splits);
-    auto kbf = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutBF16>;
-    auto kh = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutF16>;
-    auto kp = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutPartial>;
+    auto kbf = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutBF16, QUARTER>;
+    auto kh = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutF16, QUARTER>;
+    auto kp = gemm_nvfp4_kernel<WAVES_M, WAVES_N, WM, WN, kOutPartial, QUARTER>;
     auto kernel = p.splits > 1 ? kp : out_type == FOS_T_BF16 ? kbf : kh;
     if (lds_bytes > 64 * 1024) {
         // more than the default dynamic LDS limit: opt in (idempotent, no device state besides the function attribute)
@@ -1094,7 +1113,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K) {
         return g;
     } else if (tile != 128 && M % 128 == 0 && N % 256 == 0 && M >= 128 &&
                (tile == 129 || ((M / 128) * (N / 256) > 128 && (M / 128) * (N / 256) <= 256))) {
-        // 128 x 256 tiles (eight wavefronts of 128 x 32; the first four stage A) where they give
+        // 128 x 256 tiles (eight wavefronts of 128 x 32; every thread stages a quarter row of A) where they give
         // every compute unit at most one workgroup and more than half of them one: A is converted
         // once per 256 columns instead of once per 128.  Against the 128 x 128 tile, alternating
         // runs: 2048 x 4096 x 4096 71.9 -> 69.3 us, 2048 x 4096 x 14336 242.5 -> 228 us,
@@ -1190,7 +1209,9 @@ static int gemm_nvfp4_impl(const uint8_t *A, const uint8_t *B, const uint8_t *sf
     p.ksteps_per_split = g.ksteps_per_split;
     switch (g.kind) {
         case kPlanBig: return launch_gemm<1, 8, 8, 1>(p, out_type, s);
-        case kPlanWide: return launch_gemm<1, 8, 4, 1>(p, out_type, s);
+        // (quarter rows of A per thread: with half rows the first four wavefronts carried all of A's conversion; alternating
+        // series on one box, 2048 x 4096 x 4096 66.6-72.0 against 67.6-75.7 us, 1792 x 4096 x 4096 62.0-68.3 against 63.6-71.7)
+        case kPlanWide: return launch_gemm<1, 8, 4, 1, true>(p, out_type, s);
         case kPlanSkinny:
             // the 16-row kernel pays off from two K steps per wavefront on (measured at N = 14336:
             // K = 2048 7.6 us against 6.3 us with 32-row tiles, K = 4096 10.6 against 12.3);
